@@ -1,0 +1,76 @@
+"""What an architecture hands to the model builder: a description, in plain
+data, of which parts make up each layer and in which order the layers run.
+
+Nothing in here knows Llama.  An architecture (``models/llama.py`` is the one in
+this package) turns its own typed configuration into a ``ModelSpec``; the
+builder (``models/decoder.py``) looks every part up by its kind in the
+registries and puts the model together.  Because the description is per layer,
+one model may use different mixers and feed-forwards in different layers, and
+because the running order is a list of its own, a layer may run twice or read
+the cache that another call of a layer filled.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """``kind`` names an entry of a registry; ``params`` are the constructor's
+    keyword arguments (sizes and constants, never a model name)."""
+
+    kind: str
+    params: dict = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    block: str                      # arrangement of the parts, e.g. "prenorm"
+    mixer: PartSpec
+    ffn: PartSpec
+    norm1: PartSpec                 # before the mixer
+    norm2: PartSpec                 # before the feed-forward
+    # Names of the parts inside the layer's tensor-name prefix.
+    names: dict = field(default_factory=lambda: {
+        "norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm", "ffn": "mlp"})
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the running order.
+
+    ``layer``   which LayerSpec (and so which weights) runs;
+    ``cache``   which cache buffer its mixer uses; calls that name the same
+                buffer share keys and values;
+    ``writes``  false: the mixer only reads the buffer (another call filled it)
+                and computes no keys and values of its own.
+    """
+
+    layer: int
+    cache: int
+    writes: bool = True
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    vocab_size: int
+    hidden_size: int
+    layers: tuple                    # of LayerSpec
+    schedule: tuple                  # of LayerCall
+    final_norm: PartSpec
+    tie_word_embeddings: bool
+    max_position: int
+    embed_name: str = "model.embed_tokens.weight"
+    final_norm_prefix: str = "model.norm."
+    head_name: str = "lm_head.weight"
+    layer_prefix: str = "model.layers.{i}."
+    eos_token_ids: tuple = ()
+    init_std: float = 0.02           # random-weights mode: normal(0, init_std) matrices
+    norm_init_std: float = 0.0       # random-weights mode: norm weights 1 + normal(0, norm_init_std)
+
+
+def default_schedule(n_layers: int) -> tuple:
+    return tuple(LayerCall(i, i, True) for i in range(n_layers))
+
+
+__all__ = ["PartSpec", "LayerSpec", "LayerCall", "ModelSpec", "default_schedule"]

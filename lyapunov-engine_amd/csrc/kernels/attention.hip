@@ -1,0 +1,466 @@
+// Attention over the paged cache, on the matrix cores, compiled for one head
+// size (LYP_HEAD_DIM, a multiple of 16) and both element types.
+//
+// Two kernels share the fragment loaders and the online softmax:
+//   * attn_prefill: a wave takes 16 query tokens of one request and up to four
+//     query heads of one key/value head, and walks the keys the tokens may see.
+//   * attn_decode:  a wave takes one request's single new token, all query
+//     heads of one key/value head (as the 16 columns of the tile), and one
+//     64-key partition of the context; attn_combine merges the partitions.
+// Both read keys and values from pages through the request's block table, and
+// both run after the step's new keys and values have been written, so a
+// prompt portion needs no second source of keys.
+//
+// What is computed follows the reference: scale 1/sqrt(hd), grouped heads
+// (query head h reads key/value head h / g), causal mask, online softmax with
+// a running maximum and sum, 0 when nothing is visible
+// (csrc/kernels/flash_attn_v2.cu:30-31, 87, 114-166, 197;
+//  csrc/kernels/paged_attention.cu:25-30, 69-105;
+//  csrc/kernels/flash_decoding.cu:12-147).  Unlike the reference the mask uses
+// absolute positions, so a portion that starts in the middle of a prompt sees
+// the keys before it, and the page size is a run-time value.
+//
+// Page layouts (one page of one key/value head):
+//   keys   [bs][hd]   a key's head is contiguous
+//   values [hd][bs]   the keys of a page are contiguous per dimension, which is
+//                     the operand layout of the P.V product
+//
+// Every 16-key block starts at a multiple of 16 in absolute positions and the
+// decode partitions at multiples of 64, so the order of the additions for a
+// token depends on its position and its window alone, never on how the tokens
+// were cut into steps or on what else is in the batch.
+#include "common.h"
+
+#ifndef LYP_HEAD_DIM
+#error "compile with -DLYP_HEAD_DIM=<multiple of 16>"
+#endif
+
+namespace lyp {
+
+constexpr int HD = LYP_HEAD_DIM;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16, at most 256");
+constexpr int kSteps = HD / 16;     // matrix steps over the head dimension; also 16-row blocks of it
+constexpr int kSlice = HD / 4;      // contiguous run of the head dimension one lane group loads
+constexpr int kPartKeys = 64;       // keys per decode partition
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T>
+using Frag = typename Mma16<T>::Frag;
+
+template <typename T>
+__device__ __forceinline__ Frag<T> zero_frag() {
+  Frag<T> f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = from_f32<T>(0.f);
+  return f;
+}
+
+struct PagedKV {
+  const void* kpool;
+  const void* vpool;
+  const int32_t* table;  // this request's row of the block table
+  int nkv, bs, kvh;
+};
+
+// Keys kb0 .. kb0+15 as the row operand of S^T = K . Q^T.  Lane (r, j) holds
+// key kb0 + r, dimensions j * kSlice + 4 * step + {0..3}.
+template <typename T>
+__device__ __forceinline__ void load_k(Frag<T> (&kf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                       int lane) {
+  const int key = kb0 + lane % 16;
+  if (key >= lo && key < hi) {
+    const int page = kv.table[key / kv.bs];
+    if (page >= 0) {
+      const T* row = static_cast<const T*>(kv.kpool) +
+                     ((static_cast<size_t>(page) * kv.nkv + kv.kvh) * kv.bs + key % kv.bs) * HD +
+                     (lane / 16) * kSlice;
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) kf[s] = *reinterpret_cast<const Frag<T>*>(row + 4 * s);
+      return;
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) kf[s] = zero_frag<T>();
+}
+
+// Values of the same 16 keys as the row operand of O^T = V^T . P^T.  Lane
+// (r, j) holds, per 16-row block db of the head dimension, dimension
+// db * 16 + r and keys kb0 + 4 j + {0..3}.  Anything outside [lo, hi) reads as
+// zero: a page that was never written may hold any bit pattern.
+template <typename T>
+__device__ __forceinline__ void load_v(Frag<T> (&vf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                       int lane) {
+  const int key0 = kb0 + 4 * (lane / 16);
+  const int r = lane % 16;
+  const T* vpool = static_cast<const T*>(kv.vpool);
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db) vf[db] = zero_frag<T>();
+  if (kv.bs % 4 == 0) {
+    if (key0 < hi && key0 + 3 >= lo) {
+      const int page = kv.table[key0 / kv.bs];
+      if (page >= 0) {
+        const T* base = vpool + (static_cast<size_t>(page) * kv.nkv + kv.kvh) * HD * kv.bs + key0 % kv.bs;
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db) {
+          Frag<T> f = *reinterpret_cast<const Frag<T>*>(base + static_cast<size_t>(db * 16 + r) * kv.bs);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (key0 + i < lo || key0 + i >= hi) f[i] = from_f32<T>(0.f);
+          vf[db] = f;
+        }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = key0 + i;
+      if (key < lo || key >= hi) continue;
+      const int page = kv.table[key / kv.bs];
+      if (page < 0) continue;
+      const T* base = vpool + (static_cast<size_t>(page) * kv.nkv + kv.kvh) * HD * kv.bs + key % kv.bs;
+#pragma unroll
+      for (int db = 0; db < kSteps; ++db) vf[db][i] = base[static_cast<size_t>(db * 16 + r) * kv.bs];
+    }
+  }
+}
+
+// A query row as the column operand, in the same order of dimensions as load_k.
+template <typename T>
+__device__ __forceinline__ void load_q(Frag<T> (&qf)[kSteps], const T* row, bool valid, int lane) {
+  if (valid) {
+    const T* p = row + (lane / 16) * kSlice;
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) qf[s] = *reinterpret_cast<const Frag<T>*>(p + 4 * s);
+  } else {
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) qf[s] = zero_frag<T>();
+  }
+}
+
+// Running softmax of one 16-column block (lane l owns column l % 16).
+struct Softmax {
+  float m;     // running maximum, in the base-2 domain; the same in the four lane groups
+  float lsum;  // this lane group's part of the running sum
+};
+
+// Take the scores of one 16-key block (s: rows = keys kb0 + 4 (l / 16) + i,
+// column = l % 16), update the running state, rescale the output accumulator
+// and return the probabilities as the column operand of the P.V product.
+// `pos` is the column's absolute position; a key is visible when
+// key <= pos and (window == 0 or key > pos - window).
+template <typename T>
+__device__ __forceinline__ Frag<T> softmax_block(f32x4 s, float scale_log2, int kb0, int pos, int window,
+                                                 int hi, Softmax& st, f32x4 (&o)[kSteps], int lane) {
+  float sv[4];
+  float mx = LYP_NEG_INF;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = kb0 + 4 * (lane / 16) + i;
+    const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
+    sv[i] = vis ? s[i] * scale_log2 : LYP_NEG_INF;
+    mx = fmaxf(mx, sv[i]);
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  const float m_new = fmaxf(st.m, mx);
+  const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
+  const float alpha = exp2f(st.m - m_safe);  // 0 while nothing has been seen yet
+  float psum = 0.f;
+  Frag<T> pf;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float p = exp2f(sv[i] - m_safe);
+    psum += p;
+    pf[i] = from_f32<T>(p);
+  }
+  st.lsum = st.lsum * alpha + psum;
+  st.m = m_new;
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+  return pf;
+}
+
+__device__ __forceinline__ float lane_groups_sum(float v) {
+  v += __shfl_xor(v, 16, kWave);
+  v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+// --------------------------------------------------------------------- prefill
+// grid (tiles, nkv * head_groups); 256 threads.  tile -> (request, first new
+// token of the tile); wave w takes tokens 16 w .. 16 w + 15 of the tile.
+template <typename T, int NCB>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const void* kpool,
+    const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int nh, int nkv, int bs,
+    int window, float scale_log2) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = nh / nkv;
+  const int head_groups = (g + NCB - 1) / NCB;
+  const int kvh = blockIdx.y / head_groups;
+  const int hsub = (blockIdx.y % head_groups) * NCB;  // first head of the group taken here
+
+  const int seq = tile_seq[blockIdx.x];
+  const int tok0 = q_start[seq];
+  const int q_len = q_start[seq + 1] - tok0;
+  const int ctx = ctx_len[seq];
+  const int qi0 = tile_q0[blockIdx.x] + 16 * wave;  // the wave's first new token
+  if (qi0 >= q_len) return;
+  const int n_valid = min(16, q_len - qi0);
+  const int pos0 = ctx - q_len + qi0;  // absolute position of that token
+  const int pos_last = pos0 + n_valid - 1;
+
+  const int col = lane % 16;
+  const bool col_valid = col < n_valid;
+  const int pos = pos0 + col;
+  const size_t token = static_cast<size_t>(tok0) + qi0 + col;
+
+  Frag<T> qf[NCB][kSteps];
+  f32x4 o[NCB][kSteps];
+  Softmax st[NCB];
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int hh = hsub + cb;
+    const bool valid = col_valid && hh < g;
+    const T* row = q + token * q_stride + static_cast<size_t>(kvh * g + (hh < g ? hh : 0)) * HD;
+    load_q<T>(qf[cb], row, valid, lane);
+    st[cb].m = LYP_NEG_INF;
+    st[cb].lsum = 0.f;
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) o[cb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh};
+  const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int hi = pos_last + 1;  // keys at or above it are invisible to every token of the wave
+
+  for (int kb0 = (lo / 16) * 16; kb0 < hi; kb0 += 16) {
+    Frag<T> kf[kSteps], vf[kSteps];
+    load_k<T>(kf, kv, kb0, lo, hi, lane);
+    load_v<T>(vf, kv, kb0, lo, hi, lane);
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+      f32x4 s{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[k], qf[cb][k], s);
+      const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, hi, st[cb],
+                                          o[cb], lane);
+#pragma unroll
+      for (int db = 0; db < kSteps; ++db) o[cb][db] = Mma16<T>::mma(vf[db], pf, o[cb][db]);
+    }
+  }
+
+#pragma unroll
+  for (int cb = 0; cb < NCB; ++cb) {
+    const int hh = hsub + cb;
+    const float l = lane_groups_sum(st[cb].lsum);
+    if (!col_valid || hh >= g) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    T* orow = out + token * out_stride + static_cast<size_t>(kvh * g + hh) * HD + 4 * (lane / 16);
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) {
+      Frag<T> f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = from_f32<T>(o[cb][db][i] * inv);
+      *reinterpret_cast<Frag<T>*>(orow + db * 16) = f;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------- decode
+// grid (ceil(max_parts / 4), nkv * column_groups, requests); 256 threads; each
+// wave is one partition.  Column c of the tile is query head
+// kvh * g + 16 * column_group + c of the request's one new token.
+// Partials: part_o [request][head][part][hd] (not normalised), part_ml
+// [request][head][part][2] = (maximum in the base-2 domain, sum).
+template <typename T>
+__global__ __launch_bounds__(256) void attn_decode_kernel(
+    const T* __restrict__ q, int q_stride, const void* kpool, const void* vpool,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ dec_seqs,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int nh, int nkv, int bs,
+    int window, float scale_log2) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int g = nh / nkv;
+  const int col_groups = (g + 15) / 16;
+  const int kvh = blockIdx.y / col_groups;
+  const int h0 = (blockIdx.y % col_groups) * 16;
+  const int slot = blockIdx.z;
+  const int seq = dec_seqs ? dec_seqs[slot] : slot;
+  const int ctx = ctx_len[seq];
+  const int part = blockIdx.x * 4 + wave;
+  const int pos = ctx - 1;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (part * kPartKeys >= ctx || (part + 1) * kPartKeys <= lo) return;
+
+  const int col = lane % 16;
+  const bool col_valid = h0 + col < g;
+  const int head = kvh * g + h0 + (col_valid ? col : 0);
+  const size_t token = q_start[seq];
+
+  Frag<T> qf[kSteps];
+  load_q<T>(qf, q + token * q_stride + static_cast<size_t>(head) * HD, col_valid, lane);
+  f32x4 o[kSteps];
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  Softmax st{LYP_NEG_INF, 0.f};
+
+  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh};
+  const int k_begin = part * kPartKeys;
+  const int k_end = min(ctx, k_begin + kPartKeys);
+#pragma unroll 1
+  for (int kb0 = k_begin; kb0 < k_end; kb0 += 16) {
+    if (kb0 + 16 <= lo) continue;
+    Frag<T> kf[kSteps], vf[kSteps];
+    load_k<T>(kf, kv, kb0, lo, ctx, lane);
+    load_v<T>(vf, kv, kb0, lo, ctx, lane);
+    f32x4 s{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[k], qf[k], s);
+    const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[db], pf, o[db]);
+  }
+
+  const float l = lane_groups_sum(st.lsum);
+  if (!col_valid) return;
+  const size_t pidx = (static_cast<size_t>(slot) * nh + head) * max_parts + part;
+  float* po = part_o + pidx * HD + 4 * (lane / 16);
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db) *reinterpret_cast<f32x4*>(po + db * 16) = o[db];
+  if (lane / 16 == 0) {
+    part_ml[pidx * 2] = st.m;
+    part_ml[pidx * 2 + 1] = l;
+  }
+}
+
+// grid (nh, requests); 64 threads.
+template <typename T>
+__global__ __launch_bounds__(64) void attn_combine_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, int max_parts,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ dec_seqs, T* __restrict__ out, int out_stride, int nh, int window) {
+  const int head = blockIdx.x, slot = blockIdx.y;
+  const int seq = dec_seqs ? dec_seqs[slot] : slot;
+  const int ctx = ctx_len[seq];
+  const int lo = window > 0 ? max(0, ctx - window) : 0;
+  const int p_lo = lo / kPartKeys;
+  const int p_hi = (ctx + kPartKeys - 1) / kPartKeys;
+  const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
+
+  float m = LYP_NEG_INF;
+  for (int p = p_lo; p < p_hi; ++p) m = fmaxf(m, part_ml[(base + p) * 2]);
+  const float m_safe = m == LYP_NEG_INF ? 0.f : m;
+  float l = 0.f;
+  for (int p = p_lo; p < p_hi; ++p) l += exp2f(part_ml[(base + p) * 2] - m_safe) * part_ml[(base + p) * 2 + 1];
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+
+  T* orow = out + static_cast<size_t>(q_start[seq]) * out_stride + static_cast<size_t>(head) * HD;
+  for (int d = threadIdx.x; d < HD; d += 64) {
+    float acc = 0.f;
+    for (int p = p_lo; p < p_hi; ++p)
+      acc += exp2f(part_ml[(base + p) * 2] - m_safe) * part_o[(base + p) * HD + d];
+    orow[d] = from_f32<T>(acc * inv);
+  }
+}
+
+static int check_common(const char* name, int nh, int nkv, int bs, int max_blocks, int q_stride,
+                        int out_stride, int window) {
+  LYP_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: %d query heads over %d key/value heads", name, nh, nkv);
+  LYP_REQUIRE(bs > 0 && max_blocks > 0, "%s: page size %d, table width %d", name, bs, max_blocks);
+  LYP_REQUIRE(q_stride >= nh * HD && q_stride % 4 == 0, "%s: query row stride %d", name, q_stride);
+  LYP_REQUIRE(out_stride >= nh * HD && out_stride % 4 == 0, "%s: output row stride %d", name, out_stride);
+  LYP_REQUIRE(window >= 0, "%s: window %d", name, window);
+  return 0;
+}
+
+}  // namespace lyp
+
+using namespace lyp;
+
+extern "C" {
+
+int lyp_attn_head_dim() { return HD; }
+int lyp_attn_part_keys() { return kPartKeys; }
+
+int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
+                     const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
+                     const int32_t* q_start, const int32_t* ctx_len, const int32_t* tile_seq,
+                     const int32_t* tile_q0, int n_tiles, int nh, int nkv, int bs, int window, float scale,
+                     hipStream_t stream) {
+  if (check_common("attn_prefill", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
+  LYP_REQUIRE(n_tiles >= 0, "attn_prefill: %d tiles", n_tiles);
+  if (n_tiles == 0) return 0;
+  const int g = nh / nkv;
+  // Column blocks per wave, bounded by what the register file holds.
+  const int regs_per_block = kSteps * ((dtype == kF32 ? 4 : 2) + 4);
+  const int cap = 192 / regs_per_block;
+  const int want = g >= 4 ? 4 : (g >= 2 ? 2 : 1);
+  const int ncb = cap >= 4 ? want : (cap >= 2 ? (want >= 2 ? 2 : 1) : 1);
+  const int head_groups = (g + ncb - 1) / ncb;
+  LYP_REQUIRE(nkv * head_groups <= 65535, "attn_prefill: too many heads for one launch");
+  dim3 grid(n_tiles, nkv * head_groups);
+  const float scale_log2 = scale * kLog2e;
+#define LYP_PREFILL(T, NCB)                                                                              \
+  attn_prefill_kernel<T, NCB><<<grid, 256, 0, stream>>>(                                                  \
+      static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,  \
+      max_blocks, q_start, ctx_len, tile_seq, tile_q0, nh, nkv, bs, window, scale_log2)
+  if (dtype == kF32) {
+    if (ncb == 4) LYP_PREFILL(float, 4);
+    else if (ncb == 2) LYP_PREFILL(float, 2);
+    else LYP_PREFILL(float, 1);
+  } else if (dtype == kBF16) {
+    if (ncb == 4) LYP_PREFILL(bf16_t, 4);
+    else if (ncb == 2) LYP_PREFILL(bf16_t, 2);
+    else LYP_PREFILL(bf16_t, 1);
+  } else {
+    LYP_REQUIRE(false, "attn_prefill: unknown dtype %d", dtype);
+  }
+#undef LYP_PREFILL
+  LYP_LAUNCH_CHECK("attn_prefill");
+  return 0;
+}
+
+// part_o needs n_seqs * nh * max_parts * hd floats, part_ml n_seqs * nh *
+// max_parts * 2, with max_parts >= ceil(longest context / lyp_attn_part_keys()).
+int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
+                    const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
+                    const int32_t* q_start, const int32_t* ctx_len, const int32_t* dec_seqs, int n_seqs,
+                    float* part_o, float* part_ml, int max_parts, int nh, int nkv, int bs, int window,
+                    float scale, hipStream_t stream) {
+  if (check_common("attn_decode", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
+  LYP_REQUIRE(n_seqs >= 0 && max_parts > 0, "attn_decode: %d requests, %d partitions", n_seqs, max_parts);
+  LYP_REQUIRE(part_o && part_ml, "attn_decode: no workspace");
+  if (n_seqs == 0) return 0;
+  const int g = nh / nkv;
+  const int col_groups = (g + 15) / 16;
+  LYP_REQUIRE(n_seqs <= 65535 && nkv * col_groups <= 65535, "attn_decode: launch too large");
+  dim3 grid((max_parts + 3) / 4, nkv * col_groups, n_seqs);
+  dim3 cgrid(nh, n_seqs);
+  const float scale_log2 = scale * kLog2e;
+  if (dtype == kF32) {
+    attn_decode_kernel<float><<<grid, 256, 0, stream>>>(
+        static_cast<const float*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
+        dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
+    attn_combine_kernel<float><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,
+                                                         dec_seqs, static_cast<float*>(out), out_stride, nh,
+                                                         window);
+  } else if (dtype == kBF16) {
+    attn_decode_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        static_cast<const bf16_t*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
+        dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
+    attn_combine_kernel<bf16_t><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,
+                                                          dec_seqs, static_cast<bf16_t*>(out), out_stride,
+                                                          nh, window);
+  } else {
+    LYP_REQUIRE(false, "attn_decode: unknown dtype %d", dtype);
+  }
+  LYP_LAUNCH_CHECK("attn_decode");
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,267 @@
+// Row-wise kernels of a decoder step: embedding gather, RMSNorm fused with the
+// residual add, rotary position encoding fused with the paged K/V write, the
+// SwiGLU gate and a dtype cast.  All arithmetic is 32-bit; only loads and
+// stores see the storage type.
+//
+// What they compute follows the reference:
+//   embedding         python/lyapunov_engine/models/llama.py:205
+//   RMSNorm           csrc/kernels/fused_rmsnorm_swiglu.cu:15-113 (optional
+//                     residual add :42-48, x * inv_rms * gamma :96-101)
+//   rotary + K/V page csrc/kernels/fused_rope_paged.cu:7-86 (pairs (i, i+hd/2),
+//                     V copied unrotated, key slot ((page*nkv+head)*bs+off)*hd;
+//                     values are stored here as [hd][bs] per page and head,
+//                     the layout the attention kernels read)
+//   SwiGLU            csrc/kernels/fused_rmsnorm_swiglu.cu:152-179
+#include "common.h"
+
+namespace lyp {
+
+// ------------------------------------------------------------------ embedding
+template <typename TW>
+__global__ void embedding_kernel(const int32_t* __restrict__ ids, const TW* __restrict__ table,
+                                 float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  const TW* row = table + static_cast<size_t>(ids[t]) * H;
+  float* o = out + static_cast<size_t>(t) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]);
+}
+
+// -------------------------------------------------------------------- RMSNorm
+// h is the 32-bit residual stream.  With `delta`, h + delta is normed, and
+// written back to h unless `rows` selects a subset (the last norm before the
+// output head, where h is not used again).
+template <typename TW, typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                               const TW* __restrict__ w, T* __restrict__ out,
+                               const int32_t* __restrict__ rows, int H, float eps) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+  float* hrow = h + src * H;
+  const T* drow = delta ? delta + src * H : nullptr;
+  const bool write_back = drow != nullptr && rows == nullptr;
+
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = hrow[i];
+    if (drow) {
+      v += to_f32(drow[i]);
+      if (write_back) hrow[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+
+  T* orow = out + static_cast<size_t>(r) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = hrow[i];
+    if (drow && !write_back) v += to_f32(drow[i]);
+    orow[i] = from_f32<T>((v * inv) * to_f32(w[i]));
+  }
+}
+
+// RMSNorm of rows of activations in their own type (no residual stream); for
+// parts that norm something other than the hidden state.
+template <typename TW, typename T>
+__global__ void rmsnorm_act_kernel(const T* __restrict__ x, const TW* __restrict__ w,
+                                   T* __restrict__ out, int H, float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  const T* xrow = x + r * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = to_f32(xrow[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+  T* orow = out + r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    orow[i] = from_f32<T>((to_f32(xrow[i]) * inv) * to_f32(w[i]));
+}
+
+// ------------------------------------------------- rotary encoding + K/V write
+// qkv row of a token: nh query heads, nkv key heads, nkv value heads, hd each.
+// The first `rot` dimensions of every query and key head are rotated in place
+// (pair (i, i + rot/2)) by the angle of the token's absolute position; then the
+// key and value heads are copied into the token's slot of the paged cache.
+template <typename T>
+__global__ void rope_kv_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                               const float* __restrict__ cos_sin,
+                               const int32_t* __restrict__ slots, T* __restrict__ kpool,
+                               T* __restrict__ vpool, int nh, int nkv, int hd, int rot, int bs,
+                               int has_kv) {
+  const int t = blockIdx.x;
+  const int n_rot_heads = has_kv ? nh + nkv : nh;
+  const int width = has_kv ? (nh + 2 * nkv) * hd : nh * hd;
+  T* row = qkv + static_cast<size_t>(t) * width;
+
+  if (rot > 0) {
+    const int half = rot / 2;
+    const float* cs = cos_sin + static_cast<size_t>(positions[t]) * rot;
+    for (int it = threadIdx.x; it < n_rot_heads * half; it += blockDim.x) {
+      const int head = it / half, i = it % half;
+      const float c = cs[i], s = cs[half + i];
+      T* x = row + head * hd;
+      const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
+      x[i] = from_f32<T>(x1 * c - x2 * s);
+      x[i + half] = from_f32<T>(x2 * c + x1 * s);
+    }
+  }
+  if (!has_kv) return;
+  const int slot = slots[t];
+  if (slot < 0) return;  // uniform over the block: no barrier is skipped by part of it
+  __syncthreads();
+  const size_t page = slot / bs, off = slot % bs;
+  const T* k = row + nh * hd;
+  const T* v = row + (nh + nkv) * hd;
+  for (int it = threadIdx.x; it < nkv * hd; it += blockDim.x) {
+    const int kvh = it / hd, d = it % hd;
+    kpool[((page * nkv + kvh) * bs + off) * hd + d] = k[it];
+    vpool[((page * nkv + kvh) * hd + d) * bs + off] = v[it];
+  }
+}
+
+// --------------------------------------------------------------------- SwiGLU
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / I, i = idx % I;
+  const float g = to_f32(gu[t * 2 * I + i]);
+  const float u = to_f32(gu[t * 2 * I + I + i]);
+  out[idx] = from_f32<T>((g / (1.0f + expf(-g))) * u);
+}
+
+// ----------------------------------------------------------------------- cast
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx < n) out[idx] = from_f32<TO>(to_f32(in[idx]));
+}
+
+static int norm_threads(int H) { return H <= 512 ? 128 : (H >= 4096 ? 512 : 256); }
+
+}  // namespace lyp
+
+using namespace lyp;
+
+extern "C" {
+
+int lyp_embedding(const int32_t* ids, const void* table, int table_dtype, float* out, int T, int H,
+                  hipStream_t stream) {
+  LYP_REQUIRE(T >= 0 && H > 0, "embedding: bad sizes T=%d H=%d", T, H);
+  if (T == 0) return 0;
+  const int threads = H >= 1024 ? 256 : 128;
+  if (table_dtype == kF32)
+    embedding_kernel<float><<<T, threads, 0, stream>>>(ids, static_cast<const float*>(table), out, H);
+  else if (table_dtype == kBF16)
+    embedding_kernel<bf16_t><<<T, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table), out, H);
+  else
+    LYP_REQUIRE(false, "embedding: unknown table dtype %d", table_dtype);
+  LYP_LAUNCH_CHECK("embedding");
+  return 0;
+}
+
+// h [*, H] float; delta, out of act_dtype; w of w_dtype; rows optional [n_rows].
+int lyp_rmsnorm(float* h, const void* delta, const void* w, int w_dtype, void* out, int act_dtype,
+                const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
+  LYP_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  if (n_rows == 0) return 0;
+  const int threads = norm_threads(H);
+#define LYP_NORM(TW, T)                                                                         \
+  rmsnorm_kernel<TW, T><<<n_rows, threads, 0, stream>>>(h, static_cast<const T*>(delta),        \
+                                                        static_cast<const TW*>(w),              \
+                                                        static_cast<T*>(out), rows, H, eps)
+  if (w_dtype == kF32 && act_dtype == kF32) LYP_NORM(float, float);
+  else if (w_dtype == kF32 && act_dtype == kBF16) LYP_NORM(float, bf16_t);
+  else if (w_dtype == kBF16 && act_dtype == kF32) LYP_NORM(bf16_t, float);
+  else if (w_dtype == kBF16 && act_dtype == kBF16) LYP_NORM(bf16_t, bf16_t);
+  else LYP_REQUIRE(false, "rmsnorm: unknown dtypes w=%d act=%d", w_dtype, act_dtype);
+#undef LYP_NORM
+  LYP_LAUNCH_CHECK("rmsnorm");
+  return 0;
+}
+
+int lyp_rmsnorm_act(const void* x, const void* w, int w_dtype, void* out, int act_dtype, int n_rows,
+                    int H, float eps, hipStream_t stream) {
+  LYP_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm_act: bad sizes rows=%d H=%d", n_rows, H);
+  if (n_rows == 0) return 0;
+  const int threads = norm_threads(H);
+#define LYP_NORM(TW, T)                                                                      \
+  rmsnorm_act_kernel<TW, T><<<n_rows, threads, 0, stream>>>(                                 \
+      static_cast<const T*>(x), static_cast<const TW*>(w), static_cast<T*>(out), H, eps)
+  if (w_dtype == kF32 && act_dtype == kF32) LYP_NORM(float, float);
+  else if (w_dtype == kF32 && act_dtype == kBF16) LYP_NORM(float, bf16_t);
+  else if (w_dtype == kBF16 && act_dtype == kF32) LYP_NORM(bf16_t, float);
+  else if (w_dtype == kBF16 && act_dtype == kBF16) LYP_NORM(bf16_t, bf16_t);
+  else LYP_REQUIRE(false, "rmsnorm_act: unknown dtypes w=%d act=%d", w_dtype, act_dtype);
+#undef LYP_NORM
+  LYP_LAUNCH_CHECK("rmsnorm_act");
+  return 0;
+}
+
+// qkv [T, (nh + 2 nkv) hd] (or [T, nh hd] when has_kv == 0), rotated in place.
+// cos_sin [max_pos, rot]: rot/2 cosines then rot/2 sines per position; rot == 0
+// means no rotation.  slots [T]: page * bs + offset, or -1 for "do not store".
+int lyp_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const float* cos_sin,
+                      const int32_t* slots, void* kpool, void* vpool, int T, int nh, int nkv, int hd,
+                      int rot, int bs, int has_kv, hipStream_t stream) {
+  LYP_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
+  LYP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary width %d of head %d", rot, hd);
+  LYP_REQUIRE(rot == 0 || cos_sin != nullptr, "rope_kv_write: rotation without a table");
+  LYP_REQUIRE(!has_kv || (slots && kpool && vpool), "rope_kv_write: cache write without a cache");
+  if (T == 0) return 0;
+  const int threads = 256;
+  if (dtype == kF32)
+    rope_kv_kernel<float><<<T, threads, 0, stream>>>(static_cast<float*>(qkv), positions, cos_sin, slots,
+                                                     static_cast<float*>(kpool), static_cast<float*>(vpool),
+                                                     nh, nkv, hd, rot, bs, has_kv);
+  else if (dtype == kBF16)
+    rope_kv_kernel<bf16_t><<<T, threads, 0, stream>>>(static_cast<bf16_t*>(qkv), positions, cos_sin, slots,
+                                                      static_cast<bf16_t*>(kpool),
+                                                      static_cast<bf16_t*>(vpool), nh, nkv, hd, rot, bs,
+                                                      has_kv);
+  else
+    LYP_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+int lyp_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t stream) {
+  LYP_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  const size_t total = static_cast<size_t>(T) * I;
+  if (total == 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = static_cast<unsigned>((total + threads - 1) / threads);
+  if (dtype == kF32)
+    swiglu_kernel<float><<<blocks, threads, 0, stream>>>(static_cast<const float*>(gate_up),
+                                                         static_cast<float*>(out), I, total);
+  else if (dtype == kBF16)
+    swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>(static_cast<const bf16_t*>(gate_up),
+                                                          static_cast<bf16_t*>(out), I, total);
+  else
+    LYP_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+int lyp_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n, hipStream_t stream) {
+  LYP_REQUIRE(n >= 0, "cast: negative count");
+  if (n == 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = static_cast<unsigned>((n + threads - 1) / threads);
+  if (in_dtype == kBF16 && out_dtype == kF32)
+    cast_kernel<bf16_t, float><<<blocks, threads, 0, stream>>>(static_cast<const bf16_t*>(in),
+                                                               static_cast<float*>(out), n);
+  else if (in_dtype == kF32 && out_dtype == kBF16)
+    cast_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(static_cast<const float*>(in),
+                                                               static_cast<bf16_t*>(out), n);
+  else
+    LYP_REQUIRE(false, "cast: unsupported pair %d -> %d", in_dtype, out_dtype);
+  LYP_LAUNCH_CHECK("cast");
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,180 @@
+// C[M,N] = A[M,K] . W[N,K]^T on the matrix cores, for bfloat16 and for true
+// 32-bit floats (the 32x32x2 float instruction, no reduced-precision mode).
+// Both operands are row-major with the inner dimension contiguous, which is
+// how a projection's weight [out_features, in_features] is stored.
+//
+// The reference has no kernel of its own here: its projections are nn.Linear
+// calls (python/lyapunov_engine/models/llama.py:45-48, 112-117, 177).
+//
+// The inner dimension is walked in the same order for every row whatever M is,
+// and there is no split over it, so a token's result does not depend on what
+// else is in the batch.  Any M, N, K is accepted; rows that are not 16-byte
+// aligned take a scalar load path.
+#include "common.h"
+
+namespace lyp {
+
+enum GemmMode : int {
+  kStoreAct = 0,    // C has the operands' type
+  kStoreF32 = 1,    // C is float
+  kAccumF32 = 2,    // C is float and is added to (the residual stream)
+};
+
+template <typename T>
+struct VecOf;
+template <>
+struct VecOf<float> {
+  static constexpr int kVec = 4;
+};
+template <>
+struct VecOf<bf16_t> {
+  static constexpr int kVec = 8;
+};
+
+constexpr int kBK = 32;
+
+template <typename T, int BM, int BN, int WGM, int WGN, int MODE>
+__global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
+                                                      const T* __restrict__ W, void* __restrict__ Cv,
+                                                      int M, int N, int K, int lda, int ldw, int ldc,
+                                                      int vec_ok) {
+  static_assert(WGM * WGN == 4, "four waves per workgroup");
+  constexpr int VEC = VecOf<T>::kVec;
+  constexpr int KF = Mma32<T>::kElems;
+  constexpr int PAD = VEC;
+  constexpr int LDS_LD = kBK + PAD;
+  constexpr int IM = BM / (WGM * 32);
+  constexpr int JN = BN / (WGN * 32);
+  static_assert(IM >= 1 && JN >= 1, "tile too small for the wave grid");
+  using Frag = typename Mma32<T>::Frag;
+
+  __shared__ __attribute__((aligned(16))) T As[BM * LDS_LD];
+  __shared__ __attribute__((aligned(16))) T Ws[BN * LDS_LD];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+  f32x16 acc[IM][JN];
+#pragma unroll
+  for (int i = 0; i < IM; ++i)
+#pragma unroll
+    for (int j = 0; j < JN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  constexpr int VPR = kBK / VEC;  // vectors per tile row
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+
+  auto load_tile = [&](const T* __restrict__ src, int ld, int row0, int nrows_total, int k0, T* dst,
+                       int tile_rows) {
+    for (int v = tid; v < tile_rows * VPR; v += 256) {
+      const int r = v / VPR, cv = v % VPR;
+      const int gr = row0 + r, gk = k0 + cv * VEC;
+      VecT val;
+      if (gr < nrows_total && vec_ok && gk + VEC <= K) {
+        val = *reinterpret_cast<const VecT*>(src + static_cast<size_t>(gr) * ld + gk);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const bool in = gr < nrows_total && gk + e < K;
+          val[e] = in ? src[static_cast<size_t>(gr) * ld + gk + e] : from_f32<T>(0.f);
+        }
+      }
+      *reinterpret_cast<VecT*>(dst + r * LDS_LD + cv * VEC) = val;
+    }
+  };
+
+  for (int k0 = 0; k0 < K; k0 += kBK) {
+    __syncthreads();
+    load_tile(A, lda, m0, M, k0, As, BM);
+    load_tile(W, ldw, n0, N, k0, Ws, BN);
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kBK; kk += 2 * KF) {
+      Frag a[IM], b[JN];
+      const int kofs = kk + (lane / 32) * KF;
+#pragma unroll
+      for (int i = 0; i < IM; ++i)
+        a[i] = *reinterpret_cast<const Frag*>(As + ((wm * IM + i) * 32 + lane % 32) * LDS_LD + kofs);
+#pragma unroll
+      for (int j = 0; j < JN; ++j)
+        b[j] = *reinterpret_cast<const Frag*>(Ws + ((wn * JN + j) * 32 + lane % 32) * LDS_LD + kofs);
+#pragma unroll
+      for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j) acc[i][j] = Mma32<T>::mma(a[i], b[j], acc[i][j]);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < IM; ++i)
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+      const int n = n0 + (wn * JN + j) * 32 + lane % 32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + (wm * IM + i) * 32 + 8 * (v / 4) + 4 * (lane / 32) + v % 4;
+        if (m >= M) continue;
+        const size_t idx = static_cast<size_t>(m) * ldc + n;
+        if constexpr (MODE == kStoreAct) {
+          static_cast<T*>(Cv)[idx] = from_f32<T>(acc[i][j][v]);
+        } else if constexpr (MODE == kStoreF32) {
+          static_cast<float*>(Cv)[idx] = acc[i][j][v];
+        } else {
+          static_cast<float*>(Cv)[idx] += acc[i][j][v];
+        }
+      }
+    }
+}
+
+template <typename T, int MODE>
+static void launch_gemm(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                        int vec_ok, hipStream_t stream) {
+  if (M <= 32) {
+    dim3 grid((N + 127) / 128, (M + 31) / 32);
+    gemm_nt_kernel<T, 32, 128, 1, 4, MODE><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, vec_ok);
+  } else if (M <= 64) {
+    dim3 grid((N + 127) / 128, (M + 63) / 64);
+    gemm_nt_kernel<T, 64, 128, 2, 2, MODE><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, vec_ok);
+  } else {
+    dim3 grid((N + 127) / 128, (M + 127) / 128);
+    gemm_nt_kernel<T, 128, 128, 2, 2, MODE><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, vec_ok);
+  }
+}
+
+}  // namespace lyp
+
+using namespace lyp;
+
+extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int mode, int M, int N, int K,
+                           int lda, int ldw, int ldc, hipStream_t stream) {
+  LYP_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+  LYP_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm: leading dimensions %d %d %d too small", lda, ldw, ldc);
+  LYP_REQUIRE(mode >= 0 && mode <= 2, "gemm: unknown output mode %d", mode);
+  LYP_REQUIRE((M + 127) / 128 <= 65535, "gemm: M=%d too large for one launch", M);
+  if (M == 0) return 0;
+  const int vec = dtype == kF32 ? 4 : 8;
+  const size_t esz = dtype == kF32 ? 4 : 2;
+  const int vec_ok = (lda % vec == 0) && (ldw % vec == 0) &&
+                     (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(W) % 16 == 0);
+  (void)esz;
+#define LYP_GEMM(T, MODE)                                                                             \
+  launch_gemm<T, MODE>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, \
+                       vec_ok, stream)
+  if (dtype == kF32) {
+    if (mode == kStoreAct || mode == kStoreF32) LYP_GEMM(float, kStoreF32);
+    else LYP_GEMM(float, kAccumF32);
+  } else if (dtype == kBF16) {
+    if (mode == kStoreAct) LYP_GEMM(bf16_t, kStoreAct);
+    else if (mode == kStoreF32) LYP_GEMM(bf16_t, kStoreF32);
+    else LYP_GEMM(bf16_t, kAccumF32);
+  } else {
+    LYP_REQUIRE(false, "gemm: unknown dtype %d", dtype);
+  }
+#undef LYP_GEMM
+  LYP_LAUNCH_CHECK("gemm_nt");
+  return 0;
+}

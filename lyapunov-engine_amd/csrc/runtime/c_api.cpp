@@ -1,0 +1,244 @@
+// C interface of the host runtime (cache manager and scheduler), for ctypes.
+// The reference binds the same two classes with pybind11
+// (csrc/bindings.cpp:552-621).  Every function returns 0 (or a value >= 0) on
+// success and a negative number on failure, with the message kept for
+// lyp_rt_last_error().
+#include <cstring>
+#include <exception>
+#include <string>
+
+#include "cache_manager.hpp"
+#include "scheduler.hpp"
+
+namespace {
+thread_local std::string g_error;
+
+template <typename F>
+int guarded(F&& f) {
+  try {
+    return f();
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return -1;
+  } catch (...) {
+    g_error = "unknown error";
+    return -1;
+  }
+}
+
+int copy_out(const std::vector<int32_t>& v, int32_t* out, int cap) {
+  const int n = static_cast<int>(v.size());
+  if (out) std::memcpy(out, v.data(), sizeof(int32_t) * static_cast<size_t>(std::min(n, cap)));
+  return n;
+}
+}  // namespace
+
+using lyp::CacheManager;
+using lyp::Scheduler;
+
+extern "C" {
+
+const char* lyp_rt_last_error() { return g_error.c_str(); }
+
+// ------------------------------------------------------------- cache manager
+void* lyp_cache_create(int num_groups, const int* num_pages, const int* page_size, const int* window,
+                       int num_state_slots) {
+  try {
+    std::vector<lyp::GroupSpec> groups(num_groups);
+    for (int g = 0; g < num_groups; ++g) groups[g] = {num_pages[g], page_size[g], window[g]};
+    return new CacheManager(std::move(groups), num_state_slots);
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+void lyp_cache_destroy(void* h) { delete static_cast<CacheManager*>(h); }
+
+int lyp_cache_add(void* h, int64_t id) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->add(id); });
+}
+int lyp_cache_has(void* h, int64_t id) { return static_cast<CacheManager*>(h)->has(id) ? 1 : 0; }
+int lyp_cache_length(void* h, int64_t id) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->length(id); });
+}
+int lyp_cache_capacity(void* h, int64_t id) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->capacity(id); });
+}
+int lyp_cache_can_extend(void* h, int64_t id, int new_len) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->can_extend(id, new_len) ? 1 : 0; });
+}
+int lyp_cache_max_length(void* h, int64_t id) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->max_length(id); });
+}
+int lyp_cache_extend(void* h, int64_t id, int new_len) {
+  return guarded([&] {
+    static_cast<CacheManager*>(h)->extend(id, new_len);
+    return 0;
+  });
+}
+int lyp_cache_commit(void* h, int64_t id, int new_len) {
+  return guarded([&] {
+    static_cast<CacheManager*>(h)->commit(id, new_len);
+    return 0;
+  });
+}
+int lyp_cache_free(void* h, int64_t id) {
+  return guarded([&] {
+    static_cast<CacheManager*>(h)->free(id);
+    return 0;
+  });
+}
+int lyp_cache_reset(void* h) {
+  return guarded([&] {
+    static_cast<CacheManager*>(h)->reset();
+    return 0;
+  });
+}
+int lyp_cache_num_free_pages(void* h, int g) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->num_free_pages(g); });
+}
+int lyp_cache_num_free_slots(void* h) { return static_cast<CacheManager*>(h)->num_free_slots(); }
+int lyp_cache_num_requests(void* h) { return static_cast<CacheManager*>(h)->num_requests(); }
+int lyp_cache_state_slot(void* h, int64_t id) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->state_slot(id); });
+}
+// Copies up to `cap` entries; returns the table's length.
+int lyp_cache_table(void* h, int64_t id, int g, int32_t* out, int cap) {
+  return guarded([&] { return copy_out(static_cast<CacheManager*>(h)->table(id, g), out, cap); });
+}
+int lyp_cache_ref_count(void* h, int g, int page) {
+  return guarded([&] { return static_cast<CacheManager*>(h)->ref_count(g, page); });
+}
+// 0 if every invariant holds; else -1 and the description as the last error.
+int lyp_cache_check(void* h) {
+  const std::string what = static_cast<CacheManager*>(h)->check();
+  if (what.empty()) return 0;
+  g_error = what;
+  return -1;
+}
+// out[0..3] = pages taken, pages returned, window returns, high-water mark.
+void lyp_cache_counters(void* h, int64_t* out) {
+  const auto& c = static_cast<CacheManager*>(h)->counters();
+  out[0] = c.pages_taken;
+  out[1] = c.pages_returned;
+  out[2] = c.window_returns;
+  out[3] = c.high_water;
+}
+
+// ------------------------------------------------------------------ scheduler
+void* lyp_sched_create(void* cache, int max_num_seqs, int max_num_batched_tokens, int max_model_len, int max_chunk,
+                       const int32_t* eos_ids, int n_eos) {
+  try {
+    lyp::SchedulerConfig cfg;
+    cfg.max_num_seqs = max_num_seqs;
+    cfg.max_num_batched_tokens = max_num_batched_tokens;
+    cfg.max_model_len = max_model_len;
+    cfg.max_chunk = max_chunk;
+    cfg.eos_token_ids.assign(eos_ids, eos_ids + n_eos);
+    return new Scheduler(std::move(cfg), static_cast<CacheManager*>(cache));
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return nullptr;
+  }
+}
+void lyp_sched_destroy(void* h) { delete static_cast<Scheduler*>(h); }
+
+int lyp_sched_add(void* h, int64_t id, const int32_t* prompt, int n, float temperature, float top_p, int top_k,
+                  int max_tokens, int ignore_eos, uint64_t seed) {
+  return guarded([&] {
+    lyp::SamplingParams sp;
+    sp.temperature = temperature;
+    sp.top_p = top_p;
+    sp.top_k = top_k;
+    sp.max_tokens = max_tokens;
+    sp.ignore_eos = ignore_eos != 0;
+    sp.seed = seed;
+    static_cast<Scheduler*>(h)->add(id, std::vector<int32_t>(prompt, prompt + n), sp);
+    return 0;
+  });
+}
+int lyp_sched_abort(void* h, int64_t id) {
+  return guarded([&] { return static_cast<Scheduler*>(h)->abort(id) ? 1 : 0; });
+}
+int lyp_sched_has_unfinished(void* h) { return static_cast<Scheduler*>(h)->has_unfinished() ? 1 : 0; }
+int lyp_sched_num_waiting(void* h) { return static_cast<Scheduler*>(h)->num_waiting(); }
+int lyp_sched_num_running(void* h) { return static_cast<Scheduler*>(h)->num_running(); }
+
+// Plans a step.  Fills ids/start/count/wants (each with room for `cap`
+// entries) and returns the number of entries, or -1.
+int lyp_sched_schedule(void* h, int64_t* ids, int32_t* start, int32_t* count, int32_t* wants, int cap) {
+  return guarded([&] {
+    const auto plan = static_cast<Scheduler*>(h)->schedule();
+    const int n = static_cast<int>(plan.size());
+    if (n > cap) throw std::runtime_error("schedule: the plan has more entries than the caller's buffers");
+    for (int i = 0; i < n; ++i) {
+      ids[i] = plan[i].id;
+      start[i] = plan[i].start;
+      count[i] = plan[i].count;
+      wants[i] = plan[i].wants_logits ? 1 : 0;
+    }
+    return n;
+  });
+}
+int lyp_sched_post_step(void* h, const int32_t* sampled, int n) {
+  return guarded([&] {
+    static_cast<Scheduler*>(h)->post_step(std::vector<int32_t>(sampled, sampled + n));
+    return 0;
+  });
+}
+int lyp_sched_last_preempted(void* h, int64_t* out, int cap) {
+  const auto& v = static_cast<Scheduler*>(h)->last_preempted();
+  const int n = static_cast<int>(v.size());
+  for (int i = 0; i < std::min(n, cap); ++i) out[i] = v[i];
+  return n;
+}
+// out = {prompt_len, total_len, num_computed, status, preemptions}
+int lyp_sched_info(void* h, int64_t id, int32_t* out) {
+  return guarded([&] {
+    const auto& s = static_cast<Scheduler*>(h)->get(id);
+    out[0] = s.prompt_len;
+    out[1] = s.total_len();
+    out[2] = s.num_computed;
+    out[3] = static_cast<int>(s.status);
+    out[4] = s.preemptions;
+    return 0;
+  });
+}
+// Copies tokens [from, from + cap) of the request; returns how many were copied.
+int lyp_sched_tokens(void* h, int64_t id, int from, int32_t* out, int cap) {
+  return guarded([&] {
+    const auto& s = static_cast<Scheduler*>(h)->get(id);
+    const int n = std::max(0, std::min(cap, s.total_len() - from));
+    if (n > 0) std::memcpy(out, s.tokens.data() + from, sizeof(int32_t) * static_cast<size_t>(n));
+    return n;
+  });
+}
+// out = {temperature, top_p} / {top_k, max_tokens, ignore_eos}; seed separately.
+int lyp_sched_params(void* h, int64_t id, float* fout, int32_t* iout, uint64_t* seed) {
+  return guarded([&] {
+    const auto& p = static_cast<Scheduler*>(h)->get(id).params;
+    fout[0] = p.temperature;
+    fout[1] = p.top_p;
+    iout[0] = p.top_k;
+    iout[1] = p.max_tokens;
+    iout[2] = p.ignore_eos ? 1 : 0;
+    *seed = p.seed;
+    return 0;
+  });
+}
+int lyp_sched_forget(void* h, int64_t id) {
+  return guarded([&] {
+    static_cast<Scheduler*>(h)->forget(id);
+    return 0;
+  });
+}
+// out[0..3] = steps, scheduled tokens, preemptions, finished.
+void lyp_sched_counters(void* h, int64_t* out) {
+  const auto& c = static_cast<Scheduler*>(h)->counters();
+  out[0] = c.steps;
+  out[1] = c.scheduled_tokens;
+  out[2] = c.preemptions;
+  out[3] = c.finished;
+}
+
+}  // extern "C"

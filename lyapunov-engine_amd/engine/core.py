@@ -1,0 +1,39 @@
+"""Model, cache manager, device pools and step function as one object; what the
+generating engine and the trace replay both stand on."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..cache.manager import CacheManager, CachePools, GroupConfig
+from ..config.engine_config import parse_dtype
+from ..models.decoder import DecoderModel
+from ..weights.loader import TensorSource, load_model
+from .runner import ModelRunner, StepEntry
+
+
+class EngineCore:
+    def __init__(self, model: DecoderModel, model_config, *, dtype, device="cuda:0", num_blocks: int,
+                 block_size: int = 16, num_state_slots: int = 64):
+        self.model, self.model_config = model, model_config
+        self.dtype, self.device = parse_dtype(dtype), torch.device(device)
+        self.block_size = block_size
+        layout = model.cache_layout()
+        groups = [GroupConfig(num_blocks, block_size, gl.spec.window) for gl in layout.groups]
+        # A model without keys and values (state only) still gets a group, so
+        # that requests have a length and the manager one code path.
+        self.cache = CacheManager(groups or [GroupConfig(num_blocks, block_size, 0)], num_state_slots)
+        self.pools = CachePools(layout, groups, num_state_slots, self.dtype, self.device)
+        self.runner = ModelRunner(model, self.cache, self.pools, self.dtype, self.device)
+
+    @classmethod
+    def from_folder(cls, model_dir: str, *, dtype, device="cuda:0", source: Optional[TensorSource] = None, **kw):
+        model, cfg = load_model(model_dir, parse_dtype(dtype), device, source=source)
+        return cls(model, cfg, dtype=dtype, device=device, **kw)
+
+    def step(self, entries: list):
+        return self.runner.step(entries)
+
+
+__all__ = ["EngineCore", "StepEntry"]

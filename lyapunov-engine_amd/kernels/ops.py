@@ -1,0 +1,324 @@
+"""Python face of the HIP kernels: checks shapes on the host, then launches on
+torch's current stream.  Tensors are torch tensors used as device memory; no
+torch operator computes anything here.
+
+The reference's façade (python/lyapunov_engine/ops.py:12-216) falls back to
+eager PyTorch when its extension is missing.  There is no fallback here: a
+library that cannot be loaded, or an input on the wrong device, is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+STORE_ACT, STORE_F32, ACCUM_F32 = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _load(path) -> ctypes.CDLL:
+    try:
+        return ctypes.CDLL(str(path))
+    except OSError as e:
+        raise KernelError(f"cannot load the kernel library {path}: {e}") from None
+
+
+_core = None
+_attn: dict[int, ctypes.CDLL] = {}
+
+
+def core() -> ctypes.CDLL:
+    global _core
+    if _core is None:
+        lib = _load(build.core_library())
+        lib.lyp_last_error.restype = ctypes.c_char_p
+        lib.lyp_embedding.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
+        lib.lyp_rmsnorm.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
+                                    c_float, c_void_p]
+        lib.lyp_rmsnorm_act.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
+        lib.lyp_rope_kv_write.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
+        lib.lyp_cast.argtypes = [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p]
+        lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_void_p]
+        lib.lyp_sample.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p]
+        _core = lib
+    return _core
+
+
+def attention_lib(head_dim: int) -> ctypes.CDLL:
+    lib = _attn.get(head_dim)
+    if lib is None:
+        lib = _load(build.attention_library(head_dim))
+        lib.lyp_last_error.restype = ctypes.c_char_p
+        if lib.lyp_attn_head_dim() != head_dim:
+            raise KernelError(f"attention library for head size {head_dim} reports {lib.lyp_attn_head_dim()}")
+        lib.lyp_attn_prefill.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                         c_float, c_void_p]
+        lib.lyp_attn_decode.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                        c_int, c_int, c_float, c_void_p]
+        _attn[head_dim] = lib
+    return lib
+
+
+def require_gpu() -> None:
+    """The kernels are built for one architecture; say so before the first
+    launch rather than after a failed one."""
+    if not torch.cuda.is_available():
+        raise KernelError("no GPU: this package has no CPU path")
+    name = torch.cuda.get_device_properties(0).gcnArchName.split(":")[0]
+    if name != build.GPU_ARCH:
+        raise KernelError(f"the kernels are built for {build.GPU_ARCH}, this device is {name}")
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _check(rc: int, lib: ctypes.CDLL) -> None:
+    if rc != 0:
+        raise KernelError(lib.lyp_last_error().decode())
+
+
+def _dev(*ts) -> None:
+    for t in ts:
+        if t is not None and (not t.is_cuda or not t.is_contiguous()):
+            raise KernelError(f"kernel operand must be a contiguous GPU tensor, got {tuple(t.shape)} on {t.device} "
+                              f"contiguous={t.is_contiguous()}")
+
+
+def _code(dt: torch.dtype) -> int:
+    try:
+        return _CODE[dt]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dt}") from None
+
+
+# ------------------------------------------------------------------ row kernels
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] as float (the residual stream)."""
+    _dev(ids, table, out)
+    T, H = out.shape
+    if ids.dtype != torch.int32 or ids.numel() != T or table.shape[1] != H or out.dtype != torch.float32:
+        raise KernelError(f"embedding: ids {tuple(ids.shape)} {ids.dtype}, table {tuple(table.shape)}, out {tuple(out.shape)} {out.dtype}")
+    lib = core()
+    _check(lib.lyp_embedding(_p(ids), _p(table), _code(table.dtype), _p(out), T, H, _stream()), lib)
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, delta: torch.Tensor | None = None,
+            rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out = rmsnorm(h [+ delta]) * weight.  h is the float residual stream and
+    takes the sum, unless ``rows`` picks the rows to norm."""
+    _dev(h, weight, out, delta, rows)
+    H = h.shape[1]
+    n = out.shape[0]
+    if h.dtype != torch.float32 or weight.numel() != H or out.shape[1] != H:
+        raise KernelError(f"rmsnorm: h {tuple(h.shape)} {h.dtype}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    if delta is not None and (delta.shape != h.shape or delta.dtype != out.dtype):
+        raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} {delta.dtype} against h {tuple(h.shape)}, out {out.dtype}")
+    if rows is not None:
+        if rows.dtype != torch.int32 or rows.numel() != n:
+            raise KernelError("rmsnorm: rows must be int32, one per output row")
+    elif n != h.shape[0]:
+        raise KernelError("rmsnorm: output rows differ from input rows")
+    lib = core()
+    _check(lib.lyp_rmsnorm(_p(h), _p(delta), _p(weight), _code(weight.dtype), _p(out), _code(out.dtype), _p(rows), n,
+                           H, float(eps), _stream()), lib)
+    return out
+
+
+def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+    _dev(x, weight, out)
+    n, H = x.shape
+    if out.shape != x.shape or out.dtype != x.dtype or weight.numel() != H:
+        raise KernelError("rmsnorm_act: shapes or dtypes differ")
+    lib = core()
+    _check(lib.lyp_rmsnorm_act(_p(x), _p(weight), _code(weight.dtype), _p(out), _code(x.dtype), n, H, float(eps),
+                               _stream()), lib)
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor | None,
+                  slots: torch.Tensor | None, kpool: torch.Tensor | None, vpool: torch.Tensor | None, *, num_heads: int,
+                  num_kv_heads: int, head_dim: int, page_size: int, has_kv: bool = True) -> None:
+    """Rotate the query (and key) heads of ``qkv`` in place by each token's
+    position and store keys and values in the token's cache slot."""
+    _dev(qkv, positions, cos_sin, slots, kpool, vpool)
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim if has_kv else num_heads * head_dim
+    if qkv.shape[1] != width or positions.numel() != T or positions.dtype != torch.int32:
+        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} against width {width}, positions {tuple(positions.shape)}")
+    rot = 0
+    if cos_sin is not None:
+        rot = cos_sin.shape[1]
+        if cos_sin.dtype != torch.float32 or rot > head_dim or rot % 2:
+            raise KernelError(f"rope_kv_write: table {tuple(cos_sin.shape)} {cos_sin.dtype} for heads of {head_dim}")
+    if has_kv:
+        n_pages = kpool.shape[0]
+        if (slots is None or slots.numel() != T or slots.dtype != torch.int32
+                or tuple(kpool.shape) != (n_pages, num_kv_heads, page_size, head_dim)
+                or tuple(vpool.shape) != (n_pages, num_kv_heads, head_dim, page_size)
+                or kpool.dtype != qkv.dtype or vpool.dtype != qkv.dtype):
+            raise KernelError(f"rope_kv_write: pools {tuple(kpool.shape)} / {tuple(vpool.shape)} {kpool.dtype} do not "
+                              f"fit {num_kv_heads} heads of {head_dim}, pages of {page_size}, dtype {qkv.dtype}")
+    lib = core()
+    _check(lib.lyp_rope_kv_write(_p(qkv), _code(qkv.dtype), _p(positions), _p(cos_sin), _p(slots), _p(kpool),
+                                 _p(vpool), T, num_heads, num_kv_heads, head_dim, rot, page_size, int(has_kv),
+                                 _stream()), lib)
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+    _dev(gate_up, out)
+    T, I = out.shape
+    if tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError(f"swiglu: {tuple(gate_up.shape)} -> {tuple(out.shape)}")
+    lib = core()
+    _check(lib.lyp_swiglu(_p(gate_up), _p(out), _code(out.dtype), T, I, _stream()), lib)
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    if x.dtype == dtype:
+        return x
+    _dev(x)
+    out = torch.empty_like(x, dtype=dtype)
+    lib = core()
+    _check(lib.lyp_cast(_p(x), _code(x.dtype), _p(out), _code(dtype), x.numel(), _stream()), lib)
+    return out
+
+
+# ------------------------------------------------------------------------ GEMM
+def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    """out = a @ w.T (or out += ...).  a [M, K], w [N, K] of one dtype; out
+    [M, N] of that dtype or float."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(out.shape) != (M, N) or a.dtype != w.dtype:
+        raise KernelError(f"gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
+    if accumulate:
+        if out.dtype != torch.float32:
+            raise KernelError("gemm: accumulation needs a float output")
+        mode = ACCUM_F32
+    elif out.dtype == torch.float32:
+        mode = STORE_F32
+    elif out.dtype == a.dtype:
+        mode = STORE_ACT
+    else:
+        raise KernelError(f"gemm: output dtype {out.dtype} for operands of {a.dtype}")
+    lib = core()
+    _check(lib.lyp_gemm_nt(_p(a), _p(w), _p(out), _code(a.dtype), mode, M, N, K, K, K, N, _stream()), lib)
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x @ w.T for a projection weight [out_features, in_features].  A weight
+    kept in 32-bit is multiplied in 32-bit whatever the activations are."""
+    out_dtype = out_dtype or x.dtype
+    if w.dtype != x.dtype:
+        if w.dtype != torch.float32:
+            raise KernelError(f"linear: weight {w.dtype} against activations {x.dtype}")
+        x = cast(x, torch.float32)
+    if out_dtype in (x.dtype, torch.float32):
+        out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
+        return gemm_nt(x, w, out)
+    out = torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
+    return cast(gemm_nt(x, w, out), out_dtype)
+
+
+# ------------------------------------------------------------------- attention
+def attn_part_keys(head_dim: int) -> int:
+    return attention_lib(head_dim).lyp_attn_part_keys()
+
+
+def _attn_check(q, out, kpool, vpool, block_tables, nh, nkv, hd):
+    _dev(out, kpool, vpool, block_tables)
+    n_pages, bs = kpool.shape[0], kpool.shape[2]
+    if (tuple(kpool.shape) != (n_pages, nkv, bs, hd) or tuple(vpool.shape) != (n_pages, nkv, hd, bs)
+            or kpool.dtype != q.dtype or vpool.dtype != q.dtype or out.dtype != q.dtype):
+        raise KernelError(f"attention: pools {tuple(kpool.shape)} / {tuple(vpool.shape)} {kpool.dtype} do not fit "
+                          f"{nkv} heads of {hd} and queries of {q.dtype}")
+    if q.stride(1) != 1 or q.stride(0) < nh * hd or tuple(out.shape) != (q.shape[0], nh * hd):
+        raise KernelError(f"attention: q {tuple(q.shape)} strides {q.stride()}, out {tuple(out.shape)}")
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2:
+        raise KernelError("attention: block tables must be a 2-d int32 tensor")
+    return bs
+
+
+def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
+                 block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor, tile_seq: torch.Tensor,
+                 tile_q0: torch.Tensor, n_tiles: int, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                 window: int = 0, scale: float | None = None) -> torch.Tensor:
+    """Attention of the step's new tokens over the paged cache (which already
+    holds their own keys).  q is a view [T, >= nh * hd] whose first nh * hd
+    columns are the query heads; a tile is 64 new tokens of one request."""
+    if not q.is_cuda or q.dim() != 2:
+        raise KernelError("attention: q must be a 2-d GPU tensor")
+    bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
+    _dev(q_start, ctx_len, tile_seq, tile_q0)
+    lib = attention_lib(head_dim)
+    scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+    _check(lib.lyp_attn_prefill(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
+                                _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(tile_seq),
+                                _p(tile_q0), n_tiles, num_heads, num_kv_heads, bs, window, scale, _stream()), lib)
+    return out
+
+
+def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
+                block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
+                dec_seqs: torch.Tensor | None, n_seqs: int, part_o: torch.Tensor, part_ml: torch.Tensor,
+                max_parts: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
+                scale: float | None = None) -> torch.Tensor:
+    """Attention of requests that bring one new token each, split over
+    partitions of the context and merged."""
+    if not q.is_cuda or q.dim() != 2:
+        raise KernelError("attention: q must be a 2-d GPU tensor")
+    bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
+    _dev(q_start, ctx_len, dec_seqs, part_o, part_ml)
+    if part_o.dtype != torch.float32 or part_ml.dtype != torch.float32 or \
+            part_o.numel() < n_seqs * num_heads * max_parts * head_dim or \
+            part_ml.numel() < n_seqs * num_heads * max_parts * 2:
+        raise KernelError("attention: partition workspace too small")
+    lib = attention_lib(head_dim)
+    scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+    _check(lib.lyp_attn_decode(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
+                               _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(dec_seqs),
+                               n_seqs, _p(part_o), _p(part_ml), max_parts, num_heads, num_kv_heads, bs, window,
+                               scale, _stream()), lib)
+    return out
+
+
+# -------------------------------------------------------------------- sampling
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(logits, temperature, top_k, top_p, uniform, out)
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or temperature.dtype != torch.float32 or top_k.dtype != torch.int32 or \
+            top_p.dtype != torch.float32 or uniform.dtype != torch.float32 or out.dtype != torch.int32:
+        raise KernelError("sample: logits, temperature, top_p, uniform float32; top_k, out int32")
+    if any(t.numel() != R for t in (temperature, top_k, top_p, uniform, out)):
+        raise KernelError("sample: one parameter per row")
+    lib = core()
+    _check(lib.lyp_sample(_p(logits), V, R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform), _p(out),
+                          _stream()), lib)
+    return out

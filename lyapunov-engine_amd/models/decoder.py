@@ -1,0 +1,155 @@
+"""A decoder put together from a ModelSpec: embedding, the layers in their
+running order, final norm, output head.
+
+The order of work is the reference's LlamaForCausalLM.forward
+(python/lyapunov_engine/models/llama.py:196-225): embed, layers, final norm,
+lm_head.  Differences: the batch is flat (tokens of several requests, each with
+its position), the final norm and the head run only on the rows whose logits are
+wanted (the reference computes all positions and the engine keeps the last,
+engine/llm_engine.py:272, 289), logits are float, and a tied head is the
+embedding matrix itself, not a copy (models/weight_loader.py:106-109 copies).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Iterator, Optional
+
+import torch
+
+from ..config.registry import BLOCKS, NORMS
+from ..config.specs import LayerCall, ModelSpec
+from ..kernels import ops
+from ..parts.base import KVCacheSpec, LayerCache, Part, StateSpec, StepContext, WeightSource, WeightSpec
+
+
+@dataclass(frozen=True)
+class CacheGroupLayout:
+    spec: KVCacheSpec
+    buffers: tuple          # cache ids (LayerCall.cache) whose keys and values live in this group
+
+
+@dataclass(frozen=True)
+class CacheLayout:
+    groups: tuple           # of CacheGroupLayout
+    states: dict            # cache id -> StateSpec
+
+    def group_of(self, cache_id: int) -> Optional[int]:
+        for g, layout in enumerate(self.groups):
+            if cache_id in layout.buffers:
+                return g
+        return None
+
+
+class DecoderModel(Part):
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.layers = [BLOCKS.get(ls.block)(ls) for ls in spec.layers]
+        self.final_norm = NORMS.build(spec.final_norm)
+        self.schedule: tuple = tuple(spec.schedule)
+        for call in self.schedule:
+            if not 0 <= call.layer < len(self.layers):
+                raise ValueError(f"the running order names layer {call.layer}; there are {len(self.layers)}")
+        self.embed: Optional[torch.Tensor] = None
+        self.lm_head: Optional[torch.Tensor] = None
+        self.device: Optional[torch.device] = None
+        self.dtype: Optional[torch.dtype] = None
+        self._layout = self._plan_cache()
+
+    # -------------------------------------------------------------- structure
+    def named_parts(self) -> Iterator[tuple]:
+        """(tensor-name prefix, part) for every part that may own weights."""
+        def walk(prefix: str, part: Part):
+            yield prefix, part
+            for piece, child in part.children().items():
+                yield from walk(prefix + piece, child)
+
+        for i, layer in enumerate(self.layers):
+            yield from walk(self.spec.layer_prefix.format(i=i), layer)
+        yield from walk(self.spec.final_norm_prefix, self.final_norm)
+
+    def weight_table(self) -> list:
+        """(owner, WeightSpec with full tensor names) for the whole model."""
+        out = []
+        V, H = self.spec.vocab_size, self.spec.hidden_size
+        out.append((self, WeightSpec("embed", (WeightSource(self.spec.embed_name, (V, H)),))))
+        if not self.spec.tie_word_embeddings:
+            out.append((self, WeightSpec("lm_head", (WeightSource(self.spec.head_name, (V, H)),))))
+        for prefix, part in self.named_parts():
+            for ws in part.weight_specs():
+                full = tuple(WeightSource(prefix + s.name, tuple(s.shape)) for s in ws.sources)
+                out.append((part, WeightSpec(ws.attr, full, ws.init)))
+        return out
+
+    def expected_tensors(self) -> dict:
+        """Tensor name in the model file -> (shape, init kind)."""
+        out = {}
+        for _, ws in self.weight_table():
+            for s in ws.sources:
+                if s.name in out:
+                    raise ValueError(f"two parts claim the tensor {s.name!r}")
+                out[s.name] = (tuple(s.shape), ws.init)
+        return out
+
+    def ignorable_tensors(self) -> set:
+        """Names a file may hold without being used: a tied model's separate head."""
+        return {self.spec.head_name} if self.spec.tie_word_embeddings else set()
+
+    def _plan_cache(self) -> CacheLayout:
+        by_cache: dict = {}
+        states: dict = {}
+        for call in self.schedule:
+            mixer = self.layers[call.layer].mixer
+            kv, st = mixer.cache_spec(), mixer.state_spec()
+            if kv is not None:
+                if call.cache in by_cache and by_cache[call.cache] != kv:
+                    raise ValueError(f"cache buffer {call.cache} is used with two shapes: {by_cache[call.cache]} and {kv}")
+                by_cache.setdefault(call.cache, kv)
+            if st is not None:
+                if call.cache in states and states[call.cache] != st:
+                    raise ValueError(f"state buffer {call.cache} is used with two shapes")
+                states.setdefault(call.cache, st)
+        written = {c.cache for c in self.schedule if c.writes}
+        for call in self.schedule:
+            if not call.writes and call.cache not in written:
+                raise ValueError(f"layer call reads cache buffer {call.cache}, which no call writes")
+        order: list = []
+        for call in self.schedule:  # groups in order of first use
+            kv = by_cache.get(call.cache)
+            if kv is not None and kv not in order:
+                order.append(kv)
+        groups = tuple(CacheGroupLayout(kv, tuple(sorted(c for c, s in by_cache.items() if s == kv))) for kv in order)
+        return CacheLayout(groups, states)
+
+    def cache_layout(self) -> CacheLayout:
+        return self._layout
+
+    # ---------------------------------------------------------------- weights
+    def materialize(self, device, dtype):
+        self.device, self.dtype = torch.device(device), dtype
+        for layer in self.layers:
+            layer.materialize(self.device, dtype)
+        self.final_norm.materialize(self.device, dtype)
+        if self.spec.tie_word_embeddings:
+            self.lm_head = self.embed
+
+    # ---------------------------------------------------------------- compute
+    def forward(self, ctx: StepContext, caches: list) -> Optional[torch.Tensor]:
+        """Run the step's tokens through every call of the running order;
+        returns float logits [R, vocab] for ``ctx.logit_rows`` (None if R == 0).
+        ``caches[i]`` is the LayerCache of ``schedule[i]``."""
+        h = torch.empty((ctx.T, self.spec.hidden_size), dtype=torch.float32, device=ctx.device)
+        ops.embedding(ctx.token_ids, self.embed, h)
+        delta = None
+        for call, cache in zip(self.schedule, caches):
+            h, delta = self.layers[call.layer].forward(ctx, h, delta, cache)
+        if ctx.R == 0:
+            return None
+        x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
+        return ops.linear(x, self.lm_head, out_dtype=torch.float32)
+
+
+def build_model(spec: ModelSpec) -> DecoderModel:
+    return DecoderModel(spec)
+
+
+__all__ = ["DecoderModel", "CacheLayout", "CacheGroupLayout", "build_model", "LayerCall", "StateSpec"]

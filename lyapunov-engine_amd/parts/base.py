@@ -1,0 +1,198 @@
+"""Interfaces of the parts a decoder layer is made of, and of what a step hands
+to them.
+
+A part is built from sizes and constants alone (never from a model name), says
+which tensors it wants (``weight_specs``), what it needs from the cache
+(``cache_spec`` / ``state_spec``, mixers only), and computes in ``forward``.
+The model builder looks parts up in the registries of ``config.registry``; a
+part defined anywhere (a test, another package) that follows these interfaces
+and registers itself can be used by a ModelSpec without touching this package.
+
+Conventions every part may rely on:
+  * the hidden state ``h`` is the float residual stream ``[T, hidden]``;
+    a part's output ``y`` has the step's activation dtype (``ctx.dtype``) and is
+    added to ``h`` by the *next* norm (``Norm.forward(ctx, h, delta=y)``), in
+    32-bit;
+  * ``T`` is the number of tokens of the step, all requests' tokens flattened;
+    request ``b`` owns rows ``q_start[b] .. q_start[b+1]``, in position order;
+  * a part's result for a token may depend on earlier tokens of the same request
+    (through the cache it is handed) and on nothing else in the batch.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Optional
+
+import torch
+
+
+# --------------------------------------------------------------------- weights
+@dataclass(frozen=True)
+class WeightSource:
+    name: str              # tensor name in the file, relative to the part's prefix
+    shape: tuple
+
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One tensor of a part: attribute ``attr`` receives the sources
+    concatenated along dimension 0 (one source: the tensor itself)."""
+
+    attr: str
+    sources: tuple         # of WeightSource
+    init: str = "normal"   # random-weights mode: "normal" (0, std) or "ones" (1 + noise)
+
+    @property
+    def shape(self) -> tuple:
+        first = self.sources[0].shape
+        return (sum(s.shape[0] for s in self.sources),) + tuple(first[1:])
+
+
+class Part:
+    """Anything that may own weights and sub-parts."""
+
+    def weight_specs(self) -> list:
+        return []
+
+    def children(self) -> dict:
+        """Sub-parts by the piece of tensor-name prefix that leads to them
+        (for example ``{"q_norm.": self.q_norm}``)."""
+        return {}
+
+    def materialize(self, device: torch.device, dtype: torch.dtype) -> None:
+        """Build device tables that are computed rather than loaded."""
+        for c in self.children().values():
+            c.materialize(device, dtype)
+
+
+# ----------------------------------------------------------------------- cache
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values in pages.  Calls whose specs are equal share a group:
+    one pool of pages, one block table per request."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0        # 0: all keys; W: a token sees the last W keys, itself included
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """State of fixed size per live request (a slot of ``shape``), for mixers
+    that carry a summary instead of keys."""
+
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class GroupView:
+    """A cache group as a step sees it."""
+
+    page_size: int
+    block_tables: torch.Tensor        # int32 [B, max_blocks]; -1 where a page was given back
+    slot_mapping: torch.Tensor        # int32 [T]: page * page_size + offset of each new token
+    max_blocks: int
+    window: int = 0
+
+
+@dataclass
+class LayerCache:
+    """What one call of a layer gets from the cache."""
+
+    group: Optional[GroupView] = None
+    k: Optional[torch.Tensor] = None      # [pages, kv heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None      # [pages, kv heads, head_dim, page_size]
+    state: Optional[torch.Tensor] = None  # [slots, *StateSpec.shape]
+    writes: bool = True                   # false: read what another call stored
+
+
+@dataclass
+class StepContext:
+    """Everything about the batch of one step, on the device and on the host."""
+
+    device: torch.device
+    dtype: torch.dtype                    # activation dtype of the step
+    T: int
+    B: int
+    token_ids: torch.Tensor               # int32 [T]
+    positions: torch.Tensor               # int32 [T] absolute positions
+    q_start: torch.Tensor                 # int32 [B + 1]
+    ctx_len: torch.Tensor                 # int32 [B] length of each request after the step
+    state_slots: torch.Tensor             # int32 [B]
+    logit_rows: torch.Tensor              # int32 [R] rows of the flat batch whose logits are wanted
+    R: int
+    groups: list                          # of GroupView
+    # attention work lists: requests with more than one new token are cut into
+    # tiles of 64 tokens, requests with exactly one go to the split kernel
+    tile_seq: torch.Tensor
+    tile_q0: torch.Tensor
+    n_tiles: int
+    dec_seqs: Optional[torch.Tensor]
+    n_dec: int
+    max_ctx_dec: int                      # longest context among the single-token requests
+    # host copies for parts written in Python
+    q_start_host: list = field(default_factory=list)
+    ctx_len_host: list = field(default_factory=list)
+    state_slots_host: list = field(default_factory=list)
+    workspace: dict = field(default_factory=dict)   # scratch tensors shared by the layers of a step
+
+    def scratch(self, key: str, numel: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        t = self.workspace.get(key)
+        if t is None or t.numel() < numel or t.dtype != dtype:
+            t = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
+            self.workspace[key] = t
+        return t
+
+
+# ------------------------------------------------------------------ part kinds
+class Norm(Part):
+    def forward(self, ctx: StepContext, h: torch.Tensor, delta: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Add ``delta`` to ``h`` (in place, 32-bit), norm, return activations.
+        With ``rows`` only those rows are normed and ``h`` is left alone."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Turns positions into whatever the mixer applies.  The rotary kind exposes
+    ``table`` (float [max_position, rotary_dim]: cosines then sines)."""
+
+    table: Optional[torch.Tensor] = None
+    rotary_dim: int = 0
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request."""
+
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of a mixer, a feed-forward and their norms around the
+    residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, delta: Optional[torch.Tensor],
+                cache: LayerCache) -> tuple:
+        """-> (h, delta): the residual stream and the output not yet added to it."""
+        raise NotImplementedError
+
+
+__all__ = [
+    "WeightSource", "WeightSpec", "Part", "KVCacheSpec", "StateSpec", "GroupView", "LayerCache", "StepContext",
+    "Norm", "PositionEncoding", "Mixer", "FeedForward", "Block", "Any",
+]

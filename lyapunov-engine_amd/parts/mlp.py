@@ -1,0 +1,37 @@
+"""SiLU-gated feed-forward.
+
+down( silu(gate(x)) * up(x) ), no biases, with gate and up as one matrix whose
+first rows are the gate (python/lyapunov_engine/models/llama.py:109-122;
+models/weight_loader.py:155-163 builds cat([gate, up], dim=0); the activation is
+python/lyapunov_engine/ops.py:72-73).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config.registry import FEED_FORWARDS
+from ..kernels import ops
+from .base import FeedForward, StepContext, WeightSource, WeightSpec
+
+
+@FEED_FORWARDS.register("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.gate_up_proj: Optional[torch.Tensor] = None
+        self.down_proj: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        shape = (self.intermediate_size, self.hidden_size)
+        return [
+            WeightSpec("gate_up_proj", (WeightSource("gate_proj.weight", shape), WeightSource("up_proj.weight", shape))),
+            WeightSpec("down_proj", (WeightSource("down_proj.weight", (self.hidden_size, self.intermediate_size)),)),
+        ]
+
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        gate_up = ops.linear(x, self.gate_up_proj, out_dtype=ctx.dtype)
+        act = torch.empty((x.shape[0], self.intermediate_size), dtype=ctx.dtype, device=x.device)
+        ops.swiglu(gate_up, act)
+        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype)

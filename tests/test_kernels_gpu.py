@@ -1,0 +1,332 @@
+"""Each HIP kernel alone against the plain formulas, at sizes other than the
+tiny models' (odd widths, several head sizes, page sizes 4/8/16, windows)."""
+import math
+
+import pytest
+import torch
+
+from plain import llama_plain as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, f32=2e-5, bf16=2e-2):
+    return dict(rtol=f32, atol=f32) if dtype == torch.float32 else dict(rtol=bf16, atol=bf16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from lyapunov_engine_amd.kernels import ops as o
+    o.require_gpu()
+    return o
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+# ------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops, dtype):
+    V, H, T = 1000, 192, 37
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.randint(0, V, (T,), generator=torch.Generator().manual_seed(1), dtype=torch.int32)
+    out = torch.empty(T, H, dtype=torch.float32, device=DEV)
+    ops.embedding(ids.to(DEV), table.to(DEV), out)
+    torch.testing.assert_close(out.cpu(), table.float()[ids.long()], rtol=0, atol=0)
+
+
+# --------------------------------------------------------------------- rmsnorm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,T", [(96, 1), (1000, 7), (2048, 33), (4100, 3)])
+def test_rmsnorm(ops, dtype, H, T):
+    eps = 1e-5
+    h = rnd(T, H, seed=3)
+    w = (1 + 0.1 * rnd(H, seed=4)).to(dtype)
+    out = torch.empty(T, H, dtype=dtype, device=DEV)
+    hd = h.to(DEV)
+    ops.rmsnorm(hd, w.to(DEV), eps, out)
+    want = P.rms_norm(h.double(), w.double(), eps)
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 1e-5, 1e-2))
+    torch.testing.assert_close(hd.cpu(), h, rtol=0, atol=0)  # no delta: the stream is untouched
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_adds_the_residual_in_32_bit(ops, dtype):
+    T, H, eps = 9, 200, 1e-6
+    h, delta = rnd(T, H, seed=5), rnd(T, H, seed=6, dtype=dtype)
+    w = rnd(H, seed=7).to(dtype)
+    hd = h.to(DEV)
+    out = torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.rmsnorm(hd, w.to(DEV), eps, out, delta=delta.to(DEV))
+    total = h + delta.float()
+    torch.testing.assert_close(hd.cpu(), total, rtol=0, atol=0)  # the sum lands in the float stream, unrounded
+    torch.testing.assert_close(out.cpu().double(), P.rms_norm(total.double(), w.double(), eps), **tol(dtype, 1e-5, 1e-2))
+    # rows: only the picked rows are normed and the stream is left alone
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32)
+    hd2 = h.to(DEV)
+    out2 = torch.empty(3, H, dtype=dtype, device=DEV)
+    ops.rmsnorm(hd2, w.to(DEV), eps, out2, delta=delta.to(DEV), rows=rows.to(DEV))
+    torch.testing.assert_close(hd2.cpu(), h, rtol=0, atol=0)
+    torch.testing.assert_close(out2.cpu().double(), P.rms_norm(total.double(), w.double(), eps)[rows.long()],
+                               **tol(dtype, 1e-5, 1e-2))
+
+
+# ---------------------------------------------------------------------- swiglu
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("I,T", [(172, 5), (512, 1), (8192, 3)])
+def test_swiglu(ops, dtype, I, T):
+    gu = rnd(T, 2 * I, dtype=dtype, scale=2.0, seed=8)
+    out = torch.empty(T, I, dtype=dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out)
+    torch.testing.assert_close(out.cpu().double(), P.swiglu(gu.double()), **tol(dtype, 1e-5, 1e-2))
+
+
+# ------------------------------------------------------------------------ gemm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 172, 96), (33, 256, 172), (130, 1000, 200), (200, 513, 96),
+                                   (64, 128, 4096), (3, 130, 33), (65, 96, 30)])
+def test_gemm(ops, dtype, M, N, K):
+    a, w = rnd(M, K, dtype=dtype, seed=9), rnd(N, K, dtype=dtype, scale=0.05, seed=10)
+    want = a.double() @ w.double().T
+    bound = (a.double().abs() @ w.double().abs().T)  # size of the sum of magnitudes: the scale of rounding error
+    for out_dtype in {dtype, torch.float32}:
+        out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops.gemm_nt(a.to(DEV), w.to(DEV), out)
+        err = (out.cpu().double() - want).abs()
+        rel = 2e-6 if dtype == torch.float32 else (1e-5 if out_dtype == torch.float32 else 1e-2)
+        assert (err <= rel * bound + 1e-30).all(), f"max err {err.max()} vs bound {bound.max()}"
+    acc = rnd(M, N, seed=11)
+    out = acc.to(DEV)
+    ops.gemm_nt(a.to(DEV), w.to(DEV), out, accumulate=True)
+    err = (out.cpu().double() - (acc.double() + want)).abs()
+    assert (err <= 1e-5 * (bound + acc.double().abs())).all()
+
+
+def test_gemm_float_is_true_32_bit(ops):
+    """A product whose low bits a reduced-precision matrix mode would drop."""
+    K = 64
+    a = torch.full((4, K), 1.0 + 2.0 ** -12)
+    w = torch.full((8, K), 1.0 + 2.0 ** -11)
+    out = torch.empty(4, 8, dtype=torch.float32, device=DEV)
+    ops.gemm_nt(a.to(DEV), w.to(DEV), out)
+    want = float(K * (1.0 + 2.0 ** -12) * (1.0 + 2.0 ** -11))
+    assert abs(out.cpu()[0, 0].item() - want) < 1e-4  # a 10-bit mantissa would be off by ~0.05
+
+
+# ----------------------------------------------------- rotation and page write
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,bs", [(6, 2, 48, 8), (4, 4, 16, 4), (3, 1, 128, 16)])
+def test_rope_kv_write(ops, dtype, nh, nkv, hd, bs):
+    T, n_pages, max_pos = 11, 7, 64
+    qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=12)
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 42, 63, 5, 6, 7], dtype=torch.int32)
+    inv_freq = P.rope_inv_freq(hd, 10000.0)
+    cos_all, sin_all = P.rope_cos_sin(torch.arange(max_pos), inv_freq)
+    table = torch.cat((cos_all[:, : hd // 2], sin_all[:, : hd // 2]), dim=-1).contiguous()
+    slots = torch.randperm(n_pages * bs, generator=torch.Generator().manual_seed(13))[:T].to(torch.int32)
+    slots[4] = -1  # "do not store"
+    kpool = torch.zeros(n_pages, nkv, bs, hd, dtype=dtype, device=DEV)
+    vpool = torch.zeros(n_pages, nkv, hd, bs, dtype=dtype, device=DEV)
+    dev = qkv.to(DEV)
+    ops.rope_kv_write(dev, positions.to(DEV), table.to(DEV), slots.to(DEV), kpool, vpool, num_heads=nh,
+                      num_kv_heads=nkv, head_dim=hd, page_size=bs)
+    got = dev.cpu().float().view(T, nh + 2 * nkv, hd)
+    src = qkv.float().view(T, nh + 2 * nkv, hd)
+    cos, sin = P.rope_cos_sin(positions, inv_freq)
+    want_qk = P.apply_rope(src[:, : nh + nkv].transpose(0, 1), cos, sin).transpose(0, 1)
+    t = tol(dtype, 1e-6, 1e-2)
+    torch.testing.assert_close(got[:, : nh + nkv], want_qk, **t)
+    torch.testing.assert_close(got[:, nh + nkv:], src[:, nh + nkv:], rtol=0, atol=0)  # values are not rotated
+    torch.testing.assert_close(got[0, :nh], src[0, :nh], rtol=0, atol=0)  # position 0 is the identity
+    kp, vp = kpool.cpu().float(), vpool.cpu().float()
+    for i in range(T):
+        if slots[i] < 0:
+            continue
+        page, off = int(slots[i]) // bs, int(slots[i]) % bs
+        torch.testing.assert_close(kp[page, :, off, :], got[i, nh: nh + nkv], rtol=0, atol=0)
+        torch.testing.assert_close(vp[page, :, :, off], got[i, nh + nkv:], rtol=0, atol=0)
+    written = sum(1 for s in slots.tolist() if s >= 0)
+    assert int((kp.abs().sum(-1) > 0).sum()) == written * nkv  # nothing else was touched
+
+
+# ------------------------------------------------------------------- attention
+def paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=0, n_pages=None):
+    """seqs: list of (ctx_len, q_len).  Random q for the new tokens, k/v for the
+    whole context, scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    need = sum(-(-c // bs) for c, _ in seqs)
+    n_pages = n_pages or need + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    kpool = torch.randn(n_pages, nkv, bs, hd, generator=g).to(dtype) * 3  # stale data everywhere
+    vpool = torch.randn(n_pages, nkv, hd, bs, generator=g).to(dtype) * 3
+    width = max(-(-c // bs) for c, _ in seqs)
+    bt = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    qs, ks, vs, q_start = [], [], [], [0]
+    for b, (ctx, ql) in enumerate(seqs):
+        k = torch.randn(nkv, ctx, hd, generator=g).to(dtype)
+        v = torch.randn(nkv, ctx, hd, generator=g).to(dtype)
+        q = torch.randn(nh, ql, hd, generator=g).to(dtype)
+        pages = [perm.pop() for _ in range(-(-ctx // bs))]
+        bt[b, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        for p in range(ctx):
+            kpool[pages[p // bs], :, p % bs, :] = k[:, p]
+            vpool[pages[p // bs], :, :, p % bs] = v[:, p]
+        qs.append(q), ks.append(k), vs.append(v)
+        q_start.append(q_start[-1] + ql)
+    q_flat = torch.cat([q.transpose(0, 1).reshape(q.shape[1], nh * hd) for q in qs], dim=0)
+    return dict(q=q_flat, qs=qs, ks=ks, vs=vs, kpool=kpool, vpool=vpool, bt=bt,
+                q_start=torch.tensor(q_start, dtype=torch.int32),
+                ctx_len=torch.tensor([c for c, _ in seqs], dtype=torch.int32))
+
+
+def plain_attention(s, seqs, window):
+    outs = []
+    for (ctx, ql), q, k, v in zip(seqs, s["qs"], s["ks"], s["vs"]):
+        o = P.attention(q.double(), k.double(), v.double(), torch.arange(ctx - ql, ctx), torch.arange(ctx),
+                        window=window)
+        outs.append(o.transpose(0, 1).reshape(ql, -1))
+    return torch.cat(outs, dim=0)
+
+
+PREFILL_CASES = [
+    # nh, nkv, hd, bs, window, [(ctx, q_len)]
+    (4, 2, 16, 4, 0, [(5, 5), (17, 17), (33, 33)]),
+    (3, 1, 32, 16, 0, [(130, 130), (9, 9), (64, 2), (70, 7)]),
+    (6, 2, 48, 8, 0, [(100, 37), (65, 65), (200, 3)]),
+    (8, 2, 64, 16, 0, [(300, 150), (64, 64), (129, 2)]),
+    (4, 4, 128, 16, 0, [(90, 31), (17, 5)]),
+    (32, 8, 64, 16, 0, [(700, 200)]),
+    (5, 5, 80, 16, 0, [(40, 40)]),
+    (4, 2, 32, 4, 9, [(50, 50), (33, 6), (20, 2)]),
+    (2, 1, 64, 16, 40, [(200, 100), (41, 3)]),
+    (16, 1, 16, 2, 0, [(23, 11)]),  # a page size that is no multiple of 4: the scalar load path
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", PREFILL_CASES, ids=[str(c[:5]) for c in PREFILL_CASES])
+def test_attention_prefill(ops, dtype, case):
+    nh, nkv, hd, bs, window, seqs = case
+    s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=hd + bs)
+    tile_seq, tile_q0 = [], []
+    for b, (_, ql) in enumerate(seqs):
+        for q0 in range(0, ql, 64):
+            tile_seq.append(b), tile_q0.append(q0)
+    out = torch.full((s["q"].shape[0], nh * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.attn_prefill(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
+                     s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(tile_seq, dtype=torch.int32, device=DEV),
+                     torch.tensor(tile_q0, dtype=torch.int32, device=DEV), len(tile_seq), num_heads=nh,
+                     num_kv_heads=nkv, head_dim=hd, window=window)
+    want = plain_attention(s, seqs, window)
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+DECODE_CASES = [
+    (4, 2, 16, 4, 0, [1, 15, 64, 65]),
+    (3, 1, 32, 16, 0, [300, 1, 129]),
+    (32, 8, 64, 16, 0, [1000, 17]),
+    (6, 2, 48, 8, 0, [48, 200]),
+    (4, 1, 128, 16, 0, [513]),
+    (40, 2, 32, 16, 0, [77]),        # more than 16 query heads per key/value head
+    (4, 2, 32, 4, 9, [50, 5, 9, 10]),
+    (2, 1, 64, 16, 100, [700, 64]),
+    (16, 1, 16, 2, 0, [23]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", DECODE_CASES, ids=[str(c[:5]) for c in DECODE_CASES])
+def test_attention_decode(ops, dtype, case):
+    nh, nkv, hd, bs, window, ctxs = case
+    seqs = [(c, 1) for c in ctxs]
+    s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=hd + bs + 1)
+    n = len(seqs)
+    part = ops.attn_part_keys(hd)
+    max_parts = -(-max(ctxs) // part)
+    part_o = torch.full((n * nh * max_parts * hd,), float("nan"), device=DEV)
+    part_ml = torch.full((n * nh * max_parts * 2,), float("nan"), device=DEV)
+    out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
+    # the requests in shuffled order through dec_seqs
+    order = list(reversed(range(n)))
+    ops.attn_decode(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
+                    s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(order, dtype=torch.int32, device=DEV), n,
+                    part_o, part_ml, max_parts, num_heads=nh, num_kv_heads=nkv, head_dim=hd, window=window)
+    want = plain_attention(s, seqs, window)
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["prefill", "decode"])
+def test_attention_finds_one_far_key(ops, dtype, kind):
+    """Among 900 keys one, far back, matches the query strongly: the output is
+    that key's value.  Random data would hide a kernel that drops distant keys
+    or a page."""
+    nh, nkv, hd, bs, ctx, far = 4, 2, 64, 16, 900, 37
+    ql = 1 if kind == "decode" else 5
+    seqs = [(ctx, ql)]
+    s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=5)
+    k = s["ks"][0]
+    k[:, far] = 4.0
+    s["qs"][0][:] = 4.0   # score with the far key: 16 * 64 / 8 = 128; with the others ~ N(0, 32)
+    pages = s["bt"][0].tolist()
+    s["kpool"][pages[far // bs], :, far % bs, :] = k[:, far]
+    s["q"] = torch.cat([q.transpose(0, 1).reshape(q.shape[1], nh * hd) for q in s["qs"]], dim=0)
+    out = torch.empty((ql, nh * hd), dtype=dtype, device=DEV)
+    args = (s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV), s["q_start"].to(DEV),
+            s["ctx_len"].to(DEV))
+    kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd)
+    if kind == "decode":
+        mp = -(-ctx // ops.attn_part_keys(hd))
+        ops.attn_decode(*args, None, 1, torch.empty(nh * mp * hd, device=DEV), torch.empty(nh * mp * 2, device=DEV),
+                        mp, **kw)
+    else:
+        ops.attn_prefill(*args, torch.zeros(1, dtype=torch.int32, device=DEV),
+                         torch.zeros(1, dtype=torch.int32, device=DEV), 1, **kw)
+    v_far = s["vs"][0][:, far].float()  # [nkv, hd]
+    want = v_far.repeat_interleave(nh // nkv, dim=0).reshape(1, nh * hd).expand(ql, -1)
+    torch.testing.assert_close(out.cpu().float(), want, rtol=1e-2, atol=1e-2)
+
+
+# --------------------------------------------------------------------- sampler
+def test_sampler_greedy_and_draws(ops):
+    V = 1003
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(6, V, generator=g) * 3
+    logits[1, 500] = logits[1, 7] = logits[1].max() + 1  # a tie: the first index wins
+    temperature = torch.tensor([0.0, 0.0, 0.8, 1.3, 0.7, 1.0])
+    top_k = torch.tensor([-1, -1, -1, 40, -1, 5], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 1.0, 1.0, 0.6, 0.9])
+    for u_val in (0.0, 0.137, 0.5, 0.77, 0.999):
+        u = torch.full((6,), u_val)
+        out = torch.empty(6, dtype=torch.int32, device=DEV)
+        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out)
+        got = out.cpu().tolist()
+        assert got[0] == P.greedy(logits[0])
+        assert got[1] == 7
+        for r in range(2, 6):
+            probs = P.sample_filter(logits[r], float(temperature[r]), int(top_k[r]), float(top_p[r]))
+            assert probs[got[r]] > 0, f"row {r}: token {got[r]} was filtered out"
+            cdf = torch.cumsum(probs, 0)
+            lo = float(cdf[got[r]] - probs[got[r]])
+            assert lo - 1e-5 <= u_val <= float(cdf[got[r]]) + 1e-5, f"row {r}: u={u_val} not in [{lo}, {float(cdf[got[r]])}]"
+
+
+def test_sampler_top_k_one_is_greedy_and_frequencies(ops):
+    V = 50
+    logits = torch.randn(1, V, generator=torch.Generator().manual_seed(4))
+    n = 4000
+    rows = logits.expand(n, V).contiguous().to(DEV)
+    u = torch.rand(n, generator=torch.Generator().manual_seed(5))
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ones = torch.ones(n)
+    ops.sample(rows, (ones * 0.9).to(DEV), torch.ones(n, dtype=torch.int32).to(DEV), ones.to(DEV), u.to(DEV), out)
+    assert set(out.cpu().tolist()) == {int(logits.argmax())}
+    ops.sample(rows, (ones * 0.9).to(DEV), torch.full((n,), -1, dtype=torch.int32).to(DEV), ones.to(DEV), u.to(DEV), out)
+    freq = torch.bincount(out.cpu().long(), minlength=V).double() / n
+    probs = torch.softmax(logits[0].double() / 0.9, 0)
+    assert (freq - probs).abs().max() < 0.03
