@@ -1,0 +1,138 @@
+"""Decode steps replayed from captured HIP graphs.
+
+A step in which every request brings exactly one token launches some hundred
+small kernels; launched one by one from Python, the launches cost more than the
+kernels.  Such steps are captured once per (batch bucket, context bucket) and
+replayed: the step's tables are copied into fixed device buffers, the graph
+runs, the logits are read from a fixed tensor.
+
+The reference buckets by batch size {1, 2, 4, ... 64}, takes the smallest bucket
+that fits, pads with zeros and slices the result
+(python/lyapunov_engine/engine/cuda_graph_runner.py:15-16, 59-80; the C++ runner,
+csrc/engine/cuda_graph.cpp:15-68, warms up once and then captures).  Its graph
+holds a model call without a cache (cuda_graph_runner.py:43-49).  Here the graph
+holds the real step over the paged cache; padded rows have a context of 0 (the
+attention kernels skip them) and a cache slot of -1 (nothing is stored).  The
+context bucket bounds the width of the block tables and the number of attention
+partitions a launch provides for.
+
+Nothing that clears memory with a memset is recorded: the kernels write every
+value they later read.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..parts.base import GroupView, StepContext
+from .runner import ModelRunner, _align4
+
+
+def _bucket(n: int, smallest: int) -> int:
+    b = smallest
+    while b < n:
+        b *= 2
+    return b
+
+
+class _Captured:
+    def __init__(self, runner: ModelRunner, batch: int, ctx_cap: int, pool):
+        self.batch, self.ctx_cap = batch, ctx_cap
+        cache = runner.cache
+        B = batch
+        # layout of the fixed table buffer, in int32 words
+        self.sizes = [B, B, B + 1, B, B, B]   # token ids, positions, q_start, ctx_len, state slots, logit rows
+        self.widths = []
+        for gc in cache.groups:
+            width = max(1, -(-ctx_cap // gc.page_size))
+            self.widths.append(width)
+            self.sizes += [B, B * width]
+        self.offsets, total = [], 0
+        for s in self.sizes:
+            self.offsets.append(total)
+            total += _align4(s)
+        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.workspace: dict = {}
+        h = self.host.numpy()
+        h[self.offsets[2]:self.offsets[2] + B + 1] = np.arange(B + 1)
+        h[self.offsets[5]:self.offsets[5] + B] = np.arange(B)
+        self.fill(runner, [])
+        self.dev.copy_(self.host)
+
+        def view(i):
+            return self.dev[self.offsets[i]:self.offsets[i] + self.sizes[i]]
+
+        groups = [GroupView(page_size=gc.page_size, block_tables=view(7 + 2 * g).view(B, self.widths[g]),
+                            slot_mapping=view(6 + 2 * g), max_blocks=self.widths[g], window=gc.window)
+                  for g, gc in enumerate(cache.groups)]
+        empty = self.dev[:0]
+        self.ctx = StepContext(
+            device=runner.device, dtype=runner.dtype, T=B, B=B, token_ids=view(0), positions=view(1), q_start=view(2),
+            ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=B, groups=groups, tile_seq=empty,
+            tile_q0=empty, n_tiles=0, dec_seqs=None, n_dec=B, max_ctx_dec=ctx_cap, q_start_host=list(range(B + 1)),
+            ctx_len_host=[0] * B, state_slots_host=[0] * B, workspace=self.workspace)
+        caches = runner.layer_caches(self.ctx)
+        # One run outside the capture loads the libraries and sizes the scratch
+        # buffers; with every context at 0 it stores nothing in the cache.
+        runner.model.forward(self.ctx, caches)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=pool):
+            self.logits = runner.model.forward(self.ctx, caches)
+
+    def fill(self, runner: ModelRunner, entries: list) -> None:
+        """Write the step's tables into the pinned host buffer; rows past the
+        entries are inert."""
+        B, cache, h, o = self.batch, runner.cache, self.host.numpy(), self.offsets
+        n = len(entries)
+        h[o[0]:o[0] + B] = 0
+        h[o[1]:o[1] + B] = 0
+        h[o[3]:o[3] + B] = 0
+        h[o[4]:o[4] + B] = 0
+        for b, e in enumerate(entries):
+            h[o[0] + b] = e.tokens[0]
+            h[o[1] + b] = e.start
+            h[o[3] + b] = e.start + 1
+            h[o[4] + b] = cache.state_slot(e.seq_id)
+        for g, gc in enumerate(cache.groups):
+            width, ps = self.widths[g], gc.page_size
+            sm = h[o[6 + 2 * g]:o[6 + 2 * g] + B]
+            bt = h[o[7 + 2 * g]:o[7 + 2 * g] + B * width].reshape(B, width)
+            sm[:] = -1
+            bt[n:] = -1
+            for b, e in enumerate(entries):
+                t = cache.table(e.seq_id, g)
+                bt[b, :len(t)] = t
+                bt[b, len(t):] = -1
+                sm[b] = t[e.start // ps] * ps + e.start % ps
+
+    def run(self, runner: ModelRunner, entries: list) -> torch.Tensor:
+        self.fill(runner, entries)
+        self.dev.copy_(self.host, non_blocking=True)
+        self.graph.replay()
+        return self.logits[:len(entries)]
+
+
+class DecodeGraphs:
+    MIN_CTX = 256
+
+    def __init__(self, runner: ModelRunner, max_batch: int):
+        self.runner = runner
+        self.max_batch = _bucket(max_batch, 1)
+        self.captured: dict = {}
+        self.pool = None
+
+    def usable(self, entries: list) -> bool:
+        return all(len(e.tokens) == 1 and e.want == [0] for e in entries) and len(entries) <= self.max_batch
+
+    def step(self, entries: list) -> torch.Tensor:
+        """Logits [len(entries), vocab]; valid until the next graph step."""
+        ctx_need = max(e.start + 1 for e in entries)
+        key = (_bucket(len(entries), 1), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
+        cap = self.captured.get(key)
+        if cap is None:
+            if self.pool is None:
+                self.pool = torch.cuda.graph_pool_handle()
+            cap = self.captured[key] = _Captured(self.runner, key[0], key[1], self.pool)
+        return cap.run(self.runner, entries)

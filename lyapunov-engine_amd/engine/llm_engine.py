@@ -1,0 +1,177 @@
+"""The generating engine: requests in, tokens out.
+
+Names and meanings follow the reference's LLMEngine
+(python/lyapunov_engine/engine/llm_engine.py:93-312): ``add_request`` in both of
+its forms (:165-212), ``has_unfinished_requests`` (:214-217), ``step`` returning
+a ``RequestOutput`` per scheduled request with the tokens produced so far
+(:219-310), and ``RequestOutput``'s fields (:41-55).  Added: ``abort_request``,
+``generate`` (the loop of entrypoints/cli.py:41-46 over a list of prompts), a
+finish reason that tells "stop" from "length" (the reference always says
+"stop", :307), and a request counter that moves once per request (the reference
+bumps it twice for an anonymous request, :184-185, 193-194).
+
+One step: the scheduler plans (prompt portions and decoded tokens, pages taken),
+the step function runs the plan as one batch, the sampler picks a token for
+every request whose known tokens are now all in the cache, the scheduler takes
+the tokens and finishes or frees what is done.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .core import EngineCore
+from .runner import StepEntry
+from .scheduler import FINISH_REASON, Scheduler
+
+
+class RequestOutput:
+    def __init__(self, request_id, prompt_tokens: list, output_tokens: list, finished: bool,
+                 finish_reason: Optional[str] = None):
+        self.request_id = request_id
+        self.prompt_tokens = prompt_tokens
+        self.output_tokens = output_tokens
+        self.finished = finished
+        self.is_finished = finished
+        self.finish_reason = finish_reason
+
+    def __repr__(self):
+        return (f"RequestOutput(request_id={self.request_id!r}, output_tokens={self.output_tokens}, "
+                f"finished={self.finished}, finish_reason={self.finish_reason!r})")
+
+
+class LLMEngine:
+    def __init__(self, model, config: Optional[EngineConfig] = None, **kw):
+        """``model`` is an ``EngineCore``, or a model folder (then the core is
+        built from ``config``)."""
+        config = config or EngineConfig(**kw)
+        self.config = config
+        if isinstance(model, EngineCore):
+            self.core = model
+        else:
+            self.core = EngineCore.from_folder(str(model), dtype=config.dtype, device=config.device,
+                                               num_blocks=config.num_blocks, block_size=config.block_size,
+                                               num_state_slots=config.max_num_seqs)
+        spec = self.core.model.spec
+        self.max_model_len = min(config.max_model_len or spec.max_position, spec.max_position)
+        eos = config.eos_token_ids if config.eos_token_ids is not None else spec.eos_token_ids
+        self.scheduler = Scheduler(self.core.cache, max_num_seqs=config.max_num_seqs,
+                                   max_num_batched_tokens=config.max_num_batched_tokens,
+                                   max_model_len=self.max_model_len, max_chunk=config.max_chunk,
+                                   eos_token_ids=tuple(eos))
+        self.sampler = Sampler(self.core.device, seed=config.seed)
+        self.req_counter = 0
+        self._requests: dict = {}     # seq id -> (request id, SamplingParams, stream)
+        self._by_request: dict = {}   # request id -> seq id
+        self.graphs = None
+        if config.enable_graphs:
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self.core.runner, max_batch=config.max_num_seqs)
+
+    # ---------------------------------------------------------------- requests
+    def add_request(self, arg1, arg2=None, arg3=None):
+        """``add_request(prompt_tokens, sampling_params)`` or
+        ``add_request(request_id, prompt_tokens, sampling_params)``."""
+        if isinstance(arg1, (int, str)) and isinstance(arg2, (list, tuple)):
+            request_id, prompt, params = arg1, list(arg2), arg3 or SamplingParams()
+        elif isinstance(arg1, (list, tuple)):
+            request_id, prompt = self.req_counter, list(arg1)
+            params = arg2 if isinstance(arg2, SamplingParams) else SamplingParams()
+        else:
+            raise TypeError("Invalid arguments provided to add_request")
+        if request_id in self._by_request:
+            raise ValueError(f"request id {request_id!r} is in use")
+        vocab = self.core.model.spec.vocab_size
+        if any((not isinstance(t, int)) or t < 0 or t >= vocab for t in prompt):
+            raise ValueError(f"prompt holds a token outside the vocabulary of {vocab}")
+        seq_id = self.req_counter
+        self.req_counter += 1
+        self.scheduler.add(seq_id, prompt, params)
+        stream = params.seed if params.seed is not None else seq_id
+        self._requests[seq_id] = (request_id, params, stream)
+        self._by_request[request_id] = seq_id
+        return request_id
+
+    def abort_request(self, request_id) -> bool:
+        seq_id = self._by_request.get(request_id)
+        if seq_id is None:
+            return False
+        done = self.scheduler.abort(seq_id)
+        self._drop(seq_id)
+        return done
+
+    def _drop(self, seq_id: int) -> None:
+        request_id, _, _ = self._requests.pop(seq_id)
+        self._by_request.pop(request_id, None)
+        self.scheduler.forget(seq_id)
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    # -------------------------------------------------------------------- step
+    def step(self) -> list:
+        if not self.has_unfinished_requests():
+            return []
+        plan = self.scheduler.schedule()
+        if not plan:
+            return []  # everything running was preempted; the next step admits again
+        entries = [StepEntry(p.seq_id, self.scheduler.tokens(p.seq_id, p.start, p.count), p.start,
+                             [p.count - 1] if p.wants_logits else []) for p in plan]
+        if self.graphs is not None and self.graphs.usable(entries):
+            logits = self.graphs.step(entries)
+        else:
+            logits = self.core.step(entries)
+        sampled = []
+        wanting = [p for p in plan if p.wants_logits]
+        if wanting:
+            params = [self._requests[p.seq_id][1] for p in wanting]
+            streams = [self._requests[p.seq_id][2] for p in wanting]
+            indices = [self.scheduler.info(p.seq_id).total_len - self.scheduler.info(p.seq_id).prompt_len
+                       for p in wanting]
+            sampled = self.sampler.sample(logits, params, streams, indices)
+        self.scheduler.post_step(sampled)
+
+        outputs = []
+        for p in plan:
+            info = self.scheduler.info(p.seq_id)
+            tokens = self.scheduler.tokens(p.seq_id)
+            request_id = self._requests[p.seq_id][0]
+            outputs.append(RequestOutput(request_id, tokens[:info.prompt_len], tokens[info.prompt_len:],
+                                         info.finished, FINISH_REASON.get(info.status)))
+            if info.finished:
+                self._drop(p.seq_id)
+        return outputs
+
+    def generate(self, prompts: list, params=None) -> list:
+        """Run the prompts (lists of token ids) to the end; one RequestOutput
+        per prompt, in order.  ``params`` is one SamplingParams or one per prompt."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        ids = [self.add_request(list(p), sp) for p, sp in zip(prompts, params)]
+        done: dict = {}
+        while self.has_unfinished_requests():
+            for out in self.step():
+                if out.finished:
+                    done[out.request_id] = out
+        return [done[i] for i in ids]
+
+
+class LLM:
+    """``LLM(folder, dtype="bfloat16", num_blocks=..., ...).generate(prompts, params)``."""
+
+    def __init__(self, model: str, **engine_options):
+        self.engine = LLMEngine(model, EngineConfig(**engine_options))
+
+    def generate(self, prompts: list, params=None) -> list:
+        return self.engine.generate(prompts, params)
+
+
+def generate(model: str, prompts: list, params=None, **engine_options) -> list:
+    return LLM(model, **engine_options).generate(prompts, params)
+
+
+__all__ = ["LLMEngine", "LLM", "RequestOutput", "generate", "SamplingParams", "EngineConfig", "torch"]

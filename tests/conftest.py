@@ -32,8 +32,11 @@ TINY_B = dict(
                       original_max_position_embeddings=64),
     tie_word_embeddings=False,
 )
-TINY = {"A": (TINY_A, dict(seed=0, norm_init_std=0.0, block_size=4)),
-        "B": (TINY_B, dict(seed=2, norm_init_std=0.1, block_size=16))}
+# init_std is chosen large enough that attention is peaked: with the usual 0.02
+# every score is near 0, the softmax is flat, and a wrong key or a wrong
+# position barely moves the logits.
+TINY = {"A": (TINY_A, dict(seed=0, init_std=0.15, norm_init_std=0.0, block_size=4)),
+        "B": (TINY_B, dict(seed=2, init_std=0.1, norm_init_std=0.1, block_size=16))}
 
 
 @pytest.fixture(scope="session")
@@ -47,6 +50,7 @@ def model_folders(tmp_path_factory):
         out[name] = {}
         for dtype in ("float32", "bfloat16"):
             d = tmp_path_factory.mktemp(f"tiny{name}_{dtype}")
-            write_random_model(dict(cfg), str(d), opt["seed"], dtype, norm_init_std=opt["norm_init_std"])
+            write_random_model(dict(cfg), str(d), opt["seed"], dtype, init_std=opt["init_std"],
+                               norm_init_std=opt["norm_init_std"])
             out[name][dtype] = str(d)
     return out

@@ -1,0 +1,172 @@
+"""The whole model through the engine's step function, cache and kernels,
+against the plain implementation: whole prompts, decoding token by token,
+portions of changing size, and mixed batches with pages used again; in 32-bit
+and in bfloat16, for both tiny configurations."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, TINY
+from trace_util import Trace, compare, plain_logits, random_tokens, replay
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": {"a": 5, "b": 17, "c": 33, "d": 70}, "B": {"a": 1, "b": 9, "c": 64, "d": 130}}
+
+
+def requests_for(name, extra=None):
+    vocab = TINY[name][0]["vocab_size"]
+    lens = dict(LENGTHS[name], **(extra or {}))
+    return {rid: random_tokens(n, vocab, seed=100 + i) for i, (rid, n) in enumerate(sorted(lens.items()))}
+
+
+@pytest.fixture(scope="module")
+def plain(model_folders):
+    cache = {}
+
+    def get(name, reqs):
+        key = (name, tuple(sorted((k, tuple(v)) for k, v in reqs.items())))
+        if key not in cache:
+            cache[key] = plain_logits(model_folders[name]["float32"], reqs)
+        return cache[key]
+
+    return get
+
+
+def folder(model_folders, name, dtype):
+    # the 32-bit engine reads 32-bit files; the bfloat16 engine reads bfloat16 files,
+    # and is compared with the plain model of the same (rounded) weights
+    return model_folders[name][dtype]
+
+
+def plain_for(model_folders, name, dtype, reqs):
+    return plain_logits(model_folders[name][dtype], reqs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_each_request_alone_and_whole(model_folders, name, dtype):
+    reqs = requests_for(name)
+    want = plain_for(model_folders, name, dtype, reqs)
+    for rid, toks in reqs.items():
+        t = Trace({rid: toks})
+        t.step([(rid, len(toks))], end=[rid])
+        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"whole {rid}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_most_in_one_step_then_token_by_token(model_folders, name, dtype):
+    reqs = requests_for(name, {"e": 100})
+    want = plain_for(model_folders, name, dtype, reqs)
+    for rid, toks in reqs.items():
+        if len(toks) <= 33:
+            continue
+        t = Trace({rid: toks})
+        t.step([(rid, len(toks) - 32)], want="last")
+        for _ in range(32):
+            t.step([(rid, 1)])
+        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"decode {rid}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_portions_of_changing_size(model_folders, name, dtype):
+    reqs = requests_for(name, {"e": 100})
+    want = plain_for(model_folders, name, dtype, reqs)
+    sizes = [7, 2, 5, 3, 16, 2, 31, 4, 2, 9]
+    for rid, toks in reqs.items():
+        if len(toks) < 9:
+            continue
+        t = Trace({rid: toks})
+        left, i = len(toks), 0
+        while left:
+            n = min(sizes[i % len(sizes)], left)
+            if left - n == 1:
+                n += 1  # never leave a single token: portions go down to two
+            t.step([(rid, n)])
+            left -= n
+            i += 1
+        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"portions {rid}")
+
+
+def mixed_trace(reqs):
+    """Up to four live requests; portions of some beside single tokens of
+    others; requests end and later ones take their pages."""
+    t = Trace(reqs)
+    t.step([("d", 40), ("a", len(reqs["a"]))], end=["a"])
+    t.step([("d", 2), ("b", len(reqs["b"]) - 3), ("c", 20)])
+    t.step([("d", 1), ("b", 1), ("c", 2), ("e", 30)])
+    t.step([("b", 1), ("c", 1), ("e", 7)])                     # d sits this one out
+    t.step([("d", len(reqs["d"]) - 43), ("b", 1), ("c", len(reqs["c"]) - 23)], end=["b", "c"])
+    t.step([("e", 1), ("f", 64), ("g", 3)], end=["d"])
+    t.step([("e", 2), ("f", 1), ("g", 2), ("h", 33)])
+    for _ in range(5):
+        t.step([("e", 1), ("f", 1), ("g", 1), ("h", 1)])
+    t.step([("e", len(reqs["e"]) - 45), ("f", len(reqs["f"]) - 70), ("g", len(reqs["g"]) - 10),
+            ("h", len(reqs["h"]) - 38)], end=["e", "f", "g", "h"])
+    return t
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_batches_with_pages_used_again(model_folders, name, dtype):
+    reqs = requests_for(name, {"e": 100, "f": 90, "g": 12, "h": 50})
+    want = plain_for(model_folders, name, dtype, reqs)
+    t = mixed_trace(reqs)
+    total = sum(64 * -(-len(v) // 64) for v in reqs.values())
+    assert t.max_tokens < total, "the pool is meant to be too small for all requests at once"
+    compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, "mixed")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(model_folders, dtype):
+    name = "B"
+    reqs = {"long": random_tokens(400, TINY[name][0]["vocab_size"], seed=9)}
+    want = plain_for(model_folders, name, dtype, reqs)
+    t = Trace(reqs)
+    t.step([("long", 3)])
+    for _ in range(397):
+        t.step([("long", 1)])
+    compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, "long decode")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(model_folders, name, dtype):
+    """A one-token prompt, then single tokens: positions 0, 1, 2 have no page
+    edge and no history to hide behind."""
+    reqs = {"s": random_tokens(6, TINY[name][0]["vocab_size"], seed=11)}
+    want = plain_for(model_folders, name, dtype, reqs)
+    t = Trace(reqs)
+    for _ in range(6):
+        t.step([("s", 1)])
+    compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, "first tokens")
+
+
+def test_trace_run_program(model_folders, tmp_path):
+    """The program itself, as a user starts it: steps on stdin, a "done" line
+    per step, files of little-endian floats."""
+    name, dtype = "A", "float32"
+    reqs = requests_for(name)
+    want = plain_for(model_folders, name, dtype, reqs)
+    t = Trace(reqs)
+    t.step([("c", 20), ("a", 5)], end=["a"])
+    t.step([("c", 2)], want="none")
+    t.step([("c", 11), ("b", 17)], end=["b", "c"], want="last")
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders[name][dtype], "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(t.max_tokens)],
+        input="".join(json.dumps(s) + "\n" for s in t.steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    vocab = TINY[name][0]["vocab_size"]
+    got = {n: np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, vocab) for n in t.rows}
+    assert not (out / "1.f32").exists()
+    compare(t, got, want, dtype, "trace_run")

@@ -1,0 +1,91 @@
+"""Builds traces for the replay tests and compares what comes back with the
+plain implementation."""
+import math
+
+import numpy as np
+import torch
+
+from plain import llama_plain as P
+
+
+def random_tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+class Trace:
+    """Steps in the replay program's format, plus, for every step, which
+    (request, position) each row of its logits belongs to."""
+
+    def __init__(self, requests: dict):
+        self.requests = requests          # id -> all token ids of the request
+        self.fed = {r: 0 for r in requests}
+        self.steps = []
+        self.rows = {}                    # step number -> [(id, position)]
+        self.live = {}
+        self.max_tokens = 0
+
+    def step(self, portions: list, end=(), want="all"):
+        """portions: [(id, how many next tokens)].  want: "all", "last" or "none"."""
+        n = len(self.steps)
+        entries, rows = [], []
+        for rid, count in portions:
+            start = self.fed[rid]
+            toks = self.requests[rid][start:start + count]
+            assert len(toks) == count, f"request {rid} has no {count} tokens left"
+            w = list(range(count)) if want == "all" else ([count - 1] if want == "last" else [])
+            entries.append({"id": rid, "tokens": toks, "want": w})
+            rows += [(rid, start + i) for i in w]
+            self.fed[rid] += count
+            self.live[rid] = self.fed[rid]
+        self.max_tokens = max(self.max_tokens, sum(64 * math.ceil(v / 64) for v in self.live.values()))
+        for rid in end:
+            self.live.pop(rid, None)
+        self.steps.append({"step": n, "entries": entries, "end": list(end)})
+        if rows:
+            self.rows[n] = rows
+        return n
+
+
+def plain_logits(folder: str, requests: dict) -> dict:
+    """id -> [len, vocab] float64 logits of the whole request, no cache."""
+    w, cfg = P.read_model(folder)
+    return {rid: P.forward(w, cfg, toks) for rid, toks in requests.items()}
+
+
+def replay(folder: str, dtype: str, trace: Trace, max_tokens=None) -> dict:
+    """Run the trace through the engine in this process: step -> [rows, vocab]."""
+    from lyapunov_engine_amd.engine.replay import TraceReplayer
+
+    rp = TraceReplayer(folder, dtype, max_tokens or trace.max_tokens)
+    out = {}
+    for s in trace.steps:
+        logits = rp.run(s)
+        if logits is not None:
+            out[s["step"]] = logits
+    rp.core.cache.check()
+    assert rp.core.cache.num_requests() == len(trace.live), "ended requests must give everything back"
+    return out
+
+
+# atol is relative to the largest logit of the row.  Measured on these models:
+# about 2e-6 in 32-bit, about 3e-2 in bfloat16.
+TOL = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=6e-2, atol=6e-2)}
+
+
+def compare(trace: Trace, got: dict, want: dict, dtype: str, label=""):
+    """Every row of every step against the plain logits at its (request,
+    position); on failure name the first wrong place, which is where to look."""
+    assert set(got) == set(trace.rows), f"{label}: steps with logits {sorted(got)} != expected {sorted(trace.rows)}"
+    tol = TOL[dtype]
+    for n in sorted(trace.rows):
+        rows = trace.rows[n]
+        assert got[n].shape[0] == len(rows), f"{label}: step {n} has {got[n].shape[0]} rows, wanted {len(rows)}"
+        for i, (rid, pos) in enumerate(rows):
+            ref = want[rid][pos].numpy()
+            scale = max(1.0, float(np.abs(ref).max()))
+            err = np.abs(got[n][i].astype(np.float64) - ref)
+            bad = err > tol["atol"] * scale + tol["rtol"] * np.abs(ref)
+            assert not bad.any(), (f"{label}: first wrong logits at step {n}, request {rid!r}, position {pos}: "
+                                   f"max error {err.max():.3e} (scale {scale:.3f}); entries of the step: "
+                                   f"{[(e['id'], len(e['tokens'])) for e in trace.steps[n]['entries']]}")
