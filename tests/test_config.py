@@ -1,0 +1,130 @@
+"""Typed configuration, registry, and the structure a configuration turns into."""
+import json
+
+import pytest
+
+from conftest import TINY_A, TINY_B
+from lyapunov_engine_amd.config import (ARCHITECTURES, ConfigError, EngineConfig, LlamaConfig, MIXERS, architecture_of,
+                                        load_config)
+from lyapunov_engine_amd.models import build_model
+from lyapunov_engine_amd.models.llama import llama_spec
+
+LLAMA_1B = dict(
+    architectures=["LlamaForCausalLM"], vocab_size=128256, hidden_size=2048, intermediate_size=8192,
+    num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8, head_dim=64, max_position_embeddings=131072,
+    rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True, eos_token_id=[128001, 128008, 128009],
+    bos_token_id=128000, torch_dtype="bfloat16", hidden_act="silu", attention_bias=False, mlp_bias=False,
+    rope_scaling=dict(factor=32.0, high_freq_factor=4.0, low_freq_factor=1.0, original_max_position_embeddings=8192,
+                      rope_type="llama3"), model_type="llama", transformers_version="4.45.0")
+
+
+def test_every_size_comes_from_the_file():
+    cfg = LlamaConfig.from_dict(LLAMA_1B)
+    assert (cfg.vocab_size, cfg.hidden_size, cfg.intermediate_size, cfg.num_hidden_layers) == (128256, 2048, 8192, 16)
+    assert (cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim) == (32, 8, 64)
+    assert cfg.rope_scaling.rope_type == "llama3" and cfg.rope_scaling.factor == 32.0
+    assert cfg.rope_scaling.original_max_position_embeddings == 8192
+    assert cfg.tie_word_embeddings and cfg.eos_token_id == (128001, 128008, 128009) and cfg.bos_token_id == 128000
+    assert cfg.num_parameters() == 1_235_814_400
+    assert "transformers_version" in cfg.extra  # unknown keys are kept aside, not an error
+    # a missing size is an error, not a silent default of some model
+    for key in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
+                "max_position_embeddings", "rms_norm_eps", "rope_theta"):
+        d = dict(LLAMA_1B)
+        del d[key]
+        with pytest.raises(ConfigError, match=key):
+            LlamaConfig.from_dict(d)
+
+
+def test_conventional_fallbacks():
+    d = dict(TINY_A)
+    del d["head_dim"], d["num_key_value_heads"], d["tie_word_embeddings"], d["rope_scaling"]
+    cfg = LlamaConfig.from_dict(d)
+    assert cfg.head_dim == 64 // 4          # hidden_size // heads (reference: weight_loader.py:30-34)
+    assert cfg.num_key_value_heads == 4     # as many as query heads
+    assert cfg.tie_word_embeddings is False and cfg.rope_scaling is None
+    assert LlamaConfig.from_dict(dict(TINY_A, eos_token_id=7)).eos_token_id == (7,)
+    assert LlamaConfig.from_dict(dict(TINY_A, rope_scaling={"rope_type": "default"})).rope_scaling is None
+
+
+@pytest.mark.parametrize("bad,match", [
+    (dict(num_key_value_heads=3), "do not split"),
+    (dict(head_dim=15), "even"),
+    (dict(attention_bias=True), "bias"),
+    (dict(hidden_act="gelu"), "hidden_act"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": 2.0}), "yarn"),
+    (dict(rope_scaling={"rope_type": "llama3", "factor": 8.0}), "lacks"),
+    (dict(vocab_size=0), "positive"),
+    (dict(eos_token_id=999), "outside"),
+    (dict(rms_norm_eps=0.0), "rms_norm_eps"),
+])
+def test_what_is_not_implemented_is_refused(bad, match):
+    with pytest.raises(ConfigError, match=match):
+        LlamaConfig.from_dict(dict(TINY_A, **bad))
+
+
+def test_round_trip_through_json(tmp_path):
+    for raw in (TINY_A, TINY_B, LLAMA_1B):
+        cfg = LlamaConfig.from_dict(raw)
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        arch, again = load_config(str(tmp_path))
+        assert arch.name == "LlamaForCausalLM" and again == cfg
+
+
+def test_registry_picks_the_model_by_name():
+    assert architecture_of({"architectures": ["LlamaForCausalLM"]}) is ARCHITECTURES.get("LlamaForCausalLM")
+    assert architecture_of({"architectures": ["Nope", "LlamaForCausalLM"]}).name == "LlamaForCausalLM"
+    with pytest.raises(KeyError, match="LlamaForCausalLM"):   # the error lists what is known
+        architecture_of({"architectures": ["MixtralForCausalLM"]})
+    with pytest.raises(KeyError, match="architectures"):
+        architecture_of({})
+    assert "paged_attention" in MIXERS
+    with pytest.raises(KeyError, match="already registered"):
+        MIXERS.register("paged_attention", object)
+
+
+def test_the_two_tiny_configurations_differ_in_everything():
+    a, b = LlamaConfig.from_dict(TINY_A), LlamaConfig.from_dict(TINY_B)
+    for f in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
+              "num_key_value_heads", "head_dim", "max_position_embeddings", "rms_norm_eps", "rope_theta",
+              "rope_scaling", "tie_word_embeddings"):
+        assert getattr(a, f) != getattr(b, f), f
+    assert a.num_attention_heads // a.num_key_value_heads != b.num_attention_heads // b.num_key_value_heads
+    assert a.intermediate_size % 8 and b.vocab_size % 2  # widths that are no power of two
+
+
+def test_model_structure_follows_the_configuration():
+    for raw in (TINY_A, TINY_B):
+        cfg = LlamaConfig.from_dict(raw)
+        model = build_model(llama_spec(cfg))
+        names = model.expected_tensors()
+        H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+        q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+        assert names["model.embed_tokens.weight"][0] == (V, H)
+        assert ("lm_head.weight" in names) == (not cfg.tie_word_embeddings)
+        last = cfg.num_hidden_layers - 1
+        assert names[f"model.layers.{last}.self_attn.q_proj.weight"][0] == (q, H)
+        assert names[f"model.layers.{last}.self_attn.k_proj.weight"][0] == (kv, H)
+        assert names[f"model.layers.0.self_attn.o_proj.weight"][0] == (H, q)
+        assert names[f"model.layers.0.mlp.gate_proj.weight"][0] == (I, H)
+        assert names[f"model.layers.0.mlp.down_proj.weight"][0] == (H, I)
+        assert names["model.norm.weight"] == ((H,), "ones")
+        assert len(names) == 9 * cfg.num_hidden_layers + 2 + (0 if cfg.tie_word_embeddings else 1)
+        layout = model.cache_layout()
+        assert len(layout.groups) == 1 and layout.groups[0].buffers == tuple(range(cfg.num_hidden_layers))
+        assert layout.groups[0].spec.num_kv_heads == cfg.num_key_value_heads and not layout.states
+        assert sum(1 for _ in model.named_parts()) > 0
+        total = sum(int(__import__("math").prod(s)) for s, _ in names.values())
+        assert total == cfg.num_parameters()
+
+
+def test_engine_config_names_follow_the_reference():
+    c = EngineConfig()
+    assert (c.num_blocks, c.block_size, c.max_num_seqs, c.max_num_batched_tokens) == (1024, 16, 64, 2048)
+    assert EngineConfig(num_gpu_blocks=77).num_blocks == 77     # the alias (llm_engine.py:33)
+    import torch
+    assert EngineConfig(dtype="float32").dtype == torch.float32 and EngineConfig(dtype="bf16").dtype == torch.bfloat16
+    with pytest.raises(ValueError):
+        EngineConfig(dtype="float16")
+    with pytest.raises(ValueError):
+        EngineConfig(block_size=0)

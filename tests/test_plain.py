@@ -1,0 +1,209 @@
+"""Pins the plain implementation by what fixes it beside the reference's text:
+special cases that reduce to a library routine, invariants, and the vectors the
+reference's own tests hold.  Each is chosen so that a plausible mistake (a wrong
+sign or pairing, a norm in the wrong place, the gate in the wrong half) fails."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from plain import llama_plain as P
+
+torch.manual_seed(0)
+
+
+def test_rms_norm_formula_and_scale_invariance():
+    # oracle of the reference's test (tests/test_fused_ops.py:21-22), random gamma, eps 1e-5
+    x, w = torch.randn(7, 256, dtype=torch.float64), torch.randn(256, dtype=torch.float64)
+    want = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-5) * w
+    torch.testing.assert_close(P.rms_norm(x, w, 1e-5), want)
+    out = P.rms_norm(x, torch.ones(256, dtype=torch.float64), 1e-12)
+    torch.testing.assert_close(out.pow(2).mean(-1), torch.ones(7, dtype=torch.float64))  # unit RMS when w = 1
+    torch.testing.assert_close(P.rms_norm(3.0 * x, w, 1e-12), P.rms_norm(x, w, 1e-12))   # the scale of x drops out
+    # mean of squares, not variance: a constant row keeps its sign and size
+    c = torch.full((1, 8), 2.0, dtype=torch.float64)
+    torch.testing.assert_close(P.rms_norm(c, torch.ones(8, dtype=torch.float64), 0.0), torch.ones(1, 8, dtype=torch.float64))
+
+
+def test_swiglu_gate_is_the_first_half():
+    gu = torch.randn(5, 2 * 172, dtype=torch.float64)
+    torch.testing.assert_close(P.swiglu(gu), F.silu(gu[:, :172]) * gu[:, 172:])  # tests/test_fused_ops.py:71-72
+    g = torch.tensor([[10.0, -10.0, 1.0, 1.0]], dtype=torch.float64)  # gate (10, -10), up (1, 1)
+    out = P.swiglu(g)
+    assert out[0, 0] > 9.9 and abs(out[0, 1]) < 1e-3  # swapped halves would give silu(1) * +-10
+
+
+def test_mlp_uses_cat_gate_up():
+    # tests/test_weight_loader.py:47-56: gate_up == cat([gate, up], 0)
+    x, wg, wu, wd = torch.randn(3, 16), torch.randn(24, 16), torch.randn(24, 16), torch.randn(16, 24)
+    want = (F.silu(x @ wg.T) * (x @ wu.T)) @ wd.T
+    torch.testing.assert_close(P.mlp(x, wg, wu, wd), want)
+
+
+def test_rope_position_zero_is_identity_and_pairs_are_half_split():
+    hd = 16
+    inv = P.rope_inv_freq(hd, 10000.0)
+    assert inv[0] == 1.0 and torch.all(inv[1:] < inv[:-1])  # theta^0 first, then falling
+    x = torch.randn(2, 3, hd, dtype=torch.float64)
+    cos, sin = P.rope_cos_sin(torch.zeros(3, dtype=torch.long), inv)
+    torch.testing.assert_close(P.apply_rope(x, cos, sin), x)  # the set-up of tests/test_fused_rope.py:70-85
+    # a unit vector on dimension 0 at position 1 turns into (cos 1) e_0 + (sin 1) e_{hd/2}:
+    # an interleaved pairing would land on e_1, a wrong sign on -sin
+    e0 = torch.zeros(1, 1, hd, dtype=torch.float64)
+    e0[..., 0] = 1.0
+    cos, sin = P.rope_cos_sin(torch.tensor([1]), inv)
+    out = P.apply_rope(e0, cos, sin)[0, 0]
+    assert abs(out[0] - math.cos(1.0)) < 1e-6 and abs(out[hd // 2] - math.sin(1.0)) < 1e-6
+    assert out[1].abs() < 1e-12 and out.norm() == pytest.approx(1.0, abs=1e-6)
+
+
+def test_rope_scores_depend_on_distance_only():
+    hd = 32
+    inv = P.rope_inv_freq(hd, 500000.0)
+    q, k = torch.randn(1, 1, hd, dtype=torch.float64), torch.randn(1, 1, hd, dtype=torch.float64)
+
+    def score(m, n):
+        cq, sq = P.rope_cos_sin(torch.tensor([m]), inv)
+        ck, sk = P.rope_cos_sin(torch.tensor([n]), inv)
+        return float((P.apply_rope(q, cq, sq) * P.apply_rope(k, ck, sk)).sum())
+
+    assert score(7, 3) == pytest.approx(score(47, 43), abs=1e-4)
+    assert score(7, 3) != pytest.approx(score(7, 4), abs=1e-3)
+    # per pair the norm is kept
+    cq, sq = P.rope_cos_sin(torch.tensor([11]), inv)
+    r = P.apply_rope(q, cq, sq)[0, 0]
+    torch.testing.assert_close(r[:16] ** 2 + r[16:] ** 2, q[0, 0, :16] ** 2 + q[0, 0, 16:] ** 2, atol=1e-6, rtol=1e-6)
+
+
+def test_llama3_scaling_invariants():
+    inv = P.rope_inv_freq(64, 500000.0)
+    same = P.llama3_scale_inv_freq(inv, 1.0, 1.0, 4.0, 8192)
+    torch.testing.assert_close(same, inv)  # factor 1 changes nothing
+    out = P.llama3_scale_inv_freq(inv, 32.0, 1.0, 4.0, 8192)
+    wavelen = 2 * math.pi / inv
+    short, long_ = wavelen < 8192 / 4.0, wavelen > 8192 / 1.0
+    assert short.any() and long_.any() and (~short & ~long_).any()
+    torch.testing.assert_close(out[short], inv[short])            # short wavelengths untouched
+    torch.testing.assert_close(out[long_], inv[long_] / 32.0)     # long ones divided by the factor
+    assert torch.all(out[1:] <= out[:-1])                         # still falling with the index
+    assert torch.all(out <= inv + 1e-12) and torch.all(out >= inv / 32.0 - 1e-12)
+    # continuous at both thresholds: just inside the band equals just outside
+    for wl, want_ratio in ((8192 / 4.0, 1.0), (8192 / 1.0, 1 / 32.0)):
+        f = torch.tensor([2 * math.pi / (wl * 1.0001), 2 * math.pi / (wl * 0.9999)])
+        r = P.llama3_scale_inv_freq(f, 32.0, 1.0, 4.0, 8192) / f
+        assert r[0] == pytest.approx(want_ratio, rel=2e-3) and r[1] == pytest.approx(want_ratio, rel=2e-3)
+
+
+def test_attention_reduces_to_sdpa():
+    # the reference's oracle (tests/test_flash_attn.py:30-39): SDPA on repeat_interleaved K/V
+    nh, nkv, S, hd = 16, 4, 24, 32
+    q, k, v = (torch.randn(n, S, hd, dtype=torch.float64) for n in (nh, nkv, nkv))
+    pos = torch.arange(S)
+    got = P.attention(q, k, v, pos, pos)
+    want = F.scaled_dot_product_attention(q[None], k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None],
+                                          is_causal=True)[0]
+    torch.testing.assert_close(got, want)
+    # no mask: queries placed after every key see all of them
+    got = P.attention(q, k, v, pos + S, pos)
+    want = F.scaled_dot_product_attention(q[None], k.repeat_interleave(4, 0)[None], v.repeat_interleave(4, 0)[None])[0]
+    torch.testing.assert_close(got, want)
+    # as many key/value heads as query heads: plain multi-head attention
+    k2, v2 = torch.randn(nh, S, hd, dtype=torch.float64), torch.randn(nh, S, hd, dtype=torch.float64)
+    torch.testing.assert_close(P.attention(q, k2, v2, pos, pos),
+                               F.scaled_dot_product_attention(q[None], k2[None], v2[None], is_causal=True)[0])
+
+
+def test_attention_special_cases():
+    hd = 16
+    q, k, v = torch.randn(2, 1, hd), torch.randn(1, 1, hd), torch.randn(1, 1, hd)
+    out = P.attention(q, k, v, torch.tensor([0]), torch.tensor([0]))
+    torch.testing.assert_close(out, v.expand(2, 1, hd))  # one key: the output is its value
+    # grouped heads: query heads 0,1 read key/value head 0 and 2,3 read head 1 (h // g, not h % nkv)
+    q = torch.zeros(4, 1, hd)
+    k = torch.zeros(2, 3, hd)
+    v = torch.stack([torch.full((3, hd), 1.0), torch.full((3, hd), 2.0)])
+    out = P.attention(q, k, v, torch.tensor([2]), torch.arange(3))
+    assert out[:2].eq(1.0).all() and out[2:].eq(2.0).all()
+    # a query in the middle of a sequence sees the keys before it (absolute positions)
+    q, k, v = torch.randn(1, 2, hd), torch.randn(1, 6, hd), torch.randn(1, 6, hd)
+    part = P.attention(q, k, v, torch.tensor([4, 5]), torch.arange(6))
+    whole = P.attention(torch.cat([torch.randn(1, 4, hd), q], 1), k, v, torch.arange(6), torch.arange(6))
+    torch.testing.assert_close(part, whole[:, 4:])
+    # a window of 2: position 5 sees keys 4 and 5 only
+    w = P.attention(q[:, 1:], k, v, torch.tensor([5]), torch.arange(6), window=2)
+    torch.testing.assert_close(w, P.attention(q[:, 1:], k[:, 4:], v[:, 4:], torch.tensor([5]), torch.tensor([4, 5])))
+
+
+def tiny_weights(cfg, seed=0, std=0.1):
+    g = torch.Generator().manual_seed(seed)
+    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    w = {"model.embed_tokens.weight": torch.randn(V, H, generator=g) * std,
+         "model.norm.weight": 1 + 0.1 * torch.randn(H, generator=g)}
+    if not cfg.get("tie_word_embeddings"):
+        w["lm_head.weight"] = torch.randn(V, H, generator=g) * std
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        w[p + "input_layernorm.weight"] = 1 + 0.1 * torch.randn(H, generator=g)
+        w[p + "post_attention_layernorm.weight"] = 1 + 0.1 * torch.randn(H, generator=g)
+        for n, shape in (("self_attn.q_proj", (nh * hd, H)), ("self_attn.k_proj", (nkv * hd, H)),
+                         ("self_attn.v_proj", (nkv * hd, H)), ("self_attn.o_proj", (H, nh * hd)),
+                         ("mlp.gate_proj", (I, H)), ("mlp.up_proj", (I, H)), ("mlp.down_proj", (H, I))):
+            w[p + n + ".weight"] = torch.randn(*shape, generator=g) * std
+    return w
+
+
+CFG = dict(vocab_size=50, hidden_size=32, intermediate_size=40, num_hidden_layers=2, num_attention_heads=4,
+           num_key_value_heads=2, head_dim=8, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False)
+
+
+def test_forward_is_causal_and_a_prefix_is_enough():
+    w = tiny_weights(CFG)
+    toks = [3, 14, 15, 9, 26, 5, 35]
+    full = P.forward(w, CFG, toks)
+    torch.testing.assert_close(P.forward(w, CFG, toks[:4]), full[:4])       # later tokens do not reach back
+    changed = P.forward(w, CFG, toks[:6] + [1])
+    torch.testing.assert_close(changed[:6], full[:6])
+    assert not torch.allclose(changed[6], full[6])
+
+
+def test_forward_tied_head_equals_copied_matrix():
+    # the reference copies the embedding into lm_head when the file has none (weight_loader.py:106-109)
+    w = tiny_weights(dict(CFG, tie_word_embeddings=True))
+    tied = P.forward(w, dict(CFG, tie_word_embeddings=True), [1, 2, 3])
+    w2 = dict(w, **{"lm_head.weight": w["model.embed_tokens.weight"].clone()})
+    torch.testing.assert_close(tied, P.forward(w2, CFG, [1, 2, 3]))
+
+
+def test_forward_norm_placement_and_residuals():
+    """Zero projections out of the mixer and the feed-forward: the model is
+    embed -> final norm -> head, which pins the final norm and shows that both
+    branches only ever add to the stream."""
+    w = tiny_weights(CFG)
+    for k in w:
+        if k.endswith("o_proj.weight") or k.endswith("down_proj.weight"):
+            w[k] = torch.zeros_like(w[k])
+    toks = [7, 8, 9]
+    e = w["model.embed_tokens.weight"][torch.tensor(toks)].double()
+    want = P.rms_norm(e, w["model.norm.weight"].double(), CFG["rms_norm_eps"]) @ w["lm_head.weight"].double().T
+    torch.testing.assert_close(P.forward(w, CFG, toks), want)
+
+
+def test_sampling_follows_the_reference_rules():
+    logits = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, -3.0])
+    assert P.greedy(logits) == 0
+    p = P.sample_filter(logits, 0.7, top_k=1, top_p=1.0)
+    assert p[0] == 1.0                                             # top-k 1 is greedy
+    p = P.sample_filter(logits, 1.0, top_k=3, top_p=1.0)
+    assert (p[:3] > 0).all() and (p[3:] == 0).all()
+    torch.testing.assert_close(p[:3], torch.softmax(logits[:3].double(), 0))
+    # top-p: probabilities 0.574 0.211 0.128 ...; p = 0.6 keeps the token that crosses 0.6 (the second)
+    p = P.sample_filter(logits, 1.0, top_k=-1, top_p=0.6)
+    assert (p[:2] > 0).all() and (p[2:] == 0).all()
+    p = P.sample_filter(logits, 1.0, top_k=-1, top_p=0.0)
+    assert p[0] == 1.0                                             # the first is never removed
+    cold = P.sample_filter(logits, 0.01, -1, 1.0)
+    assert cold[0] > 0.999                                         # T -> 0 tends to the argmax
+    probs = torch.tensor([0.1, 0.2, 0.3, 0.4])
+    assert [P.inverse_cdf(probs, u) for u in (0.0, 0.05, 0.1, 0.29, 0.3, 0.95, 0.9999)] == [0, 0, 1, 1, 2, 3, 3]
