@@ -122,9 +122,10 @@ class DecodeGraphs:
         self.max_batch = _bucket(max_batch, 1)
         self.captured: dict = {}
         self.pool = None
+        self.safe = all(part.graph_safe for _, part in runner.model.named_parts())
 
     def usable(self, entries: list) -> bool:
-        return all(len(e.tokens) == 1 and e.want == [0] for e in entries) and len(entries) <= self.max_batch
+        return self.safe and all(len(e.tokens) == 1 and e.want == [0] for e in entries) and len(entries) <= self.max_batch
 
     def step(self, entries: list) -> torch.Tensor:
         """Logits [len(entries), vocab]; valid until the next graph step."""

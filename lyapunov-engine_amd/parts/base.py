@@ -51,6 +51,11 @@ class WeightSpec:
 class Part:
     """Anything that may own weights and sub-parts."""
 
+    # False for a part whose forward reads the host copies of the step's tables
+    # (``ctx.q_start_host`` and the like): such a forward cannot be captured in
+    # a graph and replayed with other tables, so its model steps eagerly.
+    graph_safe = True
+
     def weight_specs(self) -> list:
         return []
 

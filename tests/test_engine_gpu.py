@@ -1,0 +1,152 @@
+"""Generation through the entry points: the scheduler, the step function, the
+sampler and the graphs together, against greedy decoding with the plain model."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from conftest import ROOT, TINY
+from plain import llama_plain as P
+from trace_util import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_greedy(folder, prompt, n):
+    w, cfg = P.read_model(folder)
+    toks, margins = list(prompt), []
+    for _ in range(n):
+        logits = P.forward(w, cfg, toks)[-1]
+        top = torch.topk(logits, 2).values
+        margins.append(float(top[0] - top[1]))
+        toks.append(P.greedy(logits))
+    return toks[len(prompt):], margins
+
+
+def check_against_plain(folder, prompt, got, dtype):
+    """In 32-bit the tokens are the plain model's.  In bfloat16 a token may
+    differ only where the plain model's best two logits are closer than what
+    bfloat16 resolves; the comparison then stops (the continuations differ)."""
+    want, margins = plain_greedy(folder, prompt, len(got))
+    for i, (g, w_) in enumerate(zip(got, want)):
+        if g != w_:
+            assert dtype == "bfloat16" and margins[i] < 0.25, f"token {i}: engine {g}, plain {w_}, margin {margins[i]}"
+            return
+    assert len(got) == len(want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(model_folders, name, dtype):
+    import lyapunov_engine_amd as L
+
+    folder = model_folders[name][dtype]
+    vocab = TINY[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, seed=50 + n) for n in (5, 17, 33)]
+    llm = L.LLM(folder, dtype=dtype, num_blocks=64, block_size=TINY[name][1]["block_size"])
+    outs = llm.generate(prompts, L.SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    assert [o.request_id for o in outs] == [0, 1, 2]
+    for prompt, o in zip(prompts, outs):
+        assert o.finished and o.finish_reason == "length" and o.prompt_tokens == prompt and len(o.output_tokens) == 16
+        check_against_plain(folder, prompt, o.output_tokens, dtype)
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+def test_portions_preemption_and_graphs_do_not_change_the_tokens(model_folders, graphs):
+    """A token budget smaller than the prompts, and so few pages that requests
+    are preempted and recomputed: greedy tokens stay those of the plain model."""
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    folder = model_folders["A"]["float32"]
+    prompts = [random_tokens(n, 256, seed=70 + n) for n in (30, 9, 21, 40)]
+    engine = LLMEngine(folder, EngineConfig(dtype="float32", num_blocks=30, block_size=4, max_num_seqs=4,
+                                            max_num_batched_tokens=16, enable_graphs=graphs))
+    for i, p in enumerate(prompts):
+        engine.add_request(f"r{i}", p, SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True))
+    done, steps = {}, 0
+    while engine.has_unfinished_requests():
+        for out in engine.step():
+            if out.finished:
+                done[out.request_id] = out
+        steps += 1
+        engine.core.cache.check()
+        assert steps < 2000
+    assert engine.scheduler.counters()["preemptions"] > 0, "the pool was meant to be too small"
+    assert engine.core.cache.num_requests() == 0 and engine.core.cache.num_free_pages() == 30
+    for i, p in enumerate(prompts):
+        check_against_plain(folder, p, done[f"r{i}"].output_tokens, "float32")
+
+
+def test_graph_steps_equal_eager_steps(model_folders):
+    """The same decode steps through a captured graph, replayed several times
+    with other work in between, and eagerly: equal logits every time."""
+    from lyapunov_engine_amd.engine.core import EngineCore, StepEntry
+    from lyapunov_engine_amd.engine.graphs import DecodeGraphs
+
+    core = EngineCore.from_folder(model_folders["B"]["bfloat16"], dtype="bfloat16", num_blocks=64, block_size=16)
+    graphs = DecodeGraphs(core.runner, max_batch=8)
+    seqs = {i: random_tokens(n, 515, seed=i) for i, n in enumerate((40, 3, 17))}
+    for i, toks in seqs.items():
+        core.cache.add(i)
+        core.cache.extend(i, len(toks) + 8)
+        core.step([StepEntry(i, toks, 0, [])])
+        core.cache.commit(i, len(toks))
+    for k in range(6):
+        entries = [StepEntry(i, [(7 * k + i) % 515], len(seqs[i]) + k, [0]) for i in seqs]
+        eager = core.step(entries).clone()              # writes the same slots the graph is about to write
+        assert graphs.usable(entries)
+        torch.cuda.synchronize()
+        replayed = graphs.step(entries).clone()
+        torch.testing.assert_close(replayed, eager, rtol=0, atol=0)
+        for e in entries:
+            core.cache.commit(e.seq_id, e.start + 1)
+    assert len(graphs.captured) == 1
+
+
+def test_seeded_sampling_does_not_depend_on_batch_mates(model_folders):
+    import lyapunov_engine_amd as L
+
+    folder = model_folders["B"]["float32"]
+    prompt = random_tokens(9, 515, seed=1)
+    sp = L.SamplingParams(temperature=0.8, top_k=50, top_p=0.95, max_tokens=24, ignore_eos=True, seed=1234)
+    alone = L.LLM(folder, dtype="float32", num_blocks=64).generate([prompt], sp)[0].output_tokens
+    others = [random_tokens(n, 515, seed=n) for n in (1, 64, 130)]
+    sps = [L.SamplingParams(temperature=0.8, max_tokens=24, ignore_eos=True, seed=s) for s in (1, 2, 3)]
+    mixed = L.LLM(folder, dtype="float32", num_blocks=64, max_num_batched_tokens=48).generate(
+        others[:2] + [prompt] + others[2:], sps[:2] + [sp] + sps[2:])
+    assert mixed[2].output_tokens == alone
+    other_seed = L.SamplingParams(temperature=0.8, top_k=50, top_p=0.95, max_tokens=24, ignore_eos=True, seed=99)
+    assert L.LLM(folder, dtype="float32", num_blocks=64).generate([prompt], other_seed)[0].output_tokens != alone
+    assert len(set(alone)) > 4  # it does sample: greedy on this model repeats itself quickly
+
+
+def test_eos_stops_a_request(model_folders):
+    import lyapunov_engine_amd as L
+
+    folder = model_folders["A"]["float32"]
+    prompt = random_tokens(12, 256, seed=3)
+    want, _ = plain_greedy(folder, prompt, 10)
+    stop_at = 4
+    llm = L.LLM(folder, dtype="float32", num_blocks=32, block_size=4, eos_token_ids=(want[stop_at],))
+    out = llm.generate([prompt], L.SamplingParams(temperature=0.0, max_tokens=10))[0]
+    first = want.index(want[stop_at])
+    assert out.output_tokens == want[: first + 1] and out.finish_reason == "stop"
+    out = llm.generate([prompt], L.SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))[0]
+    assert out.output_tokens == want and out.finish_reason == "length"
+
+
+def test_command_line_generate(model_folders):
+    folder = model_folders["A"]["float32"]
+    prompt = random_tokens(7, 256, seed=8)
+    want, _ = plain_greedy(folder, prompt, 8)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "lyapunov"), "generate", "--model", folder,
+                           "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "8", "--temperature", "0",
+                           "--dtype", "float32", "--block-size", "4", "--num-blocks", "32"],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "--- Output Generation ---" in proc.stdout
+    assert proc.stdout.strip().splitlines()[-1].split() == [str(t) for t in want]
