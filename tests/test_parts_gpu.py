@@ -1,0 +1,289 @@
+"""Each part of a layer alone against its plain formula, and the generality of
+the frame: a toy architecture, defined here and registered from here, with a
+mixer that keeps state of its own, a windowed attention layer with pages of its
+own, a layer that runs twice and a layer that reads another call's cache.  No
+file of the package knows any of it."""
+import json
+import os
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+from plain import llama_plain as P
+from trace_util import Trace, random_tokens, replay
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ------------------------------------------------------------ parts on their own
+def one_layer_core(dtype, block_size=4, **over):
+    """A one-layer Llama (for its cache layout and context) with random weights."""
+    from lyapunov_engine_amd.config import LlamaConfig
+    from lyapunov_engine_amd.engine.core import EngineCore
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.models.llama import llama_spec
+    from lyapunov_engine_amd.weights import DictSource, load_weights, random_tensors
+
+    raw = dict(architectures=["LlamaForCausalLM"], vocab_size=100, hidden_size=80, intermediate_size=130,
+               num_hidden_layers=1, num_attention_heads=5, num_key_value_heads=5, head_dim=16,
+               max_position_embeddings=128, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
+    raw.update(over)
+    cfg = LlamaConfig.from_dict(raw)
+    model = build_model(llama_spec(cfg))
+    tensors = dict(random_tensors(model, 5, torch.float32, init_std=0.2, norm_init_std=0.2))
+    tdtype = torch.float32 if dtype == "float32" else torch.bfloat16
+    tensors = {k: v.to(tdtype) for k, v in tensors.items()}
+    load_weights(model, DictSource(tensors), tdtype, DEV)
+    core = EngineCore(model, cfg, dtype=dtype, device=DEV, num_blocks=64, block_size=block_size, num_state_slots=4)
+    return core, raw, {k: v.float() for k, v in tensors.items()}
+
+
+def check(got, want, dtype, what):
+    """Error against the size of the result: 32-bit to 2e-5 of the largest
+    value, bfloat16 (8 bits of mantissa, several roundings in a row) to 4e-2."""
+    scale = float(want.abs().max())
+    err = float((got.double() - want).abs().max())
+    limit = (2e-5 if dtype == "float32" else 4e-2) * scale
+    assert err <= limit, f"{what}: error {err:.3e} exceeds {limit:.3e} (largest value {scale:.3f})"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixer_ffn_norm_and_block_alone(dtype):
+    from lyapunov_engine_amd.engine.core import StepEntry
+
+    core, raw, w = one_layer_core(dtype)
+    layer = core.model.layers[0]
+    H = raw["hidden_size"]
+    # two requests: a whole prompt of 11 and a second portion (positions 6..9) of another
+    core.cache.add(0), core.cache.add(1)
+    core.cache.extend(0, 11), core.cache.extend(1, 10)
+    x_prev = torch.randn(6, H, generator=torch.Generator().manual_seed(1))
+    x_new = torch.randn(11 + 4, H, generator=torch.Generator().manual_seed(2))
+    tdtype = core.dtype
+    # first the other request's first six tokens, through the mixer alone, to fill its pages
+    ctx = core.runner.build_context([StepEntry(1, [0] * 6, 0, [])])
+    caches = core.runner.layer_caches(ctx)
+    layer.mixer.forward(ctx, x_prev.to(DEV, tdtype), caches[0])
+    core.cache.commit(1, 6)
+    ctx = core.runner.build_context([StepEntry(0, [0] * 11, 0, []), StepEntry(1, [0] * 4, 6, [])])
+    caches = core.runner.layer_caches(ctx)
+    xs = x_new.to(DEV, tdtype)
+    inv = P.model_inv_freq(raw)
+    p = "model.layers.0."
+
+    got = layer.mixer.forward(ctx, xs, caches[0]).float().cpu()
+    xa = xs[:11].float().cpu().double()
+    xb = torch.cat([x_prev.to(tdtype).float(), xs[11:].float().cpu()]).double()
+    wd = {k: v.double() for k, v in w.items()}
+    want_a = P.attention_layer(xa, torch.arange(11), wd, p + "self_attn.", raw, inv)
+    want_b = P.attention_layer(xb, torch.arange(10), wd, p + "self_attn.", raw, inv)[6:]
+    check(got, torch.cat([want_a, want_b]), dtype, "mixer")
+
+    got = layer.ffn.forward(ctx, xs).float().cpu()
+    want = P.mlp(xs.float().cpu().double(), wd[p + "mlp.gate_proj.weight"], wd[p + "mlp.up_proj.weight"],
+                 wd[p + "mlp.down_proj.weight"])
+    check(got, want, dtype, "feed-forward")
+
+    h = torch.randn(15, H, generator=torch.Generator().manual_seed(3)).to(DEV)
+    delta = torch.randn(15, H, generator=torch.Generator().manual_seed(4)).to(DEV, tdtype)
+    h0 = h.clone()
+    got = layer.norm1.forward(ctx, h, delta).float().cpu()
+    total = h0.cpu().double() + delta.float().cpu().double()
+    torch.testing.assert_close(h.cpu().double(), total, rtol=1e-6, atol=1e-6)
+    check(got, P.rms_norm(total, wd[p + "input_layernorm.weight"], raw["rms_norm_eps"]), dtype, "norm")
+
+    # the block as a whole, on request 0 alone (fresh pages), against the plain decoder layer
+    core.cache.free(0), core.cache.free(1)
+    core.cache.add(2)
+    core.cache.extend(2, 11)
+    ctx = core.runner.build_context([StepEntry(2, [0] * 11, 0, [])])
+    caches = core.runner.layer_caches(ctx)
+    h = x_new[:11].to(DEV).clone()
+    h2, pending = layer.forward(ctx, h, None, caches[0])
+    got = h2.cpu().double() + pending.float().cpu().double()
+    want = P.decoder_layer(x_new[:11].double(), torch.arange(11), wd, 0, raw, inv)
+    check(got, want, dtype, "block")
+
+
+def test_rotary_table_matches_the_plain_angles():
+    from lyapunov_engine_amd.parts.rope import RotaryEncoding, rotary_inv_freq
+
+    for scaling in (None, dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                               original_max_position_embeddings=64)):
+        enc = RotaryEncoding(32, 500000.0, 300, scaling)
+        enc.materialize(DEV, torch.float32)
+        inv = P.rope_inv_freq(32, 500000.0)
+        if scaling:
+            inv = P.llama3_scale_inv_freq(inv, 8.0, 1.0, 4.0, 64)
+        torch.testing.assert_close(rotary_inv_freq(32, 500000.0, scaling), inv, rtol=1e-6, atol=0)
+        cos, sin = P.rope_cos_sin(torch.arange(300), inv)
+        table = enc.table.cpu()
+        assert table.shape == (300, 32)  # cosines then sines (reference: tests/test_fused_rope.py:13-24)
+        torch.testing.assert_close(table[:, :16], cos[:, :16], rtol=0, atol=3e-5)
+        torch.testing.assert_close(table[:, 16:], sin[:, :16], rtol=0, atol=3e-5)
+
+
+# ------------------------------------------------------------- a toy architecture
+TOY = dict(architectures=["ToyMixForCausalLM"], vocab_size=120, hidden_size=48, intermediate_size=72, state_size=24,
+           num_heads=3, num_kv_heads=1, head_dim=16, window=6, max_position=96, eps=1e-5, theta=10000.0, decay=0.8)
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    raw: tuple
+    architectures: tuple = ("ToyMixForCausalLM",)
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(tuple(sorted((k, v) for k, v in d.items() if k != "architectures" and k != "torch_dtype")))
+
+    def to_dict(self):
+        return dict(self.raw, architectures=list(self.architectures))
+
+
+def register_toy():
+    """Everything the toy needs, through the package's public registries."""
+    from lyapunov_engine_amd.config import MIXERS, LayerCall, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from lyapunov_engine_amd.parts import Mixer, StateSpec, WeightSource, WeightSpec
+
+    class LinearRecurrence(Mixer):
+        """s_t = decay * s_{t-1} + W_in x_t ;  y_t = W_out s_t.  The state s is
+        all it keeps of a request: no pages."""
+
+        graph_safe = False  # walks the host copy of the batch layout
+
+        def __init__(self, hidden_size, state_size, decay):
+            self.hidden_size, self.state_size, self.decay = hidden_size, state_size, decay
+            self.in_proj = self.out_proj = None
+
+        def weight_specs(self):
+            return [WeightSpec("in_proj", (WeightSource("in_proj.weight", (self.state_size, self.hidden_size)),)),
+                    WeightSpec("out_proj", (WeightSource("out_proj.weight", (self.hidden_size, self.state_size)),))]
+
+        def state_spec(self):
+            return StateSpec((self.state_size,), torch.float32)
+
+        def forward(self, ctx, x, cache):
+            u = x.float() @ self.in_proj.float().T
+            out = torch.empty_like(u)
+            for b in range(ctx.B):
+                lo, hi = ctx.q_start_host[b], ctx.q_start_host[b + 1]
+                slot = ctx.state_slots_host[b]
+                first = ctx.ctx_len_host[b] - (hi - lo) == 0   # a new request starts from nothing
+                s = torch.zeros(self.state_size, device=x.device) if first else cache.state[slot].clone()
+                for t in range(lo, hi):
+                    s = self.decay * s + u[t]
+                    out[t] = s
+                cache.state[slot] = s
+            return (out @ self.out_proj.float().T).to(ctx.dtype)
+
+    MIXERS.register("toy_linear_recurrence", LinearRecurrence, replace=True)
+
+    def to_spec(cfg: ToyConfig) -> ModelSpec:
+        c = dict(cfg.raw)
+        H = c["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": c["eps"]})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
+        rope = PartSpec("rope", {"dim": c["head_dim"], "theta": c["theta"], "max_position": c["max_position"]})
+        attn = dict(hidden_size=H, num_heads=c["num_heads"], num_kv_heads=c["num_kv_heads"], head_dim=c["head_dim"])
+        full = PartSpec("paged_attention", dict(attn, position=rope))
+        windowed = PartSpec("paged_attention", dict(attn, position=None, window=c["window"]))   # no rotation either
+        borrower = PartSpec("paged_attention", dict(attn, position=rope, own_kv=False))
+        recur = PartSpec("toy_linear_recurrence", {"hidden_size": H, "state_size": c["state_size"],
+                                                   "decay": c["decay"]})
+        layers = tuple(LayerSpec("prenorm", m, ffn, norm, norm) for m in (full, recur, windowed, borrower))
+        # layer 0 runs twice (caches 0 and 3); layer 3 reads what the first call of layer 0 stored
+        schedule = (LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2), LayerCall(0, 3), LayerCall(3, 0, writes=False))
+        return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=schedule,
+                         final_norm=norm, tie_word_embeddings=False, max_position=c["max_position"])
+
+    register_architecture("ToyMixForCausalLM", ToyConfig, to_spec, replace=True)
+
+
+def toy_plain(folder, tokens):
+    """The toy model, whole sequence, from plain parts."""
+    from safetensors.torch import load_file
+
+    c = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    S = len(tokens)
+    pos = torch.arange(S)
+    nh, nkv, hd = c["num_heads"], c["num_kv_heads"], c["head_dim"]
+    inv = P.rope_inv_freq(hd, c["theta"])
+    cos, sin = P.rope_cos_sin(pos, inv)
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    stored = {}
+
+    def heads(t, n):
+        return t.view(S, n, hd).transpose(0, 1)
+
+    for layer, cache, writes in ((0, 0, True), (1, 1, True), (2, 2, True), (0, 3, True), (3, 0, False)):
+        p = f"model.layers.{layer}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
+        if layer == 1:
+            u = x @ w[p + "self_attn.in_proj.weight"].T
+            s, out = torch.zeros(c["state_size"], dtype=torch.float64), []
+            for t in range(S):
+                s = c["decay"] * s + u[t]
+                out.append(s)
+            a = torch.stack(out) @ w[p + "self_attn.out_proj.weight"].T
+        else:
+            rotate = layer != 2
+            q = heads(x @ w[p + "self_attn.q_proj.weight"].T, nh)
+            q = P.apply_rope(q, cos, sin) if rotate else q
+            if writes:
+                k = heads(x @ w[p + "self_attn.k_proj.weight"].T, nkv)
+                k = P.apply_rope(k, cos, sin) if rotate else k
+                stored[cache] = (k, heads(x @ w[p + "self_attn.v_proj.weight"].T, nkv))
+            k, v = stored[cache]
+            o = P.attention(q, k, v, pos, pos, window=c["window"] if layer == 2 else 0)
+            a = o.transpose(0, 1).reshape(S, nh * hd) @ w[p + "self_attn.o_proj.weight"].T
+        h = h + a
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
+        h = h + P.mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["lm_head.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
+    from lyapunov_engine_amd.config import ARCHITECTURES, MIXERS
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.weights import write_random_model
+
+    register_toy()
+    try:
+        folder = str(tmp_path / "toy")
+        write_random_model(dict(TOY), folder, seed=1, dtype=dtype, init_std=0.15, norm_init_std=0.1)
+        arch = ARCHITECTURES.get("ToyMixForCausalLM")
+        model = build_model(arch.to_spec(arch.config_class.from_dict(TOY)))
+        layout = model.cache_layout()
+        assert len(layout.groups) == 2                       # all keys, and a window of them: pages of their own
+        assert layout.groups[0].buffers == (0, 3) and layout.groups[1].buffers == (2,)
+        assert layout.groups[1].spec.window == 6 and list(layout.states) == [1]
+        names = model.expected_tensors()
+        assert "model.layers.1.self_attn.in_proj.weight" in names
+        assert "model.layers.3.self_attn.k_proj.weight" not in names   # the borrower has no keys of its own
+
+        reqs = {"x": random_tokens(60, 120, seed=2), "y": random_tokens(23, 120, seed=3),
+                "z": random_tokens(41, 120, seed=4)}
+        want = {k: toy_plain(folder, v) for k, v in reqs.items()}
+        from trace_util import compare
+
+        whole = Trace(reqs)
+        for rid in reqs:
+            whole.step([(rid, len(reqs[rid]))], end=[rid])
+        compare(whole, replay(folder, dtype, whole), want, dtype, "toy whole")
+
+        cut = Trace(reqs)
+        cut.step([("x", 7), ("y", 23)], end=["y"])
+        cut.step([("x", 2), ("z", 30)])
+        for _ in range(9):
+            cut.step([("x", 1), ("z", 1)])
+        cut.step([("x", 42), ("z", 2)], end=["x", "z"])
+        compare(cut, replay(folder, dtype, cut), want, dtype, "toy cut")
+    finally:
+        ARCHITECTURES.unregister("ToyMixForCausalLM")
+        MIXERS.unregister("toy_linear_recurrence")
