@@ -1,0 +1,204 @@
+"""Serving benchmark on one MI355X: decode tokens a second of the Llama 3.2 1B
+shape with random weights (BASELINE.json configs[2]), plus prefill speed and the
+decode step's share of the memory roofline.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A "step" is one decode step of the engine (schedule, model step, sampling,
+bookkeeping) with every request bringing one token.  One JSON line is printed.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # bytes/s, MI355X
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+MODEL = dict(  # BASELINE.json configs[2]: Llama 3.2 1B shape
+    architectures=["LlamaForCausalLM"], vocab_size=128256, hidden_size=2048, intermediate_size=8192,
+    num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8, head_dim=64, max_position_embeddings=8192,
+    rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192))
+FULL_LAYERS = MODEL["num_hidden_layers"]
+
+
+def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget):
+    import torch
+
+    from lyapunov_engine_amd.config import EngineConfig, LlamaConfig
+    from lyapunov_engine_amd.engine.core import EngineCore
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.models.llama import llama_spec
+    from lyapunov_engine_amd.weights import DictSource, load_weights, random_tensors
+
+    cfg = LlamaConfig.from_dict(dict(MODEL, num_hidden_layers=layers))
+    model = build_model(llama_spec(cfg))
+    tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tensors = dict(random_tensors(model, 4, tdtype, device="cuda:0"))   # seed 4, N(0, 0.02)
+    load_weights(model, DictSource(tensors), tdtype, "cuda:0")
+    del tensors
+    core = EngineCore(model, cfg, dtype=tdtype, device="cuda:0", num_blocks=num_blocks, block_size=block_size,
+                      num_state_slots=max_num_seqs)
+    engine = LLMEngine(core, EngineConfig(dtype=tdtype, num_blocks=num_blocks, block_size=block_size,
+                                          max_num_seqs=max_num_seqs, max_num_batched_tokens=budget,
+                                          max_model_len=cfg.max_position_embeddings))
+    return engine, cfg
+
+
+def weight_bytes(cfg, esz):
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    per_layer = (q + 2 * kv) * h + h * q + 3 * i * h + 2 * h
+    return (cfg.num_hidden_layers * per_layer + cfg.vocab_size * h + h) * esz   # the head matrix once per step
+
+
+def kv_bytes_per_token(cfg, esz):
+    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * esz
+
+
+def prefill_flops(cfg, T):
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    linear = 2 * T * ((q + 2 * kv) * h + h * q + 3 * i * h)
+    attn = 2 * cfg.num_attention_heads * cfg.head_dim * T * T       # causal: half of 4 nh hd T^2
+    return cfg.num_hidden_layers * (linear + attn) + 2 * cfg.vocab_size * h   # logits of the last token
+
+
+def random_prompt(n, vocab, seed):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def measure_decode(engine, cfg, batch, context, steps, warmup, seed):
+    """`batch` requests are brought to just under `context` tokens, then warmup +
+    steps decode steps run with all of them decoding together.  Requests that
+    finish their prompt first decode while the others are still in their prompt,
+    so the prompts are shortened by the number of steps that takes.  Returns
+    (seconds per step, mean context length over the timed steps)."""
+    import torch
+
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    budget = engine.config.max_num_batched_tokens
+    ctx_start = context - (warmup + steps) - 4
+    ctx_start -= batch * (-(-ctx_start // budget)) + batch      # steps the prompts take, at worst
+    assert ctx_start > 0
+    sp = SamplingParams(temperature=0.0, max_tokens=context, ignore_eos=True)
+    names = [f"d{seed}-{b}" for b in range(batch)]
+    for b, name in enumerate(names):
+        engine.add_request(name, random_prompt(ctx_start, cfg.vocab_size, seed * 1000 + b), sp)
+    seqs = [engine._by_request[n] for n in names]
+    while engine.scheduler.num_waiting() or any(
+            engine.scheduler.info(s).num_computed < engine.scheduler.info(s).prompt_len for s in seqs):
+        engine.step()                       # prompt portions until every request is decoding
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    ctx0 = sum(engine.scheduler.info(s).total_len for s in seqs) / batch
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    assert len(out) == batch and not any(o.finished for o in out), "every request must decode in every timed step"
+    ctx1 = sum(engine.scheduler.info(s).total_len for s in seqs) / batch
+    assert ctx1 - ctx0 == steps and ctx1 <= context
+    for name in names:
+        engine.abort_request(name)
+    return dt, (ctx0 + ctx1 - 1) / 2.0
+
+
+def measure_prefill(engine, cfg, tokens, repeats=5):
+    import torch
+
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    times = []
+    for r in range(repeats + 2):
+        engine.add_request(f"p{r}", random_prompt(tokens, cfg.vocab_size, 5 + r),
+                           SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = engine.step()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        assert out and out[0].finished
+    times = sorted(times[2:])
+    return times[len(times) // 2]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=8192, help="context length the decode steps run at")
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    esz = 2 if args.dtype == "bf16" else 4
+    block_size = 16
+    max_batch = 64
+    num_blocks = max_batch * (args.context // block_size + 1) + 64
+    engine, cfg = build_engine(args.layers, args.dtype, num_blocks, max_batch, block_size, budget=8192)
+
+    prefill_s = measure_prefill(engine, cfg, 2048)
+    step_s, mean_ctx = measure_decode(engine, cfg, args.batch, args.context, args.steps, args.warmup, seed=1)
+    value = args.batch / step_s
+    step_bytes = weight_bytes(cfg, esz) + args.batch * mean_ctx * kv_bytes_per_token(cfg, esz)
+    achieved = step_bytes / step_s
+
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            s, _ = measure_decode(engine, cfg, b, args.context, min(args.steps, 64), min(args.warmup, 8), seed=10 + b)
+            points[f"decode_b{b}"] = round(b / s, 1)
+        # the decode workload as configs[2] words it: 2048-token prompts, 256 steps -> contexts up to 2304
+        for b in (1, 8, 64):
+            s, _ = measure_decode(engine, cfg, b, 2304, min(args.steps, 64), min(args.warmup, 8), seed=20 + b)
+            points[f"decode_b{b}_ctx2048"] = round(b / s, 1)
+
+    peak = MFMA_PEAK[args.dtype]
+    line = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2048 tokens; % of roofline",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (random weights seed 4, random token ids)",
+        "config": {
+            "model": "llama-3.2-1b-shape", "num_hidden_layers": cfg.num_hidden_layers, "full_layers": FULL_LAYERS,
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": True,
+            "rope_scaling": "llama3 factor 32", "global_batch": args.batch, "seq_len": int(round(mean_ctx)),
+            "context_len": args.context, "kv_block_size": block_size, "prefill_tokens": 2048,
+            "parallelism": "single-gpu", "graphs": True,
+        },
+        "prefill": {"value": round(2048 / prefill_s, 1), "tokens": 2048, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(prefill_flops(cfg, 2048) / prefill_s / peak, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -110,6 +110,30 @@ struct Mma16<bf16_t> {
   }
 };
 
+// A 16x16 output tile fed with 16-byte fragments: bfloat16 takes eight values
+// per lane and one 16x16x32 instruction, float four values and four 16x16x4
+// instructions.  Lane l holds row/column l % 16 and kElems consecutive
+// inner-dimension values of group l / 16; the accumulator is laid out as in
+// Mma16.
+template <typename T>
+struct Mma16Wide;
+
+template <>
+struct Mma16Wide<float> {
+  static constexpr int kElems = 4;
+  using Frag = f32x4;
+  static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) { return Mma16<float>::mma(a, b, c); }
+};
+
+template <>
+struct Mma16Wide<bf16_t> {
+  static constexpr int kElems = 8;
+  using Frag = bf16x8;
+  static __device__ __forceinline__ f32x4 mma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
 // A 32x32 output tile.  Lane l holds row/column l % 32 and kElems consecutive
 // inner-dimension values of group l / 32; one call covers 2 * kElems values.
 // Accumulator register v of lane l is row 8 * (v / 4) + 4 * (l / 32) + v % 4,

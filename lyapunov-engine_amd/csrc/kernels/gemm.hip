@@ -6,10 +6,12 @@
 // The reference has no kernel of its own here: its projections are nn.Linear
 // calls (python/lyapunov_engine/models/llama.py:45-48, 112-117, 177).
 //
-// The inner dimension is walked in the same order for every row whatever M is,
-// and there is no split over it, so a token's result does not depend on what
-// else is in the batch.  Any M, N, K is accepted; rows that are not 16-byte
-// aligned take a scalar load path.
+// Two kernels: a tiled one for any M, N, K (rows that are not 16-byte aligned
+// take a scalar load path), and one for M <= 64 that streams the weights once.
+// In both the order of the additions for an output element is fixed by the
+// sizes of the product alone (no atomics), so a token's result does not depend
+// on which other tokens are in the batch beyond the choice of kernel, which
+// follows M.
 #include "common.h"
 
 namespace lyp {
@@ -130,6 +132,103 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
     }
 }
 
+// ---------------------------------------------------------------- few rows
+// M <= 64 (decode steps): the weight matrix is read once from memory and the
+// time is what that read takes, so the shape is chosen for memory parallelism.
+// A workgroup owns 16 rows of W (16 output features); its waves split the inner
+// dimension between them and add their parts through LDS, in a fixed order.  A
+// wave keeps the 16 x (16 MB) output tile in registers: W rows are the row
+// operand, tokens the columns.  Per 64 values of the inner dimension a lane
+// reads one contiguous run of 16 values of its row; activations come through
+// the cache, they are small.  Needs K % 64 == 0 and 16-byte aligned rows.
+template <typename T, int MB, bool F32OUT>
+__global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
+                                                           void* __restrict__ Cv, int M, int N, int K, int lda,
+                                                           int ldw, int ldc) {
+  using MM = Mma16Wide<T>;
+  using Frag = typename MM::Frag;
+  constexpr int NF = 16 / MM::kElems;  // fragments per lane per 64 values of K
+  extern __shared__ float red[];       // [waves][MB][64][4]
+
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int nwaves = blockDim.x / kWave;
+  const int n0 = blockIdx.x * 16;
+  const int r = lane % 16, j = lane / 16;
+  const int wrow = min(n0 + r, N - 1);  // rows past the end read the last row and are not stored
+
+  const int chunks = K / 64;
+  const int per_wave = (chunks + nwaves - 1) / nwaves;
+  const int c_begin = min(chunks, wave * per_wave), c_end = min(chunks, c_begin + per_wave);
+
+  f32x4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const T* wp = W + static_cast<size_t>(wrow) * ldw + j * 16;
+  const T* ap[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * 16;
+
+#pragma unroll 2
+  for (int c = c_begin; c < c_end; ++c) {
+    const int k0 = c * 64;
+    Frag wf[NF];
+#pragma unroll
+    for (int f = 0; f < NF; ++f) wf[f] = *reinterpret_cast<const Frag*>(wp + k0 + f * MM::kElems);
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      Frag xf[NF];
+#pragma unroll
+      for (int f = 0; f < NF; ++f) xf[f] = *reinterpret_cast<const Frag*>(ap[b] + k0 + f * MM::kElems);
+#pragma unroll
+      for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[f], xf[f], acc[b]);
+    }
+  }
+
+  // acc[b][i]: output feature n0 + 4 j + i, token 16 b + r
+  float* mine = red + (static_cast<size_t>(wave) * MB * 64 + lane) * 4;
+#pragma unroll
+  for (int b = 0; b < MB; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
+  __syncthreads();
+  for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
+    float sum = 0.f;
+    for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
+    const int b = e / 256, l = (e % 256) / 4, i = e % 4;
+    const int m = b * 16 + l % 16, n = n0 + 4 * (l / 16) + i;
+    if (m < M && n < N) {
+      const size_t idx = static_cast<size_t>(m) * ldc + n;
+      if constexpr (F32OUT) static_cast<float*>(Cv)[idx] = sum;
+      else static_cast<T*>(Cv)[idx] = from_f32<T>(sum);
+    }
+  }
+}
+
+// Waves per workgroup: enough of them over the whole launch to keep every
+// compute unit loading, within what LDS holds for the final sum.
+static int skinny_waves(int N, int K, int MB) {
+  const int row_blocks = (N + 15) / 16;
+  const int chunks = K / 64;
+  int waves = 1;
+  while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * waves < 4096 && waves * 2 <= chunks) waves *= 2;
+  return waves;
+}
+
+template <typename T, bool F32OUT>
+static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                          hipStream_t stream) {
+  const int MB = (M + 15) / 16;
+  const int waves = skinny_waves(N, K, MB);
+  const dim3 grid((N + 15) / 16), block(waves * kWave);
+  const size_t lds = static_cast<size_t>(waves) * MB * 256 * sizeof(float);
+#define LYP_SKINNY(MBV) \
+  gemm_skinny_kernel<T, MBV, F32OUT><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc)
+  if (MB == 1) LYP_SKINNY(1);
+  else if (MB == 2) LYP_SKINNY(2);
+  else if (MB == 3) LYP_SKINNY(3);
+  else LYP_SKINNY(4);
+#undef LYP_SKINNY
+}
+
 template <typename T, int MODE>
 static void launch_gemm(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                         int vec_ok, hipStream_t stream) {
@@ -164,6 +263,19 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
 #define LYP_GEMM(T, MODE)                                                                             \
   launch_gemm<T, MODE>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, \
                        vec_ok, stream)
+  const bool skinny = M <= 64 && K % 64 == 0 && vec_ok && mode != kAccumF32 && (N + 15) / 16 <= 2147483647 / 16;
+  if (skinny) {
+    if (dtype == kF32)
+      launch_skinny<float, true>(static_cast<const float*>(A), static_cast<const float*>(W), C, M, N, K, lda, ldw, ldc, stream);
+    else if (dtype == kBF16 && mode == kStoreF32)
+      launch_skinny<bf16_t, true>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, stream);
+    else if (dtype == kBF16)
+      launch_skinny<bf16_t, false>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, stream);
+    else
+      LYP_REQUIRE(false, "gemm: unknown dtype %d", dtype);
+    LYP_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+  }
   if (dtype == kF32) {
     if (mode == kStoreAct || mode == kStoreF32) LYP_GEMM(float, kStoreF32);
     else LYP_GEMM(float, kAccumF32);

@@ -28,14 +28,18 @@ def _tensor_seed(seed: int, name: str) -> int:
 
 
 def random_tensors(model, seed: int, dtype: torch.dtype, init_std: Optional[float] = None,
-                   norm_init_std: Optional[float] = None) -> Iterator[tuple]:
+                   norm_init_std: Optional[float] = None, device="cpu") -> Iterator[tuple]:
+    """(name, tensor) for every tensor the model expects.  On ``device="cpu"``
+    (the mode that writes model folders) values are reproducible everywhere; on
+    a GPU they come from that device's generator, which is faster for large
+    models and only used where the values do not matter."""
     spec = model.spec
     std = spec.init_std if init_std is None else init_std
     nstd = spec.norm_init_std if norm_init_std is None else norm_init_std
     for name, (shape, init) in model.expected_tensors().items():
-        gen = torch.Generator(device="cpu")
+        gen = torch.Generator(device=device)
         gen.manual_seed(_tensor_seed(seed, name))
-        t = torch.randn(shape, generator=gen, dtype=torch.float32)
+        t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device)
         if init == "ones":
             t = 1.0 + t * nstd
         elif init == "normal":

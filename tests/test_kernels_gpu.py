@@ -89,7 +89,10 @@ def test_swiglu(ops, dtype, I, T):
 # ------------------------------------------------------------------------ gemm
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 172, 96), (33, 256, 172), (130, 1000, 200), (200, 513, 96),
-                                   (64, 128, 4096), (3, 130, 33), (65, 96, 30)])
+                                   (64, 128, 4096), (3, 130, 33), (65, 96, 30),
+                                   # few rows and an inner dimension in steps of 64: the weight-streaming kernel
+                                   (1, 2048, 2048), (8, 3072, 2048), (17, 1000, 128), (64, 130, 8192), (33, 96, 64),
+                                   (5, 16, 64), (48, 515, 192), (2, 128256, 64)])
 def test_gemm(ops, dtype, M, N, K):
     a, w = rnd(M, K, dtype=dtype, seed=9), rnd(N, K, dtype=dtype, scale=0.05, seed=10)
     want = a.double() @ w.double().T
