@@ -109,6 +109,13 @@ class CacheManager:
             n = self._rc(self._lib.lyp_cache_table(self._h, seq_id, group, self._buf, len(self._buf)))
         return list(self._buf[:n])
 
+    def export(self, seq_ids, group: int, tables, slots=None) -> None:
+        """Block tables (and state slots) of several requests at once, written
+        into int32 numpy arrays: row b of ``tables`` gets the table of
+        ``seq_ids[b]`` (an int64 numpy array), as far as it goes."""
+        self._rc(self._lib.lyp_cache_export(self._h, seq_ids.ctypes.data, len(seq_ids), group, tables.ctypes.data,
+                                            tables.shape[1], slots.ctypes.data if slots is not None else None))
+
     def ref_count(self, group: int, page: int) -> int:
         return self._rc(self._lib.lyp_cache_ref_count(self._h, group, page))
 

@@ -36,6 +36,7 @@ def lib() -> ctypes.CDLL:
     L.lyp_cache_num_free_slots.argtypes = [c_void_p]
     L.lyp_cache_num_requests.argtypes = [c_void_p]
     L.lyp_cache_table.argtypes = [c_void_p, c_int64, c_int, i32p, c_int]
+    L.lyp_cache_export.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]
     L.lyp_cache_ref_count.argtypes = [c_void_p, c_int, c_int]
     L.lyp_cache_check.argtypes = [c_void_p]
     L.lyp_cache_counters.argtypes = [c_void_p, i64p]
@@ -48,8 +49,10 @@ def lib() -> ctypes.CDLL:
     L.lyp_sched_abort.argtypes = [c_void_p, c_int64]
     for name in ("has_unfinished", "num_waiting", "num_running"):
         getattr(L, f"lyp_sched_{name}").argtypes = [c_void_p]
-    L.lyp_sched_schedule.argtypes = [c_void_p, i64p, i32p, i32p, i32p, c_int]
+    L.lyp_sched_schedule.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int]
     L.lyp_sched_post_step.argtypes = [c_void_p, i32p, c_int]
+    L.lyp_sched_post_step_status.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int]
+    L.lyp_sched_plan_tokens.argtypes = [c_void_p, c_void_p, c_int]
     L.lyp_sched_last_preempted.argtypes = [c_void_p, i64p, c_int]
     L.lyp_sched_info.argtypes = [c_void_p, c_int64, i32p]
     L.lyp_sched_tokens.argtypes = [c_void_p, c_int64, c_int, i32p, c_int]

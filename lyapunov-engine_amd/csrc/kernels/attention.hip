@@ -5,8 +5,8 @@
 //   * attn_prefill: a wave takes 16 query tokens of one request and up to four
 //     query heads of one key/value head, and walks the keys the tokens may see.
 //   * attn_decode:  a wave takes one request's single new token, all query
-//     heads of one key/value head (as the 16 columns of the tile), and one
-//     64-key partition of the context; attn_combine merges the partitions.
+//     heads of one key/value head (as the 16 columns of the tile), and 64 keys
+//     of the context; a workgroup merges its waves, attn_combine the workgroups.
 // Both read keys and values from pages through the request's block table, and
 // both run after the step's new keys and values have been written, so a
 // prompt portion needs no second source of keys.
@@ -26,7 +26,8 @@
 //                     the operand layout of the P.V product
 //
 // Every 16-key block starts at a multiple of 16 in absolute positions and the
-// decode partitions at multiples of 64, so the order of the additions for a
+// decode partitions at multiples of 64 (waves) and of 64 times the waves of a
+// workgroup, so the order of the additions for a
 // token depends on its position and its window alone, never on how the tokens
 // were cut into steps or on what else is in the batch.
 #include "common.h"
@@ -272,18 +273,26 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------------- decode
-// grid (ceil(max_parts / 4), nkv * column_groups, requests); 256 threads; each
-// wave is one partition.  Column c of the tile is query head
-// kvh * g + 16 * column_group + c of the request's one new token.
+// grid (partitions, nkv * column_groups, requests); kDecodeWaves waves.  A
+// workgroup takes one partition of kDecodeWaves * 64 keys, 64 per wave, and
+// merges its waves' results through LDS, in a fixed order.  Column c of the tile
+// is query head kvh * g + 16 * column_group + c of the request's one new token.
 // Partials: part_o [request][head][part][hd] (not normalised), part_ml
 // [request][head][part][2] = (maximum in the base-2 domain, sum).
+constexpr int kDecodeWaves = HD <= 128 ? 4 : 2;
+constexpr int kBlockKeys = kDecodeWaves * kPartKeys;
+
 template <typename T>
-__global__ __launch_bounds__(256) void attn_decode_kernel(
+__global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const T* __restrict__ q, int q_stride, const void* kpool, const void* vpool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ dec_seqs,
     float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int nh, int nkv, int bs,
     int window, float scale_log2) {
+  __shared__ float s_o[kDecodeWaves][16][HD];
+  __shared__ float s_m[kDecodeWaves][16];
+  __shared__ float s_l[kDecodeWaves][16];
+
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int g = nh / nkv;
   const int col_groups = (g + 15) / 16;
@@ -292,10 +301,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int slot = blockIdx.z;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const int ctx = ctx_len[seq];
-  const int part = blockIdx.x * 4 + wave;
+  const int part = blockIdx.x;
   const int pos = ctx - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  if (part * kPartKeys >= ctx || (part + 1) * kPartKeys <= lo) return;
+  if (part * kBlockKeys >= ctx || (part + 1) * kBlockKeys <= lo) return;  // the whole workgroup
 
   const int col = lane % 16;
   const bool col_valid = h0 + col < g;
@@ -310,60 +319,99 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   Softmax st{LYP_NEG_INF, 0.f};
 
   PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh};
-  const int k_begin = part * kPartKeys;
+  const int k_begin = part * kBlockKeys + wave * kPartKeys;
   const int k_end = min(ctx, k_begin + kPartKeys);
-#pragma unroll 1
-  for (int kb0 = k_begin; kb0 < k_end; kb0 += 16) {
-    if (kb0 + 16 <= lo) continue;
-    Frag<T> kf[kSteps], vf[kSteps];
-    load_k<T>(kf, kv, kb0, lo, ctx, lane);
-    load_v<T>(vf, kv, kb0, lo, ctx, lane);
-    f32x4 s{0.f, 0.f, 0.f, 0.f};
+  if (k_begin < k_end && k_end > lo) {
+    // The next block's keys and values are on their way while this one is used.
+    Frag<T> kf[2][kSteps], vf[2][kSteps];
+    load_k<T>(kf[0], kv, k_begin, lo, ctx, lane);
+    load_v<T>(vf[0], kv, k_begin, lo, ctx, lane);
 #pragma unroll
-    for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[k], qf[k], s);
-    const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
+    for (int it = 0; it < kPartKeys / 16; ++it) {
+      const int kb0 = k_begin + 16 * it;
+      if (kb0 < k_end) {
+        const int cur = it & 1;
+        if (kb0 + 16 < k_end) {
+          load_k<T>(kf[cur ^ 1], kv, kb0 + 16, lo, ctx, lane);
+          load_v<T>(vf[cur ^ 1], kv, kb0 + 16, lo, ctx, lane);
+        }
+        if (kb0 + 16 > lo) {
+          f32x4 s{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[db], pf, o[db]);
+          for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[cur][k], qf[k], s);
+          const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
+#pragma unroll
+          for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[cur][db], pf, o[db]);
+        }
+      }
+    }
   }
 
   const float l = lane_groups_sum(st.lsum);
-  if (!col_valid) return;
-  const size_t pidx = (static_cast<size_t>(slot) * nh + head) * max_parts + part;
-  float* po = part_o + pidx * HD + 4 * (lane / 16);
 #pragma unroll
-  for (int db = 0; db < kSteps; ++db) *reinterpret_cast<f32x4*>(po + db * 16) = o[db];
-  if (lane / 16 == 0) {
-    part_ml[pidx * 2] = st.m;
-    part_ml[pidx * 2 + 1] = l;
+  for (int db = 0; db < kSteps; ++db)
+    *reinterpret_cast<f32x4*>(&s_o[wave][col][db * 16 + 4 * (lane / 16)]) = o[db];
+  if (lane < 16) {
+    s_m[wave][col] = st.m;
+    s_l[wave][col] = l;
+  }
+  __syncthreads();
+
+  const int ncols = min(16, g - h0);
+  for (int e = threadIdx.x; e < ncols * HD; e += kDecodeWaves * kWave) {
+    const int c = e / HD, d = e % HD;
+    float m = s_m[0][c];
+#pragma unroll
+    for (int w = 1; w < kDecodeWaves; ++w) m = fmaxf(m, s_m[w][c]);
+    float acc = 0.f, lsum = 0.f;
+    if (m != LYP_NEG_INF) {
+#pragma unroll
+      for (int w = 0; w < kDecodeWaves; ++w) {
+        if (s_m[w][c] == LYP_NEG_INF) continue;
+        const float wgt = exp2f(s_m[w][c] - m);
+        acc += wgt * s_o[w][c][d];
+        lsum += wgt * s_l[w][c];
+      }
+    }
+    const size_t pidx = (static_cast<size_t>(slot) * nh + kvh * g + h0 + c) * max_parts + part;
+    part_o[pidx * HD + d] = acc;
+    if (d == 0) {
+      part_ml[pidx * 2] = m;
+      part_ml[pidx * 2 + 1] = lsum;
+    }
   }
 }
 
-// grid (nh, requests); 64 threads.
+// grid (nh, requests); one wave.  Lanes first share out the partitions to find
+// the overall maximum and sum, then the dimensions of the head.
 template <typename T>
 __global__ __launch_bounds__(64) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int max_parts,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ dec_seqs, T* __restrict__ out, int out_stride, int nh, int window) {
-  const int head = blockIdx.x, slot = blockIdx.y;
+  const int head = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const int ctx = ctx_len[seq];
   const int lo = window > 0 ? max(0, ctx - window) : 0;
-  const int p_lo = lo / kPartKeys;
-  const int p_hi = (ctx + kPartKeys - 1) / kPartKeys;
+  const int p_lo = lo / kBlockKeys;
+  const int p_hi = (ctx + kBlockKeys - 1) / kBlockKeys;
   const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
 
   float m = LYP_NEG_INF;
-  for (int p = p_lo; p < p_hi; ++p) m = fmaxf(m, part_ml[(base + p) * 2]);
+  for (int p = p_lo + lane; p < p_hi; p += kWave) m = fmaxf(m, ml[p].x);
+  m = wave_max(m);
   const float m_safe = m == LYP_NEG_INF ? 0.f : m;
   float l = 0.f;
-  for (int p = p_lo; p < p_hi; ++p) l += exp2f(part_ml[(base + p) * 2] - m_safe) * part_ml[(base + p) * 2 + 1];
+  for (int p = p_lo + lane; p < p_hi; p += kWave) l += exp2f(ml[p].x - m_safe) * ml[p].y;
+  l = wave_sum(l);
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 
   T* orow = out + static_cast<size_t>(q_start[seq]) * out_stride + static_cast<size_t>(head) * HD;
-  for (int d = threadIdx.x; d < HD; d += 64) {
+  for (int d = lane; d < HD; d += kWave) {
     float acc = 0.f;
-    for (int p = p_lo; p < p_hi; ++p)
-      acc += exp2f(part_ml[(base + p) * 2] - m_safe) * part_o[(base + p) * HD + d];
+#pragma unroll 4
+    for (int p = p_lo; p < p_hi; ++p) acc += exp2f(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
     orow[d] = from_f32<T>(acc * inv);
   }
 }
@@ -385,7 +433,7 @@ using namespace lyp;
 extern "C" {
 
 int lyp_attn_head_dim() { return HD; }
-int lyp_attn_part_keys() { return kPartKeys; }
+int lyp_attn_part_keys() { return kBlockKeys; }
 
 int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
                      const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
@@ -439,18 +487,18 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
   const int g = nh / nkv;
   const int col_groups = (g + 15) / 16;
   LYP_REQUIRE(n_seqs <= 65535 && nkv * col_groups <= 65535, "attn_decode: launch too large");
-  dim3 grid((max_parts + 3) / 4, nkv * col_groups, n_seqs);
+  dim3 grid(max_parts, nkv * col_groups, n_seqs);
   dim3 cgrid(nh, n_seqs);
   const float scale_log2 = scale * kLog2e;
   if (dtype == kF32) {
-    attn_decode_kernel<float><<<grid, 256, 0, stream>>>(
+    attn_decode_kernel<float><<<grid, kDecodeWaves * kWave, 0, stream>>>(
         static_cast<const float*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
         dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
     attn_combine_kernel<float><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,
                                                          dec_seqs, static_cast<float*>(out), out_stride, nh,
                                                          window);
   } else if (dtype == kBF16) {
-    attn_decode_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+    attn_decode_kernel<bf16_t><<<grid, kDecodeWaves * kWave, 0, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
         dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
     attn_combine_kernel<bf16_t><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,

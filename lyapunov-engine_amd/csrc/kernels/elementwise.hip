@@ -61,6 +61,56 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
   }
 }
 
+// The same for rows whose length is a multiple of 4 and fits in registers: one
+// read of the row, 16-byte accesses.
+template <typename TW, typename T, int MAXV>
+__global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                   const TW* __restrict__ w, T* __restrict__ out,
+                                   const int32_t* __restrict__ rows, int H, float eps) {
+  typedef T Vec4T __attribute__((ext_vector_type(4)));
+  typedef TW Vec4W __attribute__((ext_vector_type(4)));
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+  f32x4* hrow = reinterpret_cast<f32x4*>(h + src * H);
+  const Vec4T* drow = delta ? reinterpret_cast<const Vec4T*>(delta + src * H) : nullptr;
+  const bool write_back = drow != nullptr && rows == nullptr;
+  const int nvec = H / 4;
+
+  f32x4 vals[MAXV];
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int idx = threadIdx.x + v * blockDim.x;
+    if (idx < nvec) {
+      f32x4 x = hrow[idx];
+      if (drow) {
+        const Vec4T d = drow[idx];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] += to_f32(d[i]);
+        if (write_back) hrow[idx] = x;
+      }
+      vals[v] = x;
+      ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+  Vec4T* orow = reinterpret_cast<Vec4T*>(out + static_cast<size_t>(r) * H);
+  const Vec4W* wrow = reinterpret_cast<const Vec4W*>(w);
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int idx = threadIdx.x + v * blockDim.x;
+    if (idx < nvec) {
+      const Vec4W wv = wrow[idx];
+      Vec4T o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = from_f32<T>((vals[v][i] * inv) * to_f32(wv[i]));
+      orow[idx] = o;
+    }
+  }
+}
+
 // RMSNorm of rows of activations in their own type (no residual stream); for
 // parts that norm something other than the hidden state.
 template <typename TW, typename T>
@@ -169,11 +219,22 @@ int lyp_rmsnorm(float* h, const void* delta, const void* w, int w_dtype, void* o
                 const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
   if (n_rows == 0) return 0;
-  const int threads = norm_threads(H);
-#define LYP_NORM(TW, T)                                                                         \
-  rmsnorm_kernel<TW, T><<<n_rows, threads, 0, stream>>>(h, static_cast<const T*>(delta),        \
-                                                        static_cast<const TW*>(w),              \
-                                                        static_cast<T*>(out), rows, H, eps)
+  int threads = norm_threads(H);
+  // rows of up to 16384 values in steps of 4, and 16-byte aligned operands, take the one-pass kernel
+  const bool vec = H % 4 == 0 && H <= 16384 && reinterpret_cast<uintptr_t>(h) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (vec) threads = H <= 1024 ? 64 * ((H / 4 + 255) / 256) : (H <= 4096 ? 256 : (H <= 8192 ? 512 : 1024));
+#define LYP_NORM(TW, T)                                                                              \
+  do {                                                                                               \
+    if (vec)                                                                                         \
+      rmsnorm_vec_kernel<TW, T, 4><<<n_rows, threads, 0, stream>>>(                                  \
+          h, static_cast<const T*>(delta), static_cast<const TW*>(w), static_cast<T*>(out), rows, H, eps); \
+    else                                                                                             \
+      rmsnorm_kernel<TW, T><<<n_rows, threads, 0, stream>>>(h, static_cast<const T*>(delta),         \
+                                                            static_cast<const TW*>(w),               \
+                                                            static_cast<T*>(out), rows, H, eps);     \
+  } while (0)
   if (w_dtype == kF32 && act_dtype == kF32) LYP_NORM(float, float);
   else if (w_dtype == kF32 && act_dtype == kBF16) LYP_NORM(float, bf16_t);
   else if (w_dtype == kBF16 && act_dtype == kF32) LYP_NORM(bf16_t, float);

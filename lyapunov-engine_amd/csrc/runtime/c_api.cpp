@@ -106,6 +106,21 @@ int lyp_cache_state_slot(void* h, int64_t id) {
 int lyp_cache_table(void* h, int64_t id, int g, int32_t* out, int cap) {
   return guarded([&] { return copy_out(static_cast<CacheManager*>(h)->table(id, g), out, cap); });
 }
+// For n requests at once: row b of `tables` (each `width` wide) receives the
+// block table of ids[b] in group g, as far as it goes; `slots`, if given, the
+// state slots.  Entries past a table's length are left alone.
+int lyp_cache_export(void* h, const int64_t* ids, int n, int g, int32_t* tables, int width, int32_t* slots) {
+  return guarded([&] {
+    auto* m = static_cast<CacheManager*>(h);
+    for (int b = 0; b < n; ++b) {
+      const auto& t = m->table(ids[b], g);
+      if (static_cast<int>(t.size()) > width) throw std::runtime_error("block table wider than the caller's rows");
+      std::memcpy(tables + static_cast<size_t>(b) * width, t.data(), sizeof(int32_t) * t.size());
+      if (slots) slots[b] = m->state_slot(ids[b]);
+    }
+    return 0;
+  });
+}
 int lyp_cache_ref_count(void* h, int g, int page) {
   return guarded([&] { return static_cast<CacheManager*>(h)->ref_count(g, page); });
 }
@@ -184,6 +199,32 @@ int lyp_sched_post_step(void* h, const int32_t* sampled, int n) {
   return guarded([&] {
     static_cast<Scheduler*>(h)->post_step(std::vector<int32_t>(sampled, sampled + n));
     return 0;
+  });
+}
+// As lyp_sched_post_step; also writes the status of every planned request
+// after the step (in the order of the plan) into status_out.
+int lyp_sched_post_step_status(void* h, const int32_t* sampled, int n, int32_t* status_out, int cap) {
+  return guarded([&] {
+    auto* s = static_cast<Scheduler*>(h);
+    const auto plan = s->plan();
+    if (static_cast<int>(plan.size()) > cap) throw std::runtime_error("post_step: status buffer too small");
+    s->post_step(std::vector<int32_t>(sampled, sampled + n));
+    for (size_t i = 0; i < plan.size(); ++i) status_out[i] = static_cast<int>(s->get(plan[i].id).status);
+    return static_cast<int>(plan.size());
+  });
+}
+// The tokens of the planned portions, one after the other; returns their number.
+int lyp_sched_plan_tokens(void* h, int32_t* out, int cap) {
+  return guarded([&] {
+    auto* s = static_cast<Scheduler*>(h);
+    int n = 0;
+    for (const auto& e : s->plan()) {
+      const auto& seq = s->get(e.id);
+      if (n + e.count > cap) throw std::runtime_error("plan_tokens: buffer too small");
+      std::memcpy(out + n, seq.tokens.data() + e.start, sizeof(int32_t) * static_cast<size_t>(e.count));
+      n += e.count;
+    }
+    return n;
   });
 }
 int lyp_sched_last_preempted(void* h, int64_t* out, int cap) {

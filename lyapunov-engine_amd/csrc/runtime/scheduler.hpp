@@ -98,6 +98,7 @@ class Scheduler {
   bool known(int64_t id) const { return seqs_.count(id) != 0; }
   void forget(int64_t id);  // drop a finished request's record
   const std::vector<int64_t>& last_preempted() const { return last_preempted_; }
+  const std::vector<ScheduledEntry>& plan() const { return plan_; }
 
   struct Counters {
     int64_t steps = 0, scheduled_tokens = 0, preemptions = 0, finished = 0;

@@ -54,10 +54,11 @@ class _Captured:
         self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
         self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
         self.workspace: dict = {}
-        h = self.host.numpy()
+        self.h = h = self.host.numpy()
+        self._rows = np.arange(B)
         h[self.offsets[2]:self.offsets[2] + B + 1] = np.arange(B + 1)
         h[self.offsets[5]:self.offsets[5] + B] = np.arange(B)
-        self.fill(runner, [])
+        self.fill(runner, np.zeros(0, np.int64), np.zeros(0, np.int32), np.zeros(0, np.int32))
         self.dev.copy_(self.host)
 
         def view(i):
@@ -81,37 +82,33 @@ class _Captured:
         with torch.cuda.graph(self.graph, pool=pool):
             self.logits = runner.model.forward(self.ctx, caches)
 
-    def fill(self, runner: ModelRunner, entries: list) -> None:
-        """Write the step's tables into the pinned host buffer; rows past the
-        entries are inert."""
-        B, cache, h, o = self.batch, runner.cache, self.host.numpy(), self.offsets
-        n = len(entries)
-        h[o[0]:o[0] + B] = 0
-        h[o[1]:o[1] + B] = 0
-        h[o[3]:o[3] + B] = 0
-        h[o[4]:o[4] + B] = 0
-        for b, e in enumerate(entries):
-            h[o[0] + b] = e.tokens[0]
-            h[o[1] + b] = e.start
-            h[o[3] + b] = e.start + 1
-            h[o[4] + b] = cache.state_slot(e.seq_id)
+    def fill(self, runner: ModelRunner, ids, starts, tokens) -> None:
+        """Write the step's tables into the pinned host buffer.  ids (int64),
+        starts and tokens (int32) are numpy arrays, one entry per request; rows
+        past them are inert (context 0, slot -1)."""
+        B, cache, h, o = self.batch, runner.cache, self.h, self.offsets
+        n = len(ids)
+        h[o[0]:o[0] + n] = tokens
+        h[o[1]:o[1] + n] = starts
+        h[o[3]:o[3] + n] = starts
+        h[o[3]:o[3] + n] += 1
+        for i in (0, 1, 3, 4):
+            h[o[i] + n:o[i] + B] = 0
+        rows = self._rows[:n]
         for g, gc in enumerate(cache.groups):
             width, ps = self.widths[g], gc.page_size
             sm = h[o[6 + 2 * g]:o[6 + 2 * g] + B]
             bt = h[o[7 + 2 * g]:o[7 + 2 * g] + B * width].reshape(B, width)
-            sm[:] = -1
-            bt[n:] = -1
-            for b, e in enumerate(entries):
-                t = cache.table(e.seq_id, g)
-                bt[b, :len(t)] = t
-                bt[b, len(t):] = -1
-                sm[b] = t[e.start // ps] * ps + e.start % ps
+            if n:
+                cache.export(ids, g, bt, h[o[4]:o[4] + n] if g == 0 else None)
+                sm[:n] = bt[rows, starts // ps] * ps + starts % ps
+            sm[n:] = -1
 
-    def run(self, runner: ModelRunner, entries: list) -> torch.Tensor:
-        self.fill(runner, entries)
+    def run(self, runner: ModelRunner, ids, starts, tokens) -> torch.Tensor:
+        self.fill(runner, ids, starts, tokens)
         self.dev.copy_(self.host, non_blocking=True)
         self.graph.replay()
-        return self.logits[:len(entries)]
+        return self.logits[:len(ids)]
 
 
 class DecodeGraphs:
@@ -129,11 +126,18 @@ class DecodeGraphs:
 
     def step(self, entries: list) -> torch.Tensor:
         """Logits [len(entries), vocab]; valid until the next graph step."""
-        ctx_need = max(e.start + 1 for e in entries)
-        key = (_bucket(len(entries), 1), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
+        return self.step_arrays(np.asarray([e.seq_id for e in entries], dtype=np.int64),
+                                np.asarray([e.start for e in entries], dtype=np.int32),
+                                np.asarray([e.tokens[0] for e in entries], dtype=np.int32))
+
+    def step_arrays(self, ids, starts, tokens) -> torch.Tensor:
+        """The same from numpy arrays: request ids (int64), position and id of
+        each request's one new token (int32)."""
+        ctx_need = int(starts.max()) + 1
+        key = (_bucket(len(ids), 1), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
         cap = self.captured.get(key)
         if cap is None:
             if self.pool is None:
                 self.pool = torch.cuda.graph_pool_handle()
             cap = self.captured[key] = _Captured(self.runner, key[0], key[1], self.pool)
-        return cap.run(self.runner, entries)
+        return cap.run(self.runner, ids, starts, tokens)

@@ -26,7 +26,7 @@ from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .core import EngineCore
 from .runner import StepEntry
-from .scheduler import FINISH_REASON, Scheduler
+from .scheduler import FINISH_REASON, STATUS, Scheduler
 
 
 class RequestOutput:
@@ -42,6 +42,14 @@ class RequestOutput:
     def __repr__(self):
         return (f"RequestOutput(request_id={self.request_id!r}, output_tokens={self.output_tokens}, "
                 f"finished={self.finished}, finish_reason={self.finish_reason!r})")
+
+
+class _Request:
+    __slots__ = ("request_id", "params", "stream", "prompt", "outputs")
+
+    def __init__(self, request_id, params, stream, prompt):
+        self.request_id, self.params, self.stream, self.prompt = request_id, params, stream, prompt
+        self.outputs: list = []
 
 
 class LLMEngine:
@@ -65,7 +73,7 @@ class LLMEngine:
                                    eos_token_ids=tuple(eos))
         self.sampler = Sampler(self.core.device, seed=config.seed)
         self.req_counter = 0
-        self._requests: dict = {}     # seq id -> (request id, SamplingParams, stream)
+        self._requests: dict = {}     # seq id -> _Request
         self._by_request: dict = {}   # request id -> seq id
         self.graphs = None
         if config.enable_graphs:
@@ -92,7 +100,7 @@ class LLMEngine:
         self.req_counter += 1
         self.scheduler.add(seq_id, prompt, params)
         stream = params.seed if params.seed is not None else seq_id
-        self._requests[seq_id] = (request_id, params, stream)
+        self._requests[seq_id] = _Request(request_id, params, stream, prompt)
         self._by_request[request_id] = seq_id
         return request_id
 
@@ -105,8 +113,8 @@ class LLMEngine:
         return done
 
     def _drop(self, seq_id: int) -> None:
-        request_id, _, _ = self._requests.pop(seq_id)
-        self._by_request.pop(request_id, None)
+        req = self._requests.pop(seq_id)
+        self._by_request.pop(req.request_id, None)
         self.scheduler.forget(seq_id)
 
     def has_unfinished_requests(self) -> bool:
@@ -114,36 +122,46 @@ class LLMEngine:
 
     # -------------------------------------------------------------------- step
     def step(self) -> list:
+        """One iteration.  Returns a RequestOutput for every request that took
+        part; ``output_tokens`` of an unfinished request is the engine's own
+        growing list (copy it to keep a snapshot)."""
         if not self.has_unfinished_requests():
             return []
-        plan = self.scheduler.schedule()
-        if not plan:
+        ids, start, count, wants = self.scheduler.schedule_arrays()
+        n = len(ids)
+        if n == 0:
             return []  # everything running was preempted; the next step admits again
-        entries = [StepEntry(p.seq_id, self.scheduler.tokens(p.seq_id, p.start, p.count), p.start,
-                             [p.count - 1] if p.wants_logits else []) for p in plan]
-        if self.graphs is not None and self.graphs.usable(entries):
-            logits = self.graphs.step(entries)
+        tokens = self.scheduler.plan_tokens()
+        if self.graphs is not None and self.graphs.safe and n <= self.graphs.max_batch and \
+                bool((count == 1).all()) and bool(wants.all()):
+            logits = self.graphs.step_arrays(ids, start, tokens)
         else:
+            entries, at = [], 0
+            for i in range(n):
+                c = int(count[i])
+                entries.append(StepEntry(int(ids[i]), tokens[at:at + c].tolist(), int(start[i]),
+                                         [c - 1] if wants[i] else []))
+                at += c
             logits = self.core.step(entries)
+        reqs = [self._requests[int(i)] for i in ids]
+        wanting = [r for r, w in zip(reqs, wants) if w]
         sampled = []
-        wanting = [p for p in plan if p.wants_logits]
         if wanting:
-            params = [self._requests[p.seq_id][1] for p in wanting]
-            streams = [self._requests[p.seq_id][2] for p in wanting]
-            indices = [self.scheduler.info(p.seq_id).total_len - self.scheduler.info(p.seq_id).prompt_len
-                       for p in wanting]
-            sampled = self.sampler.sample(logits, params, streams, indices)
-        self.scheduler.post_step(sampled)
-
-        outputs = []
-        for p in plan:
-            info = self.scheduler.info(p.seq_id)
-            tokens = self.scheduler.tokens(p.seq_id)
-            request_id = self._requests[p.seq_id][0]
-            outputs.append(RequestOutput(request_id, tokens[:info.prompt_len], tokens[info.prompt_len:],
-                                         info.finished, FINISH_REASON.get(info.status)))
-            if info.finished:
-                self._drop(p.seq_id)
+            sampled = self.sampler.sample(logits, [r.params for r in wanting], [r.stream for r in wanting],
+                                          [len(r.outputs) for r in wanting])
+        status = self.scheduler.post_step_status(sampled)
+        outputs, k = [], 0
+        for i in range(n):
+            req = reqs[i]
+            if wants[i]:
+                req.outputs.append(sampled[k])
+                k += 1
+            code = int(status[i])
+            finished = code >= 2
+            outputs.append(RequestOutput(req.request_id, req.prompt, req.outputs, finished,
+                                         FINISH_REASON.get(STATUS[code])))
+            if finished:
+                self._drop(int(ids[i]))
         return outputs
 
     def generate(self, prompts: list, params=None) -> list:

@@ -7,6 +7,8 @@ from __future__ import annotations
 from ctypes import c_float, c_int32, c_int64, c_uint64
 from dataclasses import dataclass
 
+import numpy as np
+
 from ..cache import runtime_lib
 from ..cache.manager import CacheManager
 from ..sampling.params import SamplingParams
@@ -51,10 +53,12 @@ class Scheduler:
         if not self._h:
             raise SchedulerError(runtime_lib.last_error())
         self._cap = max(max_num_seqs, 1) + 8
-        self._ids = (c_int64 * self._cap)()
-        self._start = (c_int32 * self._cap)()
-        self._count = (c_int32 * self._cap)()
-        self._wants = (c_int32 * self._cap)()
+        self._ids = np.zeros(self._cap, dtype=np.int64)
+        self._start = np.zeros(self._cap, dtype=np.int32)
+        self._count = np.zeros(self._cap, dtype=np.int32)
+        self._wants = np.zeros(self._cap, dtype=np.int32)
+        self._status = np.zeros(self._cap, dtype=np.int32)
+        self._tokens = np.zeros(max(max_num_batched_tokens, 1), dtype=np.int32)
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -84,9 +88,30 @@ class Scheduler:
     def num_running(self) -> int:
         return self._lib.lyp_sched_num_running(self._h)
 
+    def schedule_arrays(self):
+        """Plan a step -> (ids, start, count, wants): numpy views, valid until
+        the next call."""
+        n = self._rc(self._lib.lyp_sched_schedule(self._h, self._ids.ctypes.data, self._start.ctypes.data,
+                                                  self._count.ctypes.data, self._wants.ctypes.data, self._cap))
+        return self._ids[:n], self._start[:n], self._count[:n], self._wants[:n]
+
     def schedule(self) -> list:
-        n = self._rc(self._lib.lyp_sched_schedule(self._h, self._ids, self._start, self._count, self._wants, self._cap))
-        return [Scheduled(self._ids[i], self._start[i], self._count[i], bool(self._wants[i])) for i in range(n)]
+        ids, start, count, wants = self.schedule_arrays()
+        return [Scheduled(int(i), int(s), int(c), bool(w)) for i, s, c, w in zip(ids, start, count, wants)]
+
+    def plan_tokens(self):
+        """The tokens of the planned portions, one after the other (a numpy
+        view, valid until the next call)."""
+        n = self._rc(self._lib.lyp_sched_plan_tokens(self._h, self._tokens.ctypes.data, len(self._tokens)))
+        return self._tokens[:n]
+
+    def post_step_status(self, sampled):
+        """post_step, returning the status code of every planned request after
+        the step (index into STATUS), in the order of the plan."""
+        arr = np.ascontiguousarray(sampled, dtype=np.int32)
+        n = self._rc(self._lib.lyp_sched_post_step_status(self._h, arr.ctypes.data, len(arr),
+                                                          self._status.ctypes.data, self._cap))
+        return self._status[:n]
 
     def post_step(self, sampled: list) -> None:
         arr = (c_int32 * max(1, len(sampled)))(*sampled)

@@ -39,6 +39,17 @@ class Sampler:
     def __init__(self, device, seed: int = 0):
         self.device = torch.device(device)
         self.seed = seed
+        self._cap = 0
+        self._host = self._dev = self._out = None
+
+    def _reserve(self, rows: int) -> None:
+        if rows > self._cap:
+            self._cap = max(rows, 2 * self._cap, 64)
+            # rows of the parameter block: temperature, top_p, uniform, top_k (as int32 bits)
+            self._host = torch.zeros((4, self._cap), dtype=torch.float32).pin_memory()
+            self._dev = torch.zeros((4, self._cap), dtype=torch.float32, device=self.device)
+            self._out = torch.zeros(self._cap, dtype=torch.int32, device=self.device)
+            self._greedy_on_device = True   # the device block is all zeros: temperature 0 everywhere
 
     def sample(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> list:
         """logits [R, vocab] float on the device; one SamplingParams, stream id
@@ -46,17 +57,25 @@ class Sampler:
         R = logits.shape[0]
         if not (len(params) == len(streams) == len(indices) == R):
             raise ValueError("one set of sampling parameters per row of logits")
-        host = torch.empty((4, R), dtype=torch.float32)
-        for r, (p, s, i) in enumerate(zip(params, streams, indices)):
-            host[0, r] = p.temperature
-            host[1, r] = p.top_p
-            host[2, r] = uniform(self.seed, s, i)
-            host[3, r] = 0.0
-        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32)
-        dev = host.to(self.device)
-        out = torch.empty(R, dtype=torch.int32, device=self.device)
-        ops.sample(logits, dev[0], top_k.to(self.device), dev[1], dev[2], out)
-        return out.cpu().tolist()
+        self._reserve(R)
+        if all(p.temperature < 1e-4 for p in params):
+            if not self._greedy_on_device:
+                self._dev.zero_()
+                self._greedy_on_device = True
+        else:
+            h = self._host
+            hk = h[3].view(torch.int32)
+            for r, (p, s, i) in enumerate(zip(params, streams, indices)):
+                h[0, r] = p.temperature
+                h[1, r] = p.top_p
+                h[2, r] = uniform(self.seed, s, i)
+                hk[r] = p.top_k
+            self._dev[:, :R].copy_(h[:, :R], non_blocking=True)
+            self._greedy_on_device = False
+        d = self._dev
+        out = self._out[:R]
+        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out)
+        return out.tolist()
 
 
 __all__ = ["Sampler", "SamplingParams", "uniform"]
