@@ -61,16 +61,23 @@ struct PagedKV {
   const void* vpool;
   const int32_t* table;  // this request's row of the block table
   int nkv, bs, kvh;
+  int max_blocks;        // width of the row: an index below it may always be read
 };
+
+// The table entry for a key, read whether or not the key is inside the
+// request: the index is clamped to the row, the result is used only for keys
+// that exist.  Lets the read start before the request's length is known.
+__device__ __forceinline__ int page_of(const PagedKV& kv, int key) {
+  return kv.table[min(key / kv.bs, kv.max_blocks - 1)];
+}
 
 // Keys kb0 .. kb0+15 as the row operand of S^T = K . Q^T.  Lane (r, j) holds
 // key kb0 + r, dimensions j * kSlice + 4 * step + {0..3}.
 template <typename T>
-__device__ __forceinline__ void load_k(Frag<T> (&kf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
-                                       int lane) {
+__device__ __forceinline__ void load_k_page(Frag<T> (&kf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                            int lane, int page) {
   const int key = kb0 + lane % 16;
   if (key >= lo && key < hi) {
-    const int page = kv.table[key / kv.bs];
     if (page >= 0) {
       const T* row = static_cast<const T*>(kv.kpool) +
                      ((static_cast<size_t>(page) * kv.nkv + kv.kvh) * kv.bs + key % kv.bs) * HD +
@@ -84,13 +91,21 @@ __device__ __forceinline__ void load_k(Frag<T> (&kf)[kSteps], const PagedKV& kv,
   for (int s = 0; s < kSteps; ++s) kf[s] = zero_frag<T>();
 }
 
+template <typename T>
+__device__ __forceinline__ void load_k(Frag<T> (&kf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                       int lane) {
+  load_k_page<T>(kf, kv, kb0, lo, hi, lane, page_of(kv, kb0 + lane % 16));
+}
+
 // Values of the same 16 keys as the row operand of O^T = V^T . P^T.  Lane
 // (r, j) holds, per 16-row block db of the head dimension, dimension
 // db * 16 + r and keys kb0 + 4 j + {0..3}.  Anything outside [lo, hi) reads as
 // zero: a page that was never written may hold any bit pattern.
+// `page0` is the table entry of the lane's first key (used when a page holds a
+// multiple of four keys, so that the lane's four keys share it).
 template <typename T>
-__device__ __forceinline__ void load_v(Frag<T> (&vf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
-                                       int lane) {
+__device__ __forceinline__ void load_v_page(Frag<T> (&vf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                            int lane, int page0) {
   const int key0 = kb0 + 4 * (lane / 16);
   const int r = lane % 16;
   const T* vpool = static_cast<const T*>(kv.vpool);
@@ -98,7 +113,7 @@ __device__ __forceinline__ void load_v(Frag<T> (&vf)[kSteps], const PagedKV& kv,
   for (int db = 0; db < kSteps; ++db) vf[db] = zero_frag<T>();
   if (kv.bs % 4 == 0) {
     if (key0 < hi && key0 + 3 >= lo) {
-      const int page = kv.table[key0 / kv.bs];
+      const int page = page0;
       if (page >= 0) {
         const T* base = vpool + (static_cast<size_t>(page) * kv.nkv + kv.kvh) * HD * kv.bs + key0 % kv.bs;
 #pragma unroll
@@ -123,6 +138,12 @@ __device__ __forceinline__ void load_v(Frag<T> (&vf)[kSteps], const PagedKV& kv,
       for (int db = 0; db < kSteps; ++db) vf[db][i] = base[static_cast<size_t>(db * 16 + r) * kv.bs];
     }
   }
+}
+
+template <typename T>
+__device__ __forceinline__ void load_v(Frag<T> (&vf)[kSteps], const PagedKV& kv, int kb0, int lo, int hi,
+                                       int lane) {
+  load_v_page<T>(vf, kv, kb0, lo, hi, lane, page_of(kv, kb0 + 4 * (lane / 16)));
 }
 
 // A query row as the column operand, in the same order of dimensions as load_k.
@@ -235,7 +256,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     for (int db = 0; db < kSteps; ++db) o[cb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh};
+  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
   const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int hi = pos_last + 1;  // keys at or above it are invisible to every token of the wave
 
@@ -300,8 +321,20 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int h0 = (blockIdx.y % col_groups) * 16;
   const int slot = blockIdx.z;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
-  const int ctx = ctx_len[seq];
   const int part = blockIdx.x;
+  constexpr int kBlocks = kPartKeys / 16;  // 16-key blocks per wave
+  const int k_begin = part * kBlockKeys + wave * kPartKeys;
+
+  // Table entries of the wave's keys, read before the request's length is
+  // known, so that they travel together with it.
+  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
+  int page_k[kBlocks], page_v[kBlocks];
+#pragma unroll
+  for (int it = 0; it < kBlocks; ++it) {
+    page_k[it] = page_of(kv, k_begin + 16 * it + lane % 16);
+    page_v[it] = page_of(kv, k_begin + 16 * it + 4 * (lane / 16));
+  }
+  const int ctx = ctx_len[seq];
   const int pos = ctx - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   if (part * kBlockKeys >= ctx || (part + 1) * kBlockKeys <= lo) return;  // the whole workgroup
@@ -318,30 +351,31 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   Softmax st{LYP_NEG_INF, 0.f};
 
-  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh};
-  const int k_begin = part * kBlockKeys + wave * kPartKeys;
   const int k_end = min(ctx, k_begin + kPartKeys);
   if (k_begin < k_end && k_end > lo) {
-    // The next block's keys and values are on their way while this one is used.
-    Frag<T> kf[2][kSteps], vf[2][kSteps];
-    load_k<T>(kf[0], kv, k_begin, lo, ctx, lane);
-    load_v<T>(vf[0], kv, k_begin, lo, ctx, lane);
+    // Blocks are loaded a group at a time, the whole group in flight at once;
+    // the group is as large as the register file allows for this head size.
+    constexpr int kGroup = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
 #pragma unroll
-    for (int it = 0; it < kPartKeys / 16; ++it) {
-      const int kb0 = k_begin + 16 * it;
-      if (kb0 < k_end) {
-        const int cur = it & 1;
-        if (kb0 + 16 < k_end) {
-          load_k<T>(kf[cur ^ 1], kv, kb0 + 16, lo, ctx, lane);
-          load_v<T>(vf[cur ^ 1], kv, kb0 + 16, lo, ctx, lane);
-        }
-        if (kb0 + 16 > lo) {
+    for (int g0 = 0; g0 < kBlocks; g0 += kGroup) {
+      if (k_begin + 16 * g0 >= k_end) break;
+      Frag<T> kf[kGroup][kSteps], vf[kGroup][kSteps];
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const int kb0 = k_begin + 16 * (g0 + u);
+        load_k_page<T>(kf[u], kv, kb0, lo, ctx, lane, page_k[g0 + u]);
+        load_v_page<T>(vf[u], kv, kb0, lo, ctx, lane, page_v[g0 + u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kGroup; ++u) {
+        const int kb0 = k_begin + 16 * (g0 + u);
+        if (kb0 < k_end && kb0 + 16 > lo) {
           f32x4 s{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[cur][k], qf[k], s);
+          for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[u][k], qf[k], s);
           const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
 #pragma unroll
-          for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[cur][db], pf, o[db]);
+          for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf, o[db]);
         }
       }
     }

@@ -30,22 +30,29 @@ __global__ void embedding_kernel(const int32_t* __restrict__ ids, const TW* __re
 // h is the 32-bit residual stream.  With `delta`, h + delta is normed, and
 // written back to h unless `rows` selects a subset (the last norm before the
 // output head, where h is not used again).
-template <typename TW, typename T>
-__global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
-                               const TW* __restrict__ w, T* __restrict__ out,
+// `delta` may come as n_parts partial sums, part_stride elements apart, that
+// are added up here in order (what the few-rows product leaves behind).
+template <typename TW, typename TD, typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_parts,
+                               size_t part_stride, const TW* __restrict__ w, T* __restrict__ out,
                                const int32_t* __restrict__ rows, int H, float eps) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   float* hrow = h + src * H;
-  const T* drow = delta ? delta + src * H : nullptr;
+  const TD* drow = delta ? delta + src * H : nullptr;
   const bool write_back = drow != nullptr && rows == nullptr;
+  auto delta_at = [&](int i) {
+    float d = 0.f;
+    for (int p = 0; p < n_parts; ++p) d += to_f32(drow[p * part_stride + i]);
+    return d;
+  };
 
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hrow[i];
     if (drow) {
-      v += to_f32(drow[i]);
+      v += delta_at(i);
       if (write_back) hrow[i] = v;
     }
     ss += v * v;
@@ -56,26 +63,28 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delt
   T* orow = out + static_cast<size_t>(r) * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = hrow[i];
-    if (drow && !write_back) v += to_f32(drow[i]);
+    if (drow && !write_back) v += delta_at(i);
     orow[i] = from_f32<T>((v * inv) * to_f32(w[i]));
   }
 }
 
 // The same for rows whose length is a multiple of 4 and fits in registers: one
 // read of the row, 16-byte accesses.
-template <typename TW, typename T, int MAXV>
-__global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
-                                   const TW* __restrict__ w, T* __restrict__ out,
+template <typename TW, typename TD, typename T, int MAXV>
+__global__ void rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_parts,
+                                   size_t part_stride, const TW* __restrict__ w, T* __restrict__ out,
                                    const int32_t* __restrict__ rows, int H, float eps) {
   typedef T Vec4T __attribute__((ext_vector_type(4)));
+  typedef TD Vec4D __attribute__((ext_vector_type(4)));
   typedef TW Vec4W __attribute__((ext_vector_type(4)));
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   f32x4* hrow = reinterpret_cast<f32x4*>(h + src * H);
-  const Vec4T* drow = delta ? reinterpret_cast<const Vec4T*>(delta + src * H) : nullptr;
+  const Vec4D* drow = delta ? reinterpret_cast<const Vec4D*>(delta + src * H) : nullptr;
   const bool write_back = drow != nullptr && rows == nullptr;
   const int nvec = H / 4;
+  const size_t part_vecs = part_stride / 4;
 
   f32x4 vals[MAXV];
   float ss = 0.f;
@@ -85,9 +94,11 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ 
     if (idx < nvec) {
       f32x4 x = hrow[idx];
       if (drow) {
-        const Vec4T d = drow[idx];
+        for (int p = 0; p < n_parts; ++p) {
+          const Vec4D d = drow[p * part_vecs + idx];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) x[i] += to_f32(d[i]);
+          for (int i = 0; i < 4; ++i) x[i] += to_f32(d[i]);
+        }
         if (write_back) hrow[idx] = x;
       }
       vals[v] = x;
@@ -174,13 +185,17 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, const int32_t* __restrict__ 
 }
 
 // --------------------------------------------------------------------- SwiGLU
+// interleave == 0: a row of gu is all gates, then all ups.  interleave == 8:
+// tiles of 16 columns, eight gates then the eight ups that go with them.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, int interleave) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t t = idx / I, i = idx % I;
-  const float g = to_f32(gu[t * 2 * I + i]);
-  const float u = to_f32(gu[t * 2 * I + I + i]);
+  const size_t gi = interleave ? (i / 8) * 16 + i % 8 : i;
+  const size_t ui = interleave ? gi + 8 : I + i;
+  const float g = to_f32(gu[t * 2 * I + gi]);
+  const float u = to_f32(gu[t * 2 * I + ui]);
   out[idx] = from_f32<T>((g / (1.0f + expf(-g))) * u);
 }
 
@@ -214,32 +229,45 @@ int lyp_embedding(const int32_t* ids, const void* table, int table_dtype, float*
   return 0;
 }
 
-// h [*, H] float; delta, out of act_dtype; w of w_dtype; rows optional [n_rows].
-int lyp_rmsnorm(float* h, const void* delta, const void* w, int w_dtype, void* out, int act_dtype,
-                const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
+// h [*, H] float; out of act_dtype; w of w_dtype; rows optional [n_rows].
+// delta (optional) is either one tensor of act_dtype (delta_parts == 0) or
+// delta_parts float tensors, part_stride elements apart, whose sum is meant.
+int lyp_rmsnorm(float* h, const void* delta, int delta_parts, long long part_stride, const void* w, int w_dtype,
+                void* out, int act_dtype, const int32_t* rows, int n_rows, int H, float eps, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  LYP_REQUIRE(delta_parts >= 0 && (delta_parts == 0 || delta != nullptr), "rmsnorm: partial sums without data");
   if (n_rows == 0) return 0;
   int threads = norm_threads(H);
+  const bool parts = delta_parts > 0;
+  const int n_parts = parts ? delta_parts : 1;
+  const size_t stride = parts ? static_cast<size_t>(part_stride) : 0;
   // rows of up to 16384 values in steps of 4, and 16-byte aligned operands, take the one-pass kernel
   const bool vec = H % 4 == 0 && H <= 16384 && reinterpret_cast<uintptr_t>(h) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(delta) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(out) % 16 == 0;
+                   reinterpret_cast<uintptr_t>(out) % 16 == 0 && stride % 4 == 0;
   if (vec) threads = H <= 1024 ? 64 * ((H / 4 + 255) / 256) : (H <= 4096 ? 256 : (H <= 8192 ? 512 : 1024));
-#define LYP_NORM(TW, T)                                                                              \
-  do {                                                                                               \
-    if (vec)                                                                                         \
-      rmsnorm_vec_kernel<TW, T, 4><<<n_rows, threads, 0, stream>>>(                                  \
-          h, static_cast<const T*>(delta), static_cast<const TW*>(w), static_cast<T*>(out), rows, H, eps); \
-    else                                                                                             \
-      rmsnorm_kernel<TW, T><<<n_rows, threads, 0, stream>>>(h, static_cast<const T*>(delta),         \
-                                                            static_cast<const TW*>(w),               \
-                                                            static_cast<T*>(out), rows, H, eps);     \
+#define LYP_NORM(TW, TD, T)                                                                           \
+  do {                                                                                                \
+    if (vec)                                                                                          \
+      rmsnorm_vec_kernel<TW, TD, T, 4><<<n_rows, threads, 0, stream>>>(                               \
+          h, static_cast<const TD*>(delta), n_parts, stride, static_cast<const TW*>(w),               \
+          static_cast<T*>(out), rows, H, eps);                                                        \
+    else                                                                                              \
+      rmsnorm_kernel<TW, TD, T><<<n_rows, threads, 0, stream>>>(                                      \
+          h, static_cast<const TD*>(delta), n_parts, stride, static_cast<const TW*>(w),               \
+          static_cast<T*>(out), rows, H, eps);                                                        \
   } while (0)
-  if (w_dtype == kF32 && act_dtype == kF32) LYP_NORM(float, float);
-  else if (w_dtype == kF32 && act_dtype == kBF16) LYP_NORM(float, bf16_t);
-  else if (w_dtype == kBF16 && act_dtype == kF32) LYP_NORM(bf16_t, float);
-  else if (w_dtype == kBF16 && act_dtype == kBF16) LYP_NORM(bf16_t, bf16_t);
+#define LYP_NORM_D(TW, T)               \
+  do {                                  \
+    if (parts) LYP_NORM(TW, float, T);  \
+    else LYP_NORM(TW, T, T);            \
+  } while (0)
+  if (w_dtype == kF32 && act_dtype == kF32) LYP_NORM_D(float, float);
+  else if (w_dtype == kF32 && act_dtype == kBF16) LYP_NORM_D(float, bf16_t);
+  else if (w_dtype == kBF16 && act_dtype == kF32) LYP_NORM_D(bf16_t, float);
+  else if (w_dtype == kBF16 && act_dtype == kBF16) LYP_NORM_D(bf16_t, bf16_t);
   else LYP_REQUIRE(false, "rmsnorm: unknown dtypes w=%d act=%d", w_dtype, act_dtype);
+#undef LYP_NORM_D
 #undef LYP_NORM
   LYP_LAUNCH_CHECK("rmsnorm");
   return 0;
@@ -290,18 +318,19 @@ int lyp_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const floa
   return 0;
 }
 
-int lyp_swiglu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t stream) {
+int lyp_swiglu(const void* gate_up, void* out, int dtype, int T, int I, int interleave, hipStream_t stream) {
   LYP_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  LYP_REQUIRE(interleave == 0 || (interleave == 8 && I % 8 == 0), "swiglu: interleave %d with I=%d", interleave, I);
   const size_t total = static_cast<size_t>(T) * I;
   if (total == 0) return 0;
   const int threads = 256;
   const unsigned blocks = static_cast<unsigned>((total + threads - 1) / threads);
   if (dtype == kF32)
     swiglu_kernel<float><<<blocks, threads, 0, stream>>>(static_cast<const float*>(gate_up),
-                                                         static_cast<float*>(out), I, total);
+                                                         static_cast<float*>(out), I, total, interleave);
   else if (dtype == kBF16)
     swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>(static_cast<const bf16_t*>(gate_up),
-                                                          static_cast<bf16_t*>(out), I, total);
+                                                          static_cast<bf16_t*>(out), I, total, interleave);
   else
     LYP_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("swiglu");

@@ -135,13 +135,21 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
 // ---------------------------------------------------------------- few rows
 // M <= 64 (decode steps): the weight matrix is read once from memory and the
 // time is what that read takes, so the shape is chosen for memory parallelism.
-// A workgroup owns 16 rows of W (16 output features); its waves split the inner
-// dimension between them and add their parts through LDS, in a fixed order.  A
-// wave keeps the 16 x (16 MB) output tile in registers: W rows are the row
-// operand, tokens the columns.  Per 64 values of the inner dimension a lane
+// A workgroup owns 16 rows of W (16 output features) and, when the matrix has
+// few rows, one of several slices of the inner dimension (grid.y); its waves
+// split the slice between them and add their parts through LDS, in a fixed
+// order.  A wave keeps the 16 x (16 MB) output tile in registers: W rows are the
+// row operand, tokens the columns.  Per 64 values of the inner dimension a lane
 // reads one contiguous run of 16 values of its row; activations come through
 // the cache, they are small.  Needs K % 64 == 0 and 16-byte aligned rows.
-template <typename T, int MB, bool F32OUT>
+//
+// Epilogues: store in the operands' type; store float; SiLU-gate (rows 0-7 of
+// the tile are gate features, rows 8-15 the matching up features: the output
+// has half as many columns); or float partial sums per slice, [slice][M][N],
+// which the consumer adds up (the RMSNorm kernels do).
+enum SkinnyEpilogue : int { kEpiAct = 0, kEpiF32 = 1, kEpiSwiglu = 2, kEpiParts = 3 };
+
+template <typename T, int MB, int EPI>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
                                                            int ldw, int ldc) {
@@ -157,8 +165,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   const int wrow = min(n0 + r, N - 1);  // rows past the end read the last row and are not stored
 
   const int chunks = K / 64;
-  const int per_wave = (chunks + nwaves - 1) / nwaves;
-  const int c_begin = min(chunks, wave * per_wave), c_end = min(chunks, c_begin + per_wave);
+  const int per_slice = (chunks + gridDim.y - 1) / gridDim.y;
+  const int s_begin = min(chunks, static_cast<int>(blockIdx.y) * per_slice), s_end = min(chunks, s_begin + per_slice);
+  const int per_wave = (s_end - s_begin + nwaves - 1) / nwaves;
+  const int c_begin = min(s_end, s_begin + wave * per_wave), c_end = min(s_end, c_begin + per_wave);
 
   f32x4 acc[MB];
 #pragma unroll
@@ -169,7 +179,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
   for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * 16;
 
-#pragma unroll 2
+#pragma unroll 4
   for (int c = c_begin; c < c_end; ++c) {
     const int k0 = c * 64;
     Frag wf[NF];
@@ -190,38 +200,65 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
   for (int b = 0; b < MB; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
   __syncthreads();
-  for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
+  auto total = [&](int e) {
     float sum = 0.f;
     for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
+    return sum;
+  };
+  for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
     const int b = e / 256, l = (e % 256) / 4, i = e % 4;
-    const int m = b * 16 + l % 16, n = n0 + 4 * (l / 16) + i;
-    if (m < M && n < N) {
-      const size_t idx = static_cast<size_t>(m) * ldc + n;
-      if constexpr (F32OUT) static_cast<float*>(Cv)[idx] = sum;
-      else static_cast<T*>(Cv)[idx] = from_f32<T>(sum);
+    const int row = 4 * (l / 16) + i;
+    const int m = b * 16 + l % 16, n = n0 + row;
+    if (m >= M || n >= N) continue;
+    if constexpr (EPI == kEpiSwiglu) {
+      if (row >= 8) continue;
+      const float gate = total(e), up = total(e + 128);  // the same token, row + 8
+      static_cast<T*>(Cv)[static_cast<size_t>(m) * ldc + (n0 / 2 + row)] =
+          from_f32<T>((gate / (1.0f + expf(-gate))) * up);
+    } else if constexpr (EPI == kEpiParts) {
+      static_cast<float*>(Cv)[(static_cast<size_t>(blockIdx.y) * M + m) * ldc + n] = total(e);
+    } else if constexpr (EPI == kEpiF32) {
+      static_cast<float*>(Cv)[static_cast<size_t>(m) * ldc + n] = total(e);
+    } else {
+      static_cast<T*>(Cv)[static_cast<size_t>(m) * ldc + n] = from_f32<T>(total(e));
     }
   }
 }
 
+static bool skinny_ok(int M, int K, int lda, int ldw, const void* A, const void* W, int dtype) {
+  const int vec = dtype == kF32 ? 4 : 8;
+  return M >= 1 && M <= 64 && K % 64 == 0 && lda % vec == 0 && ldw % vec == 0 &&
+         reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+}
+
+// Slices of the inner dimension for a product whose result may come as partial
+// sums: a matrix with few rows does not give every compute unit a workgroup.
+static int skinny_slices(int N, int K) {
+  const int row_blocks = (N + 15) / 16;
+  int slices = 1;
+  while (slices < 8 && row_blocks * slices < 512 && K / (slices * 2) >= 512) slices *= 2;
+  return slices;
+}
+
 // Waves per workgroup: enough of them over the whole launch to keep every
 // compute unit loading, within what LDS holds for the final sum.
-static int skinny_waves(int N, int K, int MB) {
+static int skinny_waves(int N, int K, int MB, int slices) {
   const int row_blocks = (N + 15) / 16;
-  const int chunks = K / 64;
+  const int chunks = K / 64 / slices;
   int waves = 1;
-  while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * waves < 4096 && waves * 2 <= chunks) waves *= 2;
+  while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * slices * waves < 4096 && waves * 2 <= chunks) waves *= 2;
   return waves;
 }
 
-template <typename T, bool F32OUT>
+template <typename T, int EPI>
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
-                          hipStream_t stream) {
+                          int slices, hipStream_t stream) {
   const int MB = (M + 15) / 16;
-  const int waves = skinny_waves(N, K, MB);
-  const dim3 grid((N + 15) / 16), block(waves * kWave);
+  const int waves = skinny_waves(N, K, MB, slices);
+  const dim3 grid((N + 15) / 16, slices), block(waves * kWave);
   const size_t lds = static_cast<size_t>(waves) * MB * 256 * sizeof(float);
 #define LYP_SKINNY(MBV) \
-  gemm_skinny_kernel<T, MBV, F32OUT><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc)
+  gemm_skinny_kernel<T, MBV, EPI><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc)
   if (MB == 1) LYP_SKINNY(1);
   else if (MB == 2) LYP_SKINNY(2);
   else if (MB == 3) LYP_SKINNY(3);
@@ -263,14 +300,13 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
 #define LYP_GEMM(T, MODE)                                                                             \
   launch_gemm<T, MODE>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, \
                        vec_ok, stream)
-  const bool skinny = M <= 64 && K % 64 == 0 && vec_ok && mode != kAccumF32 && (N + 15) / 16 <= 2147483647 / 16;
-  if (skinny) {
+  if (mode != kAccumF32 && skinny_ok(M, K, lda, ldw, A, W, dtype)) {
     if (dtype == kF32)
-      launch_skinny<float, true>(static_cast<const float*>(A), static_cast<const float*>(W), C, M, N, K, lda, ldw, ldc, stream);
+      launch_skinny<float, kEpiF32>(static_cast<const float*>(A), static_cast<const float*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else if (dtype == kBF16 && mode == kStoreF32)
-      launch_skinny<bf16_t, true>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, stream);
+      launch_skinny<bf16_t, kEpiF32>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else if (dtype == kBF16)
-      launch_skinny<bf16_t, false>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, stream);
+      launch_skinny<bf16_t, kEpiAct>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else
       LYP_REQUIRE(false, "gemm: unknown dtype %d", dtype);
     LYP_LAUNCH_CHECK("gemm_skinny");
@@ -288,5 +324,48 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
   }
 #undef LYP_GEMM
   LYP_LAUNCH_CHECK("gemm_nt");
+  return 0;
+}
+
+// How many partial sums lyp_gemm_nt_parts would produce for this product; 0 if
+// it does not apply (then use lyp_gemm_nt).
+extern "C" int lyp_gemm_parts_hint(const void* A, const void* W, int dtype, int M, int N, int K, int lda, int ldw) {
+  if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 0;
+  const int slices = skinny_slices(N, K);
+  return slices > 1 ? slices : 0;
+}
+
+// parts[slice][M][N] (float) = partial sums of A . W^T over slices of the inner
+// dimension; their sum, in order, is the product.  `slices` must be what
+// lyp_gemm_parts_hint said.
+extern "C" int lyp_gemm_nt_parts(const void* A, const void* W, float* parts, int dtype, int slices, int M, int N,
+                                 int K, int lda, int ldw, hipStream_t stream) {
+  LYP_REQUIRE(skinny_ok(M, K, lda, ldw, A, W, dtype) && slices == skinny_slices(N, K) && slices > 1,
+              "gemm_parts: M=%d N=%d K=%d slices=%d is not a case for partial sums", M, N, K, slices);
+  if (dtype == kF32)
+    launch_skinny<float, kEpiParts>(static_cast<const float*>(A), static_cast<const float*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiParts>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
+  else
+    LYP_REQUIRE(false, "gemm_parts: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_parts");
+  return 0;
+}
+
+// out[M, N/2] = silu(gate) * up where W's rows come in tiles of 16: eight gate
+// features, then the eight up features that go with them.  Returns 1 (and does
+// nothing) when the few-rows kernel does not apply: then run lyp_gemm_nt and
+// lyp_swiglu with the same interleave.
+extern "C" int lyp_gemm_swiglu(const void* A, const void* W, void* out, int dtype, int M, int N, int K, int lda,
+                               int ldw, int ldo, hipStream_t stream) {
+  LYP_REQUIRE(N % 16 == 0 && ldo >= N / 2, "gemm_swiglu: %d rows of weights, output stride %d", N, ldo);
+  if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
+  if (dtype == kF32)
+    launch_skinny<float, kEpiSwiglu>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiSwiglu>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
+  else
+    LYP_REQUIRE(false, "gemm_swiglu: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_swiglu");
   return 0;
 }

@@ -43,12 +43,17 @@ def core() -> ctypes.CDLL:
         lib = _load(build.core_library())
         lib.lyp_last_error.restype = ctypes.c_char_p
         lib.lyp_embedding.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
-        lib.lyp_rmsnorm.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int,
-                                    c_float, c_void_p]
+        lib.lyp_rmsnorm.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_int, c_void_p,
+                                    c_int, c_int, c_float, c_void_p]
         lib.lyp_rmsnorm_act.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
         lib.lyp_rope_kv_write.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
-        lib.lyp_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]
+        lib.lyp_swiglu.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_gemm_parts_hint.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int]
+        lib.lyp_gemm_nt_parts.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, c_void_p]
+        lib.lyp_gemm_swiglu.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_int, c_void_p]
         lib.lyp_cast.argtypes = [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p]
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
@@ -127,22 +132,29 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torc
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, delta: torch.Tensor | None = None,
             rows: torch.Tensor | None = None) -> torch.Tensor:
     """out = rmsnorm(h [+ delta]) * weight.  h is the float residual stream and
-    takes the sum, unless ``rows`` picks the rows to norm."""
+    takes the sum, unless ``rows`` picks the rows to norm.  ``delta`` is [T, H]
+    in out's dtype, or float partial sums [S, T, H] (see ``linear``)."""
     _dev(h, weight, out, delta, rows)
     H = h.shape[1]
     n = out.shape[0]
     if h.dtype != torch.float32 or weight.numel() != H or out.shape[1] != H:
         raise KernelError(f"rmsnorm: h {tuple(h.shape)} {h.dtype}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
-    if delta is not None and (delta.shape != h.shape or delta.dtype != out.dtype):
-        raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} {delta.dtype} against h {tuple(h.shape)}, out {out.dtype}")
+    parts, stride = 0, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            if delta.dtype != torch.float32 or tuple(delta.shape[1:]) != tuple(h.shape):
+                raise KernelError(f"rmsnorm: partial sums {tuple(delta.shape)} {delta.dtype} against h {tuple(h.shape)}")
+            parts, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+        elif delta.shape != h.shape or delta.dtype != out.dtype:
+            raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} {delta.dtype} against h {tuple(h.shape)}, out {out.dtype}")
     if rows is not None:
         if rows.dtype != torch.int32 or rows.numel() != n:
             raise KernelError("rmsnorm: rows must be int32, one per output row")
     elif n != h.shape[0]:
         raise KernelError("rmsnorm: output rows differ from input rows")
     lib = core()
-    _check(lib.lyp_rmsnorm(_p(h), _p(delta), _p(weight), _code(weight.dtype), _p(out), _code(out.dtype), _p(rows), n,
-                           H, float(eps), _stream()), lib)
+    _check(lib.lyp_rmsnorm(_p(h), _p(delta), parts, stride, _p(weight), _code(weight.dtype), _p(out), _code(out.dtype),
+                           _p(rows), n, H, float(eps), _stream()), lib)
     return out
 
 
@@ -186,15 +198,40 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Ten
                                  _stream()), lib)
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleave: int = 0) -> torch.Tensor:
+    """out = silu(gate) * up.  interleave 0: gate_up[:, :I] are the gates and
+    gate_up[:, I:] the ups; interleave 8: columns come in tiles of 16, eight
+    gates then the eight ups that go with them."""
     _dev(gate_up, out)
     T, I = out.shape
     if tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != out.dtype:
         raise KernelError(f"swiglu: {tuple(gate_up.shape)} -> {tuple(out.shape)}")
     lib = core()
-    _check(lib.lyp_swiglu(_p(gate_up), _p(out), _code(out.dtype), T, I, _stream()), lib)
+    _check(lib.lyp_swiglu(_p(gate_up), _p(out), _code(out.dtype), T, I, interleave, _stream()), lib)
     return out
+
+
+def linear_swiglu(x: torch.Tensor, w: torch.Tensor, interleave: int) -> torch.Tensor:
+    """silu(x @ Wgate.T) * (x @ Wup.T) for the fused matrix w [2 I, K] laid out
+    as ``swiglu`` describes.  With few rows and interleave 8 it is one kernel."""
+    I = w.shape[0] // 2
+    if w.dtype != x.dtype:
+        if w.dtype != torch.float32:
+            raise KernelError(f"linear_swiglu: weight {w.dtype} against activations {x.dtype}")
+        return cast(linear_swiglu(cast(x, torch.float32), w, interleave), x.dtype)
+    out = torch.empty((x.shape[0], I), dtype=x.dtype, device=x.device)
+    if interleave == 8 and x.shape[0] <= 64:
+        _dev(x, w)
+        lib = core()
+        rc = lib.lyp_gemm_swiglu(_p(x), _p(w), _p(out), _code(x.dtype), x.shape[0], w.shape[0], w.shape[1],
+                                 x.stride(0), w.stride(0), I, _stream())
+        if rc == 0:
+            return out
+        if rc < 0:
+            _check(rc, lib)
+    gate_up = torch.empty((x.shape[0], 2 * I), dtype=x.dtype, device=x.device)
+    gemm_nt(x, w, gate_up)
+    return swiglu(gate_up, out, interleave)
 
 
 def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -231,19 +268,47 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
+           may_split: bool = False) -> torch.Tensor:
     """x @ w.T for a projection weight [out_features, in_features].  A weight
-    kept in 32-bit is multiplied in 32-bit whatever the activations are."""
+    kept in 32-bit is multiplied in 32-bit whatever the activations are.
+
+    With ``may_split`` the result may come back as float partial sums
+    [S, rows, out_features] instead (few rows, few output features: the inner
+    dimension is then cut into S slices so that every compute unit has work);
+    ``rmsnorm`` takes such a delta and adds the slices up, ``sum_parts`` does it
+    for any other consumer."""
     out_dtype = out_dtype or x.dtype
     if w.dtype != x.dtype:
         if w.dtype != torch.float32:
             raise KernelError(f"linear: weight {w.dtype} against activations {x.dtype}")
         x = cast(x, torch.float32)
+    if may_split and x.shape[0] <= 64:
+        _dev(x, w)
+        lib = core()
+        M, K, N = x.shape[0], x.shape[1], w.shape[0]
+        slices = lib.lyp_gemm_parts_hint(_p(x), _p(w), _code(x.dtype), M, N, K, x.stride(0), w.stride(0))
+        if slices > 1:
+            parts = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+            _check(lib.lyp_gemm_nt_parts(_p(x), _p(w), _p(parts), _code(x.dtype), slices, M, N, K, x.stride(0),
+                                         w.stride(0), _stream()), lib)
+            return parts
     if out_dtype in (x.dtype, torch.float32):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
         return gemm_nt(x, w, out)
     out = torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
     return cast(gemm_nt(x, w, out), out_dtype)
+
+
+def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Add up the partial sums ``linear(..., may_split=True)`` may return."""
+    if parts.dim() == 2:
+        return parts if parts.dtype == dtype else cast(parts, dtype)
+    h = torch.zeros(parts.shape[1:], dtype=torch.float32, device=parts.device)
+    ones = torch.ones(parts.shape[2], dtype=torch.float32, device=parts.device)
+    out = torch.empty(parts.shape[1:], dtype=dtype, device=parts.device)
+    rmsnorm(h, ones, 0.0, out, delta=parts)     # the sum lands in h; the normed output is not what is wanted
+    return h if dtype == torch.float32 else cast(h, dtype)
 
 
 # ------------------------------------------------------------------- attention

@@ -77,7 +77,7 @@ class DecoderModel(Part):
         for prefix, part in self.named_parts():
             for ws in part.weight_specs():
                 full = tuple(WeightSource(prefix + s.name, tuple(s.shape)) for s in ws.sources)
-                out.append((part, WeightSpec(ws.attr, full, ws.init)))
+                out.append((part, WeightSpec(ws.attr, full, ws.init, ws.interleave)))
         return out
 
     def expected_tensors(self) -> dict:

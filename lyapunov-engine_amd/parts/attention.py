@@ -83,4 +83,4 @@ class PagedAttention(Mixer):
             part_ml = ctx.scratch("attn_part_ml", n * 2)
             ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.dec_seqs,
                             ctx.n_dec, part_o, part_ml, max_parts, **common)
-        return ops.linear(out, self.o_proj, out_dtype=ctx.dtype)
+        return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True)

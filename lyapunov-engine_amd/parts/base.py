@@ -12,7 +12,8 @@ Conventions every part may rely on:
   * the hidden state ``h`` is the float residual stream ``[T, hidden]``;
     a part's output ``y`` has the step's activation dtype (``ctx.dtype``) and is
     added to ``h`` by the *next* norm (``Norm.forward(ctx, h, delta=y)``), in
-    32-bit;
+    32-bit; ``y`` may also be float partial sums ``[S, T, hidden]`` (what
+    ``ops.linear(..., may_split=True)`` returns), which that norm adds up;
   * ``T`` is the number of tokens of the step, all requests' tokens flattened;
     request ``b`` owns rows ``q_start[b] .. q_start[b+1]``, in position order;
   * a part's result for a token may depend on earlier tokens of the same request
@@ -41,6 +42,7 @@ class WeightSpec:
     attr: str
     sources: tuple         # of WeightSource
     init: str = "normal"   # random-weights mode: "normal" (0, std) or "ones" (1 + noise)
+    interleave: int = 0    # n > 0: rows alternate between the sources in runs of n (n of the first, n of the second, ...)
 
     @property
     def shape(self) -> tuple:

@@ -20,18 +20,21 @@ from .base import FeedForward, StepContext, WeightSource, WeightSpec
 class SwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        # Rows of the fused matrix in tiles of 16 (eight gates, their eight ups) let a
+        # decode step gate inside the product; widths that are no multiple of 8 keep
+        # the plain order, gates first.
+        self.interleave = 8 if intermediate_size % 8 == 0 else 0
         self.gate_up_proj: Optional[torch.Tensor] = None
         self.down_proj: Optional[torch.Tensor] = None
 
     def weight_specs(self):
         shape = (self.intermediate_size, self.hidden_size)
         return [
-            WeightSpec("gate_up_proj", (WeightSource("gate_proj.weight", shape), WeightSource("up_proj.weight", shape))),
+            WeightSpec("gate_up_proj", (WeightSource("gate_proj.weight", shape), WeightSource("up_proj.weight", shape)),
+                       interleave=self.interleave),
             WeightSpec("down_proj", (WeightSource("down_proj.weight", (self.hidden_size, self.intermediate_size)),)),
         ]
 
     def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
-        gate_up = ops.linear(x, self.gate_up_proj, out_dtype=ctx.dtype)
-        act = torch.empty((x.shape[0], self.intermediate_size), dtype=ctx.dtype, device=x.device)
-        ops.swiglu(gate_up, act)
-        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype)
+        act = ops.linear_swiglu(x, self.gate_up_proj, self.interleave)
+        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype, may_split=True)

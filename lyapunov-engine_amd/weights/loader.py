@@ -104,6 +104,12 @@ def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, 
         keep = torch.float32 if torch.float32 in kinds else kinds.pop()
         pieces = [p.to(device=device, dtype=keep, non_blocking=False) for p in pieces]
         t = pieces[0] if len(pieces) == 1 else torch.cat(pieces, dim=0)
+        if ws.interleave:
+            n, k = ws.interleave, len(pieces)
+            rows = pieces[0].shape[0]
+            if any(p.shape != pieces[0].shape for p in pieces) or rows % n:
+                raise WeightError(f"{ws.attr}: rows of {[tuple(p.shape) for p in pieces]} cannot alternate in runs of {n}")
+            t = t.view(k, rows // n, n, *t.shape[1:]).transpose(0, 1).reshape(t.shape)
         setattr(owner, ws.attr, t.contiguous())
     model.materialize(device, dtype)
     return model

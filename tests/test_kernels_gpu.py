@@ -86,6 +86,54 @@ def test_swiglu(ops, dtype, I, T):
     torch.testing.assert_close(out.cpu().double(), P.swiglu(gu.double()), **tol(dtype, 1e-5, 1e-2))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_in_tiles_and_inside_the_product(ops, dtype):
+    """Gates and ups in tiles of 16 columns, and the few-rows product that gates
+    in its epilogue, against the plain gate-first formula."""
+    I, K = 48, 128
+    g = torch.Generator().manual_seed(2)
+    wg, wu = (torch.randn(I, K, generator=g) * 0.1).to(dtype), (torch.randn(I, K, generator=g) * 0.1).to(dtype)
+    w = torch.stack([wg.view(-1, 8, K), wu.view(-1, 8, K)], dim=1).reshape(2 * I, K).contiguous()
+    for M in (1, 7, 33, 64, 70):
+        x = (torch.randn(M, K, generator=g)).to(dtype)
+        want = P.mlp(x.double(), wg.double(), wu.double(), torch.eye(I, dtype=torch.float64))
+        got = ops.linear_swiglu(x.to(DEV), w.to(DEV), 8)
+        torch.testing.assert_close(got.cpu().double(), want, **tol(dtype, 1e-5, 2e-2))
+    gu = rnd(5, 2 * I, dtype=dtype, seed=3)
+    out = torch.empty(5, I, dtype=dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out, 8)
+    tiles = gu.double().view(5, -1, 2, 8)
+    want = torch.nn.functional.silu(tiles[:, :, 0]) * tiles[:, :, 1]
+    torch.testing.assert_close(out.cpu().double(), want.reshape(5, I), **tol(dtype, 1e-5, 1e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (33, 96, 1024), (64, 515, 4096), (5, 4096, 2048)])
+def test_linear_partial_sums(ops, dtype, M, N, K):
+    """A product that comes back in slices of the inner dimension: the slices add
+    up to the product, through sum_parts and through the norm's residual add."""
+    a, w = rnd(M, K, dtype=dtype, seed=21), rnd(N, K, dtype=dtype, scale=0.05, seed=22)
+    want = a.double() @ w.double().T
+    bound = a.double().abs() @ w.double().abs().T
+    y = ops.linear(a.to(DEV), w.to(DEV), may_split=True)
+    rel = 2e-6 if dtype == torch.float32 else 1e-5
+    if y.dim() == 3:
+        assert y.dtype == torch.float32 and y.shape[1:] == (M, N) and y.shape[0] > 1
+        assert ((y.cpu().double().sum(0) - want).abs() <= rel * bound + 1e-30).all()
+        total = ops.sum_parts(y, torch.float32)
+        assert ((total.cpu().double() - want).abs() <= rel * bound + 1e-30).all()
+        h = rnd(M, N, seed=23).to(DEV)
+        h0 = h.clone()
+        out = torch.empty(M, N, dtype=dtype, device=DEV)
+        ops.rmsnorm(h, torch.ones(N, dtype=dtype, device=DEV), 1e-5, out, delta=y)
+        assert (((h - h0).cpu().double() - want).abs() <= rel * bound + 1e-5).all()
+        torch.testing.assert_close(out.cpu().double(), P.rms_norm(h.cpu().double(), torch.ones(N, dtype=torch.float64), 1e-5),
+                                   **tol(dtype, 1e-5, 1e-2))
+    else:
+        assert N >= 4096 or K < 1024  # only products with few output features and a long inner dimension are sliced
+        assert ((y.cpu().double() - want).abs() <= (1e-2 if dtype == torch.bfloat16 else rel) * bound + 1e-30).all()
+
+
 # ------------------------------------------------------------------------ gemm
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 172, 96), (33, 256, 172), (130, 1000, 200), (200, 513, 96),

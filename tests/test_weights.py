@@ -90,9 +90,14 @@ def test_folder_round_trip_and_fusing(tmp_path):
         att, ffn = model.layers[1].mixer, model.layers[1].ffn
         want_qkv = torch.cat([f.tensor(p + f"self_attn.{n}_proj.weight").float() for n in "qkv"], 0)
         assert torch.equal(att.qkv_proj, want_qkv)                 # q, k, v rows in this order
-        want_gu = torch.cat([f.tensor(p + "mlp.gate_proj.weight").float(), f.tensor(p + "mlp.up_proj.weight").float()], 0)
-        assert torch.equal(ffn.gate_up_proj, want_gu)              # gate rows first (weight_loader.py:155-163)
+        gate, up = f.tensor(p + "mlp.gate_proj.weight").float(), f.tensor(p + "mlp.up_proj.weight").float()
         assert ffn.gate_up_proj.shape == (2 * cfg.intermediate_size, cfg.hidden_size)
+        if ffn.interleave:                                          # tiles of 16 rows: eight gates, their eight ups
+            tiles = ffn.gate_up_proj.view(-1, 2, 8, cfg.hidden_size)
+            assert torch.equal(tiles[:, 0].reshape(gate.shape), gate) and torch.equal(tiles[:, 1].reshape(up.shape), up)
+        else:                                                       # gate rows first (weight_loader.py:155-163)
+            assert torch.equal(ffn.gate_up_proj, torch.cat([gate, up], 0))
+        assert bool(ffn.interleave) == (cfg.intermediate_size % 8 == 0)
         assert torch.equal(model.layers[1].norm2.weight, f.tensor(p + "post_attention_layernorm.weight").float())
         if cfg.tie_word_embeddings:
             assert model.lm_head is model.embed                     # one matrix, two uses
