@@ -42,7 +42,7 @@ constexpr int HD = LYP_HEAD_DIM;
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16, at most 256");
 constexpr int kSteps = HD / 16;     // matrix steps over the head dimension; also 16-row blocks of it
 constexpr int kSlice = HD / 4;      // contiguous run of the head dimension one lane group loads
-constexpr int kPartKeys = 64;       // keys per decode partition
+constexpr int kPartKeys = 64;       // a wave's share of a decode partition is a multiple of this
 constexpr float kLog2e = 1.4426950408889634f;
 
 template <typename T>
@@ -165,33 +165,42 @@ struct Softmax {
   float lsum;  // this lane group's part of the running sum
 };
 
+// 2^x by the hardware instruction alone: arguments here are at most 0 and
+// results below the normal range may be flushed.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // Take the scores of one 16-key block (s: rows = keys kb0 + 4 (l / 16) + i,
 // column = l % 16), update the running state, rescale the output accumulator
 // and return the probabilities as the column operand of the P.V product.
 // `pos` is the column's absolute position; a key is visible when
-// key <= pos and (window == 0 or key > pos - window).
-template <typename T>
+// key <= pos and (window == 0 or key > pos - window).  With MASKED false every
+// key of the block is visible to every column and the tests are skipped.
+template <typename T, bool MASKED = true>
 __device__ __forceinline__ Frag<T> softmax_block(f32x4 s, float scale_log2, int kb0, int pos, int window,
                                                  int hi, Softmax& st, f32x4 (&o)[kSteps], int lane) {
   float sv[4];
   float mx = LYP_NEG_INF;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int key = kb0 + 4 * (lane / 16) + i;
-    const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
-    sv[i] = vis ? s[i] * scale_log2 : LYP_NEG_INF;
+    if constexpr (MASKED) {
+      const int key = kb0 + 4 * (lane / 16) + i;
+      const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
+      sv[i] = vis ? s[i] * scale_log2 : LYP_NEG_INF;
+    } else {
+      sv[i] = s[i] * scale_log2;
+    }
     mx = fmaxf(mx, sv[i]);
   }
   mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
   mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
   const float m_new = fmaxf(st.m, mx);
   const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
-  const float alpha = exp2f(st.m - m_safe);  // 0 while nothing has been seen yet
+  const float alpha = fast_exp2(st.m - m_safe);  // 0 while nothing has been seen yet
   float psum = 0.f;
   Frag<T> pf;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float p = exp2f(sv[i] - m_safe);
+    const float p = fast_exp2(sv[i] - m_safe);
     psum += p;
     pf[i] = from_f32<T>(p);
   }
@@ -295,26 +304,48 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
 // ---------------------------------------------------------------------- decode
 // grid (partitions, nkv * column_groups, requests); kDecodeWaves waves.  A
-// workgroup takes one partition of kDecodeWaves * 64 keys, 64 per wave, and
-// merges its waves' results through LDS, in a fixed order.  Column c of the tile
-// is query head kvh * g + 16 * column_group + c of the request's one new token.
+// workgroup takes one partition of kDecodeWaves * keys_per_wave keys and merges
+// its waves' results through LDS, in a fixed order.  Column c of the tile is
+// query head kvh * g + 16 * column_group + c of the request's one new token.
+// How many keys a wave takes is the launch's choice (lyp_attn_decode_plan): few
+// when there is little work, so that it spreads over the chip; many when there
+// is a lot, so that the fixed cost of a workgroup is paid less often.
 // Partials: part_o [request][head][part][hd] (not normalised), part_ml
 // [request][head][part][2] = (maximum in the base-2 domain, sum).
 constexpr int kDecodeWaves = HD <= 128 ? 4 : 2;
-constexpr int kBlockKeys = kDecodeWaves * kPartKeys;
+constexpr int kDecodeDepth = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // 16-key blocks in flight per wave
+
+// One 16-key block of keys and values.  FULL: the page size is a multiple of 16
+// and every key of the block is inside the request and visible, so the block
+// lies in one page (`page`, the same for the whole wave), nothing is masked and
+// the addresses are a wave-wide base plus a constant per lane.
+template <typename T>
+__device__ __forceinline__ void load_block_full(Frag<T> (&kf)[kSteps], Frag<T> (&vf)[kSteps], const PagedKV& kv,
+                                                int kb0, int page, int lane) {
+  const int off = kb0 % kv.bs;
+  const size_t head = static_cast<size_t>(page) * kv.nkv + kv.kvh;
+  const T* krow = static_cast<const T*>(kv.kpool) + (head * kv.bs + off) * HD + (lane % 16) * HD + (lane / 16) * kSlice;
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) kf[s] = *reinterpret_cast<const Frag<T>*>(krow + 4 * s);
+  const T* vrow = static_cast<const T*>(kv.vpool) + head * HD * kv.bs + off + (lane % 16) * kv.bs + 4 * (lane / 16);
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db)
+    vf[db] = *reinterpret_cast<const Frag<T>*>(vrow + static_cast<size_t>(db) * 16 * kv.bs);
+}
 
 template <typename T>
 __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const T* __restrict__ q, int q_stride, const void* kpool, const void* vpool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ dec_seqs,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int nh, int nkv, int bs,
-    int window, float scale_log2) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int keys_per_wave, int nh, int nkv,
+    int bs, int window, float scale_log2) {
   __shared__ float s_o[kDecodeWaves][16][HD];
   __shared__ float s_m[kDecodeWaves][16];
   __shared__ float s_l[kDecodeWaves][16];
 
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // the same in every lane: keeps what follows scalar
   const int g = nh / nkv;
   const int col_groups = (g + 15) / 16;
   const int kvh = blockIdx.y / col_groups;
@@ -322,22 +353,11 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int slot = blockIdx.z;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const int part = blockIdx.x;
-  constexpr int kBlocks = kPartKeys / 16;  // 16-key blocks per wave
-  const int k_begin = part * kBlockKeys + wave * kPartKeys;
-
-  // Table entries of the wave's keys, read before the request's length is
-  // known, so that they travel together with it.
-  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
-  int page_k[kBlocks], page_v[kBlocks];
-#pragma unroll
-  for (int it = 0; it < kBlocks; ++it) {
-    page_k[it] = page_of(kv, k_begin + 16 * it + lane % 16);
-    page_v[it] = page_of(kv, k_begin + 16 * it + 4 * (lane / 16));
-  }
+  const int block_keys = kDecodeWaves * keys_per_wave;
   const int ctx = ctx_len[seq];
   const int pos = ctx - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  if (part * kBlockKeys >= ctx || (part + 1) * kBlockKeys <= lo) return;  // the whole workgroup
+  if (part * block_keys >= ctx || (part + 1) * block_keys <= lo) return;  // the whole workgroup
 
   const int col = lane % 16;
   const bool col_valid = h0 + col < g;
@@ -351,32 +371,46 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   Softmax st{LYP_NEG_INF, 0.f};
 
-  const int k_end = min(ctx, k_begin + kPartKeys);
-  if (k_begin < k_end && k_end > lo) {
-    // Blocks are loaded a group at a time, the whole group in flight at once;
-    // the group is as large as the register file allows for this head size.
-    constexpr int kGroup = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
+  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
+  const bool aligned = bs % 16 == 0;
+  const int k_begin = part * block_keys + wave * keys_per_wave;
+  const int k_first = max(k_begin, (lo / 16) * 16);
+  const int k_end = min(ctx, k_begin + keys_per_wave);
+
+  Frag<T> kf[kDecodeDepth][kSteps], vf[kDecodeDepth][kSteps];
+  auto is_full = [&](int kb0) { return aligned && kb0 >= lo && kb0 + 16 <= ctx; };
+  auto load = [&](int u, int kb0) {
+    if (is_full(kb0)) {
+      load_block_full<T>(kf[u], vf[u], kv, kb0, kv.table[kb0 / bs], lane);
+    } else {
+      load_k<T>(kf[u], kv, kb0, lo, ctx, lane);
+      load_v<T>(vf[u], kv, kb0, lo, ctx, lane);
+    }
+  };
+  auto compute = [&](int u, int kb0) {
+    f32x4 s{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int g0 = 0; g0 < kBlocks; g0 += kGroup) {
-      if (k_begin + 16 * g0 >= k_end) break;
-      Frag<T> kf[kGroup][kSteps], vf[kGroup][kSteps];
+    for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[u][k], qf[k], s);
+    Frag<T> pf;
+    if (is_full(kb0)) pf = softmax_block<T, false>(s, scale_log2, kb0, pos, window, ctx, st, o, lane);
+    else pf = softmax_block<T, true>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
 #pragma unroll
-      for (int u = 0; u < kGroup; ++u) {
-        const int kb0 = k_begin + 16 * (g0 + u);
-        load_k_page<T>(kf[u], kv, kb0, lo, ctx, lane, page_k[g0 + u]);
-        load_v_page<T>(vf[u], kv, kb0, lo, ctx, lane, page_v[g0 + u]);
-      }
+    for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf, o[db]);
+  };
+
+  // kDecodeDepth blocks are on their way at any time: a buffer is refilled for
+  // the block kDecodeDepth ahead as soon as its block has been used.
 #pragma unroll
-      for (int u = 0; u < kGroup; ++u) {
-        const int kb0 = k_begin + 16 * (g0 + u);
-        if (kb0 < k_end && kb0 + 16 > lo) {
-          f32x4 s{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < kDecodeDepth; ++u)
+    if (k_first + 16 * u < k_end) load(u, k_first + 16 * u);
+  for (int kb0 = k_first; kb0 < k_end; kb0 += 16 * kDecodeDepth) {
 #pragma unroll
-          for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[u][k], qf[k], s);
-          const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
-#pragma unroll
-          for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf, o[db]);
-        }
+    for (int u = 0; u < kDecodeDepth; ++u) {
+      const int cur = kb0 + 16 * u;
+      if (cur < k_end) {
+        compute(u, cur);
+        const int next = cur + 16 * kDecodeDepth;
+        if (next < k_end) load(u, next);
       }
     }
   }
@@ -386,7 +420,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int db = 0; db < kSteps; ++db)
     *reinterpret_cast<f32x4*>(&s_o[wave][col][db * 16 + 4 * (lane / 16)]) = o[db];
   if (lane < 16) {
-    s_m[wave][col] = st.m;
+    s_m[wave][col] = col_valid ? st.m : LYP_NEG_INF;
     s_l[wave][col] = l;
   }
   __syncthreads();
@@ -402,7 +436,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
 #pragma unroll
       for (int w = 0; w < kDecodeWaves; ++w) {
         if (s_m[w][c] == LYP_NEG_INF) continue;
-        const float wgt = exp2f(s_m[w][c] - m);
+        const float wgt = fast_exp2(s_m[w][c] - m);
         acc += wgt * s_o[w][c][d];
         lsum += wgt * s_l[w][c];
       }
@@ -422,13 +456,14 @@ template <typename T>
 __global__ __launch_bounds__(64) void attn_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, int max_parts,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ dec_seqs, T* __restrict__ out, int out_stride, int nh, int window) {
+    const int32_t* __restrict__ dec_seqs, T* __restrict__ out, int out_stride, int nh, int window,
+    int block_keys) {
   const int head = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const int ctx = ctx_len[seq];
   const int lo = window > 0 ? max(0, ctx - window) : 0;
-  const int p_lo = lo / kBlockKeys;
-  const int p_hi = (ctx + kBlockKeys - 1) / kBlockKeys;
+  const int p_lo = lo / block_keys;
+  const int p_hi = (ctx + block_keys - 1) / block_keys;
   const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
   const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
 
@@ -437,7 +472,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   m = wave_max(m);
   const float m_safe = m == LYP_NEG_INF ? 0.f : m;
   float l = 0.f;
-  for (int p = p_lo + lane; p < p_hi; p += kWave) l += exp2f(ml[p].x - m_safe) * ml[p].y;
+  for (int p = p_lo + lane; p < p_hi; p += kWave) l += fast_exp2(ml[p].x - m_safe) * ml[p].y;
   l = wave_sum(l);
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 
@@ -445,7 +480,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   for (int d = lane; d < HD; d += kWave) {
     float acc = 0.f;
 #pragma unroll 4
-    for (int p = p_lo; p < p_hi; ++p) acc += exp2f(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+    for (int p = p_lo; p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
     orow[d] = from_f32<T>(acc * inv);
   }
 }
@@ -467,7 +502,26 @@ using namespace lyp;
 extern "C" {
 
 int lyp_attn_head_dim() { return HD; }
-int lyp_attn_part_keys() { return kBlockKeys; }
+// Keys per workgroup for a decode launch over n_seqs requests whose longest
+// context is max_ctx.  Both are rounded up to powers of two first, so that a
+// captured launch (sized for a bucket) and a direct one choose alike.
+int lyp_attn_decode_plan(int n_seqs, int max_ctx, int nh, int nkv) {
+  auto pow2 = [](int v, int least) {
+    int p = least;
+    while (p < v) p *= 2;
+    return p;
+  };
+  const int B = pow2(n_seqs, 1), C = pow2(max_ctx, 256);
+  const int g = nh / (nkv > 0 ? nkv : 1);
+  const long long base = static_cast<long long>(B) * nkv * ((g + 15) / 16);
+  int kpw = kPartKeys;
+  while (kpw < 1024) {
+    const int next_block = kDecodeWaves * kpw * 2;
+    if (base * ((C + next_block - 1) / next_block) < 512) break;
+    kpw *= 2;
+  }
+  return kDecodeWaves * kpw;
+}
 
 int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
                      const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
@@ -507,13 +561,17 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   return 0;
 }
 
-// part_o needs n_seqs * nh * max_parts * hd floats, part_ml n_seqs * nh *
-// max_parts * 2, with max_parts >= ceil(longest context / lyp_attn_part_keys()).
+// part_keys: keys per workgroup, from lyp_attn_decode_plan.  part_o needs
+// n_seqs * nh * max_parts * hd floats, part_ml n_seqs * nh * max_parts * 2, with
+// max_parts >= ceil(longest context / part_keys).
 int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
                     const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                     const int32_t* q_start, const int32_t* ctx_len, const int32_t* dec_seqs, int n_seqs,
-                    float* part_o, float* part_ml, int max_parts, int nh, int nkv, int bs, int window,
-                    float scale, hipStream_t stream) {
+                    float* part_o, float* part_ml, int max_parts, int part_keys, int nh, int nkv, int bs,
+                    int window, float scale, hipStream_t stream) {
+  LYP_REQUIRE(part_keys > 0 && part_keys % (kDecodeWaves * kPartKeys) == 0,
+              "attn_decode: %d keys per workgroup is no multiple of %d", part_keys, kDecodeWaves * kPartKeys);
+  const int keys_per_wave = part_keys / kDecodeWaves;
   if (check_common("attn_decode", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
   LYP_REQUIRE(n_seqs >= 0 && max_parts > 0, "attn_decode: %d requests, %d partitions", n_seqs, max_parts);
   LYP_REQUIRE(part_o && part_ml, "attn_decode: no workspace");
@@ -527,17 +585,17 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
   if (dtype == kF32) {
     attn_decode_kernel<float><<<grid, kDecodeWaves * kWave, 0, stream>>>(
         static_cast<const float*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
-        dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
+        dec_seqs, part_o, part_ml, max_parts, keys_per_wave, nh, nkv, bs, window, scale_log2);
     attn_combine_kernel<float><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,
                                                          dec_seqs, static_cast<float*>(out), out_stride, nh,
-                                                         window);
+                                                         window, part_keys);
   } else if (dtype == kBF16) {
     attn_decode_kernel<bf16_t><<<grid, kDecodeWaves * kWave, 0, stream>>>(
         static_cast<const bf16_t*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,
-        dec_seqs, part_o, part_ml, max_parts, nh, nkv, bs, window, scale_log2);
+        dec_seqs, part_o, part_ml, max_parts, keys_per_wave, nh, nkv, bs, window, scale_log2);
     attn_combine_kernel<bf16_t><<<cgrid, 64, 0, stream>>>(part_o, part_ml, max_parts, q_start, ctx_len,
                                                           dec_seqs, static_cast<bf16_t*>(out), out_stride,
-                                                          nh, window);
+                                                          nh, window, part_keys);
   } else {
     LYP_REQUIRE(false, "attn_decode: unknown dtype %d", dtype);
   }

@@ -75,7 +75,8 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
                                          c_float, c_void_p]
         lib.lyp_attn_decode.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                        c_int, c_int, c_float, c_void_p]
+                                        c_int, c_int, c_int, c_float, c_void_p]
+        lib.lyp_attn_decode_plan.argtypes = [c_int, c_int, c_int, c_int]
         _attn[head_dim] = lib
     return lib
 
@@ -312,8 +313,9 @@ def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------- attention
-def attn_part_keys(head_dim: int) -> int:
-    return attention_lib(head_dim).lyp_attn_part_keys()
+def attn_decode_plan(n_seqs: int, max_ctx: int, num_heads: int, num_kv_heads: int, head_dim: int) -> int:
+    """Keys per workgroup (the partition size) for a decode launch of this size."""
+    return attention_lib(head_dim).lyp_attn_decode_plan(n_seqs, max_ctx, num_heads, num_kv_heads)
 
 
 def _attn_check(q, out, kpool, vpool, block_tables, nh, nkv, hd):
@@ -352,7 +354,7 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
 def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
                 block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                 dec_seqs: torch.Tensor | None, n_seqs: int, part_o: torch.Tensor, part_ml: torch.Tensor,
-                max_parts: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
+                max_parts: int, part_keys: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
                 scale: float | None = None) -> torch.Tensor:
     """Attention of requests that bring one new token each, split over
     partitions of the context and merged."""
@@ -368,8 +370,8 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
     scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
     _check(lib.lyp_attn_decode(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
                                _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(dec_seqs),
-                               n_seqs, _p(part_o), _p(part_ml), max_parts, num_heads, num_kv_heads, bs, window,
-                               scale, _stream()), lib)
+                               n_seqs, _p(part_o), _p(part_ml), max_parts, part_keys, num_heads, num_kv_heads, bs,
+                               window, scale, _stream()), lib)
     return out
 
 

@@ -76,11 +76,11 @@ class PagedAttention(Mixer):
             ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.tile_seq,
                              ctx.tile_q0, ctx.n_tiles, **common)
         if ctx.n_dec:
-            part = ops.attn_part_keys(self.head_dim)
+            part = ops.attn_decode_plan(ctx.n_dec, ctx.max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
             max_parts = max(1, (ctx.max_ctx_dec + part - 1) // part)
             n = ctx.n_dec * self.num_heads * max_parts
             part_o = ctx.scratch("attn_part_o", n * self.head_dim)
             part_ml = ctx.scratch("attn_part_ml", n * 2)
             ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.dec_seqs,
-                            ctx.n_dec, part_o, part_ml, max_parts, **common)
+                            ctx.n_dec, part_o, part_ml, max_parts, part, **common)
         return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True)

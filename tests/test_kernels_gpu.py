@@ -297,7 +297,7 @@ def test_attention_decode(ops, dtype, case):
     seqs = [(c, 1) for c in ctxs]
     s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=hd + bs + 1)
     n = len(seqs)
-    part = ops.attn_part_keys(hd)
+    part = ops.attn_decode_plan(n, max(ctxs), nh, nkv, hd)
     max_parts = -(-max(ctxs) // part)
     part_o = torch.full((n * nh * max_parts * hd,), float("nan"), device=DEV)
     part_ml = torch.full((n * nh * max_parts * 2,), float("nan"), device=DEV)
@@ -306,7 +306,7 @@ def test_attention_decode(ops, dtype, case):
     order = list(reversed(range(n)))
     ops.attn_decode(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
                     s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(order, dtype=torch.int32, device=DEV), n,
-                    part_o, part_ml, max_parts, num_heads=nh, num_kv_heads=nkv, head_dim=hd, window=window)
+                    part_o, part_ml, max_parts, part, num_heads=nh, num_kv_heads=nkv, head_dim=hd, window=window)
     want = plain_attention(s, seqs, window)
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
 
@@ -332,9 +332,10 @@ def test_attention_finds_one_far_key(ops, dtype, kind):
             s["ctx_len"].to(DEV))
     kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd)
     if kind == "decode":
-        mp = -(-ctx // ops.attn_part_keys(hd))
+        part = ops.attn_decode_plan(1, ctx, nh, nkv, hd)
+        mp = -(-ctx // part)
         ops.attn_decode(*args, None, 1, torch.empty(nh * mp * hd, device=DEV), torch.empty(nh * mp * 2, device=DEV),
-                        mp, **kw)
+                        mp, part, **kw)
     else:
         ops.attn_prefill(*args, torch.zeros(1, dtype=torch.int32, device=DEV),
                          torch.zeros(1, dtype=torch.int32, device=DEV), 1, **kw)
