@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch
@@ -246,6 +247,14 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------------ GEMM
+# Large bfloat16 products go to the vendor's matrix library (through torch), as
+# the reference's projections go to cuBLAS (nn.Linear, models/llama.py:45-48,
+# 112-117, 177).  Products with few rows (decode steps), every float product
+# (true 32-bit) and everything when LYAPUNOV_AMD_GEMM=own use the kernels here.
+LIBRARY_GEMM = os.environ.get("LYAPUNOV_AMD_GEMM", "library") != "own"
+LIBRARY_GEMM_MIN_ROWS = 65
+
+
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
     """out = a @ w.T (or out += ...).  a [M, K], w [N, K] of one dtype; out
     [M, N] of that dtype or float."""
@@ -254,6 +263,9 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
     N = w.shape[0]
     if w.shape[1] != K or tuple(out.shape) != (M, N) or a.dtype != w.dtype:
         raise KernelError(f"gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
+    if LIBRARY_GEMM and a.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and not accumulate \
+            and M >= LIBRARY_GEMM_MIN_ROWS:
+        return torch.matmul(a, w.t(), out=out)
     if accumulate:
         if out.dtype != torch.float32:
             raise KernelError("gemm: accumulation needs a float output")
