@@ -2,8 +2,9 @@
 // size (LYP_HEAD_DIM, a multiple of 16) and both element types.
 //
 // Two kernels share the fragment loaders and the online softmax:
-//   * attn_prefill: a wave takes 16 query tokens of one request and up to four
-//     query heads of one key/value head, and walks the keys the tokens may see.
+//   * attn_prefill: a workgroup takes a run of new tokens of one request and up
+//     to four query heads of one key/value head; the keys and values they may
+//     see pass through LDS, shared by its waves (a wave: one head, 16 tokens).
 //   * attn_decode:  a wave takes one request's single new token, all query
 //     heads of one key/value head (as the 16 columns of the tile), and 64 keys
 //     of the context; a workgroup merges its waves, attn_combine the workgroups.
@@ -34,6 +35,13 @@
 
 #ifndef LYP_HEAD_DIM
 #error "compile with -DLYP_HEAD_DIM=<multiple of 16>"
+#endif
+#ifndef LYP_PREFILL_QB   // 16-token blocks per wave when a workgroup takes four heads
+#if LYP_HEAD_DIM <= 64
+#define LYP_PREFILL_QB 2
+#else
+#define LYP_PREFILL_QB 1
+#endif
 #endif
 
 namespace lyp {
@@ -213,107 +221,55 @@ __device__ __forceinline__ Frag<T> softmax_block(f32x4 s, float scale_log2, int 
   return pf;
 }
 
+// The same for NB consecutive 16-key blocks at once (s[u]: block kb0 + 16 u):
+// one maximum, one rescaling of the accumulator and one pass of exponentials
+// for all of them, which is most of the arithmetic outside the matrix cores.
+template <typename T, bool MASKED, int NB>
+__device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf)[NB], float scale_log2, int kb0,
+                                              int pos, int window, int hi, Softmax& st, f32x4 (&o)[kSteps],
+                                              int lane) {
+  float sv[NB][4];
+  float mx = LYP_NEG_INF;
+#pragma unroll
+  for (int u = 0; u < NB; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (MASKED) {
+        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
+        const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
+        sv[u][i] = vis ? s[u][i] * scale_log2 : LYP_NEG_INF;
+      } else {
+        sv[u][i] = s[u][i] * scale_log2;
+      }
+      mx = fmaxf(mx, sv[u][i]);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  const float m_new = fmaxf(st.m, mx);
+  const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
+  const float alpha = fast_exp2(st.m - m_safe);
+  float psum = 0.f;
+#pragma unroll
+  for (int u = 0; u < NB; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = fast_exp2(sv[u][i] - m_safe);
+      psum += p;
+      pf[u][i] = from_f32<T>(p);
+    }
+  st.lsum = st.lsum * alpha + psum;
+  st.m = m_new;
+#pragma unroll
+  for (int db = 0; db < kSteps; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+}
+
 __device__ __forceinline__ float lane_groups_sum(float v) {
   v += __shfl_xor(v, 16, kWave);
   v += __shfl_xor(v, 32, kWave);
   return v;
 }
-
-// --------------------------------------------------------------------- prefill
-// grid (tiles, nkv * head_groups); 256 threads.  tile -> (request, first new
-// token of the tile); wave w takes tokens 16 w .. 16 w + 15 of the tile.
-template <typename T, int NCB>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
-    const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const void* kpool,
-    const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int nh, int nkv, int bs,
-    int window, float scale_log2) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int g = nh / nkv;
-  const int head_groups = (g + NCB - 1) / NCB;
-  const int kvh = blockIdx.y / head_groups;
-  const int hsub = (blockIdx.y % head_groups) * NCB;  // first head of the group taken here
-
-  const int seq = tile_seq[blockIdx.x];
-  const int tok0 = q_start[seq];
-  const int q_len = q_start[seq + 1] - tok0;
-  const int ctx = ctx_len[seq];
-  const int qi0 = tile_q0[blockIdx.x] + 16 * wave;  // the wave's first new token
-  if (qi0 >= q_len) return;
-  const int n_valid = min(16, q_len - qi0);
-  const int pos0 = ctx - q_len + qi0;  // absolute position of that token
-  const int pos_last = pos0 + n_valid - 1;
-
-  const int col = lane % 16;
-  const bool col_valid = col < n_valid;
-  const int pos = pos0 + col;
-  const size_t token = static_cast<size_t>(tok0) + qi0 + col;
-
-  Frag<T> qf[NCB][kSteps];
-  f32x4 o[NCB][kSteps];
-  Softmax st[NCB];
-#pragma unroll
-  for (int cb = 0; cb < NCB; ++cb) {
-    const int hh = hsub + cb;
-    const bool valid = col_valid && hh < g;
-    const T* row = q + token * q_stride + static_cast<size_t>(kvh * g + (hh < g ? hh : 0)) * HD;
-    load_q<T>(qf[cb], row, valid, lane);
-    st[cb].m = LYP_NEG_INF;
-    st[cb].lsum = 0.f;
-#pragma unroll
-    for (int db = 0; db < kSteps; ++db) o[cb][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
-  const int lo = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int hi = pos_last + 1;  // keys at or above it are invisible to every token of the wave
-
-  for (int kb0 = (lo / 16) * 16; kb0 < hi; kb0 += 16) {
-    Frag<T> kf[kSteps], vf[kSteps];
-    load_k<T>(kf, kv, kb0, lo, hi, lane);
-    load_v<T>(vf, kv, kb0, lo, hi, lane);
-#pragma unroll
-    for (int cb = 0; cb < NCB; ++cb) {
-      f32x4 s{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[k], qf[cb][k], s);
-      const Frag<T> pf = softmax_block<T>(s, scale_log2, kb0, col_valid ? pos : -1, window, hi, st[cb],
-                                          o[cb], lane);
-#pragma unroll
-      for (int db = 0; db < kSteps; ++db) o[cb][db] = Mma16<T>::mma(vf[db], pf, o[cb][db]);
-    }
-  }
-
-#pragma unroll
-  for (int cb = 0; cb < NCB; ++cb) {
-    const int hh = hsub + cb;
-    const float l = lane_groups_sum(st[cb].lsum);
-    if (!col_valid || hh >= g) continue;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* orow = out + token * out_stride + static_cast<size_t>(kvh * g + hh) * HD + 4 * (lane / 16);
-#pragma unroll
-    for (int db = 0; db < kSteps; ++db) {
-      Frag<T> f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) f[i] = from_f32<T>(o[cb][db][i] * inv);
-      *reinterpret_cast<Frag<T>*>(orow + db * 16) = f;
-    }
-  }
-}
-
-// ---------------------------------------------------------------------- decode
-// grid (partitions, nkv * column_groups, requests); kDecodeWaves waves.  A
-// workgroup takes one partition of kDecodeWaves * keys_per_wave keys and merges
-// its waves' results through LDS, in a fixed order.  Column c of the tile is
-// query head kvh * g + 16 * column_group + c of the request's one new token.
-// How many keys a wave takes is the launch's choice (lyp_attn_decode_plan): few
-// when there is little work, so that it spreads over the chip; many when there
-// is a lot, so that the fixed cost of a workgroup is paid less often.
-// Partials: part_o [request][head][part][hd] (not normalised), part_ml
-// [request][head][part][2] = (maximum in the base-2 domain, sum).
-constexpr int kDecodeWaves = HD <= 128 ? 4 : 2;
-constexpr int kDecodeDepth = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // 16-key blocks in flight per wave
 
 // One 16-key block of keys and values.  FULL: the page size is a multiple of 16
 // and every key of the block is inside the request and visible, so the block
@@ -332,6 +288,301 @@ __device__ __forceinline__ void load_block_full(Frag<T> (&kf)[kSteps], Frag<T> (
   for (int db = 0; db < kSteps; ++db)
     vf[db] = *reinterpret_cast<const Frag<T>*>(vrow + static_cast<size_t>(db) * 16 * kv.bs);
 }
+
+// --------------------------------------------------------------------- prefill
+// grid (tiles * sub-tiles, nkv * head_groups); 256 threads (four waves).  A
+// workgroup takes QW consecutive new tokens of one request and GH query heads of
+// one key/value head; wave w takes head w % GH and token sub-block w / GH (QB
+// blocks of 16 tokens).  The keys and values the tokens may see are brought
+// into LDS tile by tile (the next tile travels while the current one is used)
+// and shared by the four waves, so that a key is read from memory once for all
+// the heads of its group.
+template <typename T>
+struct PrefillTile {
+  static constexpr int kKeys = HD * sizeof(T) <= 128 ? 64 : (HD * sizeof(T) <= 256 ? 32 : 16);
+  static constexpr int kVec = 16 / sizeof(T);          // elements per 16-byte access
+  static constexpr int kKLd = HD + 4;                  // padded row of the key tile [keys][hd]
+  static constexpr int kVLd = kKeys + 4;               // padded row of the value tile [hd][keys]
+  static constexpr int kElems = kKeys * kKLd + HD * kVLd;
+  static constexpr int kBufs = 2 * kElems * sizeof(T) <= 60 * 1024 ? 2 : 1;
+  static constexpr int kKVecs = kKeys * HD / kVec;     // 16-byte pieces of a key tile
+  static constexpr int kPerThread = (kKVecs + 255) / 256;
+};
+
+template <typename T, int GH, int QB>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const void* kpool,
+    const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
+    int bs, int window, float scale_log2) {
+  using PT = PrefillTile<T>;
+  constexpr int KT = PT::kKeys, NB = KT / 16, VEC = PT::kVec;
+  constexpr int QW = (4 / GH) * QB * 16;  // new tokens per workgroup
+  constexpr int kSubs = 64 / QW;          // workgroups per 64-token tile of the host's list
+  static_assert(QW <= 64 && 64 % QW == 0, "a workgroup takes a whole fraction of a 64-token tile");
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  __shared__ __attribute__((aligned(16))) T lds[PT::kBufs * PT::kElems];
+
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int g = nh / nkv;
+  const int head_groups = (g + GH - 1) / GH;
+  const int kvh = blockIdx.y / head_groups;
+  const int hsub = (blockIdx.y % head_groups) * GH;
+
+  // The host lists tiles in rising order of position; the longest are started first.
+  const int tile = n_tiles - 1 - static_cast<int>(blockIdx.x) / kSubs;
+  const int seq = tile_seq[tile];
+  const int tok0 = q_start[seq];
+  const int q_len = q_start[seq + 1] - tok0;
+  const int ctx = ctx_len[seq];
+  const int q0_wg = tile_q0[tile] + (static_cast<int>(blockIdx.x) % kSubs) * QW;
+  if (q0_wg >= q_len) return;  // the whole workgroup
+  const int pos_first = ctx - q_len + q0_wg;
+  const int pos_last_wg = pos_first + min(QW, q_len - q0_wg) - 1;
+  const int lo_wg = window > 0 ? max(0, pos_first - window + 1) : 0;
+  const int hi_wg = pos_last_wg + 1;
+
+  // this wave's head and tokens
+  const int hw = hsub + wave % GH;
+  const int q0_w = q0_wg + (wave / GH) * QB * 16;
+  const bool wave_active = hw < g && q0_w < q_len;
+  const int col = lane % 16;
+  const int head = kvh * g + (hw < g ? hw : 0);
+
+  Frag<T> qf[QB][kSteps];
+  f32x4 o[QB][kSteps];
+  Softmax st[QB];
+  int pos0[QB];
+  bool col_valid[QB];
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    const int qi = q0_w + 16 * b + col;
+    col_valid[b] = wave_active && qi < q_len;
+    pos0[b] = ctx - q_len + q0_w + 16 * b;
+    load_q<T>(qf[b], q + (static_cast<size_t>(tok0) + qi) * q_stride + static_cast<size_t>(head) * HD, col_valid[b],
+              lane);
+    st[b] = Softmax{LYP_NEG_INF, 0.f};
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) o[b][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int pos_last_w = min(pos_last_wg, pos0[0] + QB * 16 - 1);
+
+  // ---- bringing a tile in: global -> registers -> LDS
+  const int32_t* table = block_tables + static_cast<size_t>(seq) * max_blocks;
+  const T* kp = static_cast<const T*>(kpool);
+  const T* vp = static_cast<const T*>(vpool);
+  const bool v_vectors = bs % VEC == 0;
+  VecT kreg[PT::kPerThread], vreg[PT::kPerThread];
+  auto zero_vec = [] {
+    VecT z;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) z[e] = from_f32<T>(0.f);
+    return z;
+  };
+  // Where this thread's pieces of a tile lie (the same for every tile).
+  constexpr int kPer16 = 16 / VEC;
+  int k_row[PT::kPerThread], k_d0[PT::kPerThread], v_blk[PT::kPerThread], v_d[PT::kPerThread], v_c[PT::kPerThread];
+#pragma unroll
+  for (int n = 0; n < PT::kPerThread; ++n) {
+    const int v = tid + n * 256;
+    k_row[n] = v / (HD / VEC);
+    k_d0[n] = (v % (HD / VEC)) * VEC;
+    v_blk[n] = v / (HD * kPer16);
+    v_d[n] = (v % (HD * kPer16)) / kPer16;
+    v_c[n] = (v % kPer16) * VEC;
+  }
+  const bool aligned = bs % 16 == 0;
+  // Table entries of a tile's 16-key blocks: the same for the whole workgroup,
+  // and read a tile ahead of the data so that the two reads do not queue up.
+  auto tile_pages = [&](int kt0, int (&pg)[NB]) {
+#pragma unroll
+    for (int u = 0; u < NB; ++u) pg[u] = table[min((kt0 + 16 * u) / bs, max_blocks - 1)];
+  };
+  auto fetch = [&](int kt0, const int (&pg)[NB]) {
+    if (aligned && kt0 >= lo_wg && kt0 + KT <= hi_wg) {
+      // the whole tile exists and is wanted: no tests, one table entry per 16 keys
+#pragma unroll
+      for (int n = 0; n < PT::kPerThread; ++n) {
+        if (tid + n * 256 >= PT::kKVecs) continue;
+        int page_k = pg[0], page_v = pg[0];
+#pragma unroll
+        for (int u = 1; u < NB; ++u) {
+          if (k_row[n] / 16 == u) page_k = pg[u];
+          if (v_blk[n] == u) page_v = pg[u];
+        }
+        const int off_k = (kt0 + (k_row[n] / 16) * 16) % bs + k_row[n] % 16;
+        kreg[n] = *reinterpret_cast<const VecT*>(
+            kp + ((static_cast<size_t>(page_k) * nkv + kvh) * bs + off_k) * HD + k_d0[n]);
+        const int off_v = (kt0 + 16 * v_blk[n]) % bs + v_c[n];
+        vreg[n] = *reinterpret_cast<const VecT*>(
+            vp + ((static_cast<size_t>(page_v) * nkv + kvh) * HD + v_d[n]) * bs + off_v);
+      }
+      return;
+    }
+#pragma unroll
+    for (int n = 0; n < PT::kPerThread; ++n) {
+      kreg[n] = zero_vec();
+      vreg[n] = zero_vec();
+      if (tid + n * 256 >= PT::kKVecs) continue;
+      {  // keys: 16 bytes of key kt0 + k_row
+        const int key = kt0 + k_row[n];
+        if (key >= lo_wg && key < hi_wg) {
+          const int page = table[key / bs];
+          if (page >= 0)
+            kreg[n] = *reinterpret_cast<const VecT*>(
+                kp + ((static_cast<size_t>(page) * nkv + kvh) * bs + key % bs) * HD + k_d0[n]);
+        }
+      }
+      {  // values: 16-key blocks one after the other, inside a block dimension by dimension
+        const int d = v_d[n], key0 = kt0 + 16 * v_blk[n] + v_c[n];
+        if (key0 < hi_wg && key0 + VEC > lo_wg) {
+          if (v_vectors) {
+            const int page = table[key0 / bs];
+            if (page >= 0) {
+              VecT x = *reinterpret_cast<const VecT*>(
+                  vp + ((static_cast<size_t>(page) * nkv + kvh) * HD + d) * bs + key0 % bs);
+#pragma unroll
+              for (int e = 0; e < VEC; ++e)
+                if (key0 + e < lo_wg || key0 + e >= hi_wg) x[e] = from_f32<T>(0.f);
+              vreg[n] = x;
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const int key = key0 + e;
+              if (key < lo_wg || key >= hi_wg) continue;
+              const int page = table[key / bs];
+              if (page >= 0) vreg[n][e] = vp[((static_cast<size_t>(page) * nkv + kvh) * HD + d) * bs + key % bs];
+            }
+          }
+        }
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+    T* ks = lds + buf * PT::kElems;
+    T* vs = ks + KT * PT::kKLd;
+#pragma unroll
+    for (int n = 0; n < PT::kPerThread; ++n) {
+      if (tid + n * 256 >= PT::kKVecs) continue;
+      const int kr = k_row[n], d0 = k_d0[n];
+      // rows are padded by 4 elements, so a 16-byte store may straddle an 8-byte boundary: two halves
+      typedef T HalfT __attribute__((ext_vector_type(VEC / 2)));
+      HalfT lo_h, hi_h;
+#pragma unroll
+      for (int e = 0; e < VEC / 2; ++e) {
+        lo_h[e] = kreg[n][e];
+        hi_h[e] = kreg[n][e + VEC / 2];
+      }
+      *reinterpret_cast<HalfT*>(ks + kr * PT::kKLd + d0) = lo_h;
+      *reinterpret_cast<HalfT*>(ks + kr * PT::kKLd + d0 + VEC / 2) = hi_h;
+      const int d = v_d[n], c0 = 16 * v_blk[n] + v_c[n];
+#pragma unroll
+      for (int e = 0; e < VEC / 2; ++e) {
+        lo_h[e] = vreg[n][e];
+        hi_h[e] = vreg[n][e + VEC / 2];
+      }
+      *reinterpret_cast<HalfT*>(vs + d * PT::kVLd + c0) = lo_h;
+      *reinterpret_cast<HalfT*>(vs + d * PT::kVLd + c0 + VEC / 2) = hi_h;
+    }
+  };
+
+  // ---- one tile's worth of work for this wave
+  auto compute = [&](int buf, int kt0) {
+    const T* ks = lds + buf * PT::kElems;
+    const T* vs = ks + KT * PT::kKLd;
+    f32x4 sc[QB][NB];
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      Frag<T> kf[kSteps];
+      const T* krow = ks + (16 * u + lane % 16) * PT::kKLd + (lane / 16) * kSlice;
+#pragma unroll
+      for (int k = 0; k < kSteps; ++k) kf[k] = *reinterpret_cast<const Frag<T>*>(krow + 4 * k);
+#pragma unroll
+      for (int b = 0; b < QB; ++b) {
+        sc[b][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < kSteps; ++k) sc[b][u] = Mma16<T>::mma(kf[k], qf[b][k], sc[b][u]);
+      }
+    }
+    Frag<T> pf[QB][NB];
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+      // every token of the block sees the whole tile: no masks
+      const bool full = kt0 + KT - 1 <= pos0[b] && kt0 >= lo_wg && pos0[b] + 15 <= pos_last_wg &&
+                        (window == 0 || kt0 > pos0[b] + 15 - window);
+      if (full)
+        softmax_group<T, false, NB>(sc[b], pf[b], scale_log2, kt0, pos0[b] + col, window, hi_wg, st[b], o[b], lane);
+      else
+        softmax_group<T, true, NB>(sc[b], pf[b], scale_log2, kt0, col_valid[b] ? pos0[b] + col : -1, window, hi_wg,
+                                   st[b], o[b], lane);
+    }
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      Frag<T> vf[kSteps];
+      const T* vrow = vs + (lane % 16) * PT::kVLd + 16 * u + 4 * (lane / 16);
+#pragma unroll
+      for (int db = 0; db < kSteps; ++db) vf[db] = *reinterpret_cast<const Frag<T>*>(vrow + db * 16 * PT::kVLd);
+#pragma unroll
+      for (int b = 0; b < QB; ++b)
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db) o[b][db] = Mma16<T>::mma(vf[db], pf[b][u], o[b][db]);
+    }
+  };
+
+  const int kt_first = (lo_wg / KT) * KT;
+  int pages[NB];
+  tile_pages(kt_first, pages);
+  fetch(kt_first, pages);
+  tile_pages(kt_first + KT, pages);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kt0 = kt_first; kt0 < hi_wg; kt0 += KT) {
+    const bool more = kt0 + KT < hi_wg;
+    if (more) {
+      fetch(kt0 + KT, pages);
+      tile_pages(kt0 + 2 * KT, pages);  // for the fetch of the next round
+    }
+    if (wave_active && kt0 <= pos_last_w) compute(buf, kt0);
+    if (PT::kBufs == 1) __syncthreads();  // everyone is done with the only buffer before it is overwritten
+    const int next = PT::kBufs == 2 ? buf ^ 1 : 0;
+    if (more) stash(next);
+    __syncthreads();
+    buf = next;
+  }
+
+#pragma unroll
+  for (int b = 0; b < QB; ++b) {
+    const float l = lane_groups_sum(st[b].lsum);
+    if (!col_valid[b]) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const size_t token = static_cast<size_t>(tok0) + q0_w + 16 * b + col;
+    T* orow = out + token * out_stride + static_cast<size_t>(head) * HD + 4 * (lane / 16);
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) {
+      Frag<T> f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f[i] = from_f32<T>(o[b][db][i] * inv);
+      *reinterpret_cast<Frag<T>*>(orow + db * 16) = f;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------- decode
+// grid (partitions, nkv * column_groups, requests); kDecodeWaves waves.  A
+// workgroup takes one partition of kDecodeWaves * keys_per_wave keys and merges
+// its waves' results through LDS, in a fixed order.  Column c of the tile is
+// query head kvh * g + 16 * column_group + c of the request's one new token.
+// How many keys a wave takes is the launch's choice (lyp_attn_decode_plan): few
+// when there is little work, so that it spreads over the chip; many when there
+// is a lot, so that the fixed cost of a workgroup is paid less often.
+// Partials: part_o [request][head][part][hd] (not normalised), part_ml
+// [request][head][part][2] = (maximum in the base-2 domain, sum).
+constexpr int kDecodeWaves = HD <= 128 ? 4 : 2;
+constexpr int kDecodeDepth = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // 16-key blocks in flight per wave
 
 template <typename T>
 __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
@@ -532,30 +783,31 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   LYP_REQUIRE(n_tiles >= 0, "attn_prefill: %d tiles", n_tiles);
   if (n_tiles == 0) return 0;
   const int g = nh / nkv;
-  // Column blocks per wave, bounded by what the register file holds.
-  const int regs_per_block = kSteps * ((dtype == kF32 ? 4 : 2) + 4);
-  const int cap = 192 / regs_per_block;
-  const int want = g >= 4 ? 4 : (g >= 2 ? 2 : 1);
-  const int ncb = cap >= 4 ? want : (cap >= 2 ? (want >= 2 ? 2 : 1) : 1);
-  const int head_groups = (g + ncb - 1) / ncb;
+  // Heads per workgroup: as many of the group as four waves hold; the waves
+  // that are left over take further tokens.
+  const int gh = g >= 4 ? 4 : (g >= 2 ? 2 : 1);
+  const int head_groups = (g + gh - 1) / gh;
   LYP_REQUIRE(nkv * head_groups <= 65535, "attn_prefill: too many heads for one launch");
-  dim3 grid(n_tiles, nkv * head_groups);
   const float scale_log2 = scale * kLog2e;
-#define LYP_PREFILL(T, NCB)                                                                              \
-  attn_prefill_kernel<T, NCB><<<grid, 256, 0, stream>>>(                                                  \
-      static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,  \
-      max_blocks, q_start, ctx_len, tile_seq, tile_q0, nh, nkv, bs, window, scale_log2)
-  if (dtype == kF32) {
-    if (ncb == 4) LYP_PREFILL(float, 4);
-    else if (ncb == 2) LYP_PREFILL(float, 2);
-    else LYP_PREFILL(float, 1);
-  } else if (dtype == kBF16) {
-    if (ncb == 4) LYP_PREFILL(bf16_t, 4);
-    else if (ncb == 2) LYP_PREFILL(bf16_t, 2);
-    else LYP_PREFILL(bf16_t, 1);
-  } else {
-    LYP_REQUIRE(false, "attn_prefill: unknown dtype %d", dtype);
-  }
+#define LYP_PREFILL(T, GH, QB)                                                                              \
+  do {                                                                                                      \
+    constexpr int kQW = (4 / GH) * QB * 16;                                                                 \
+    dim3 grid(n_tiles*(64 / kQW), nkv * head_groups);                                                      \
+    attn_prefill_kernel<T, GH, QB><<<grid, 256, 0, stream>>>(                                               \
+        static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,   \
+        max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2);         \
+  } while (0)
+#define LYP_PREFILL_T(T)                    \
+  do {                                      \
+    if (gh == 4) LYP_PREFILL(T, 4, kQB4);   \
+    else if (gh == 2) LYP_PREFILL(T, 2, 1); \
+    else LYP_PREFILL(T, 1, 1);              \
+  } while (0)
+  constexpr int kQB4 = LYP_PREFILL_QB;
+  if (dtype == kF32) LYP_PREFILL_T(float);
+  else if (dtype == kBF16) LYP_PREFILL_T(bf16_t);
+  else LYP_REQUIRE(false, "attn_prefill: unknown dtype %d", dtype);
+#undef LYP_PREFILL_T
 #undef LYP_PREFILL
   LYP_LAUNCH_CHECK("attn_prefill");
   return 0;

@@ -134,7 +134,13 @@ def _run_with_progress(cmds: list[list[str]], what: str) -> None:
 def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str, str] | None = None,
                   force: bool = False) -> Path:
     """Return the path of the library, compiling it if it is not there."""
-    defines = defines or {}
+    defines = dict(defines or {})
+    # For experiments: LYAPUNOV_AMD_EXTRA_DEFINES="NAME=VALUE,OTHER=1" adds macros to every HIP compile
+    # (the library's name changes with them, so the regular build is left alone).
+    if hip and os.environ.get("LYAPUNOV_AMD_EXTRA_DEFINES"):
+        for item in os.environ["LYAPUNOV_AMD_EXTRA_DEFINES"].split(","):
+            k, _, v = item.partition("=")
+            defines[k.strip()] = v.strip() or "1"
     compiler = hipcc_path() if hip else cxx_path()
     flags = (HIP_FLAGS if hip else CXX_FLAGS) + [f"-D{k}={v}" for k, v in sorted(defines.items())]
     include = ["-I", str(CSRC / "kernels"), "-I", str(CSRC / "runtime")]
@@ -162,7 +168,7 @@ def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str
         finally:
             shutil.rmtree(work, ignore_errors=True)
         for old in out_dir.glob(f"lib{name}-*.so"):
-            if old != target:
+            if old != target and not os.environ.get("LYAPUNOV_AMD_EXTRA_DEFINES"):
                 try:
                     old.unlink()
                 except OSError:
