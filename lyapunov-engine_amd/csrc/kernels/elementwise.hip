@@ -199,6 +199,37 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   out[idx] = from_f32<T>((g / (1.0f + expf(-g))) * u);
 }
 
+// The same, eight outputs per thread with 16-byte accesses; needs I % 8 == 0
+// and 16-byte aligned rows.  In the tiled layout a thread's eight gates and
+// eight ups are 32 consecutive bytes (bfloat16) of the input.
+template <typename T>
+__global__ void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total8,
+                                  int interleave) {
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;  // one run of eight outputs
+  if (idx >= total8) return;
+  const size_t per_row = I / 8;
+  const size_t t = idx / per_row, c = idx % per_row;
+  const T* row = gu + t * 2 * I;
+  const T* gp = interleave ? row + c * 16 : row + c * 8;
+  const T* up = interleave ? gp + 8 : row + I + c * 8;
+  T* op = out + t * I + c * 8;
+#pragma unroll
+  for (int h = 0; h < 8 / VEC; ++h) {
+    const VecT g = *reinterpret_cast<const VecT*>(gp + h * VEC);
+    const VecT u = *reinterpret_cast<const VecT*>(up + h * VEC);
+    VecT o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float gf = to_f32(g[e]);
+      const float ex = sizeof(T) == 4 ? expf(-gf) : __expf(-gf);
+      o[e] = from_f32<T>((gf / (1.0f + ex)) * to_f32(u[e]));
+    }
+    *reinterpret_cast<VecT*>(op + h * VEC) = o;
+  }
+}
+
 // ----------------------------------------------------------------------- cast
 template <typename TI, typename TO>
 __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
@@ -324,15 +355,24 @@ int lyp_swiglu(const void* gate_up, void* out, int dtype, int T, int I, int inte
   const size_t total = static_cast<size_t>(T) * I;
   if (total == 0) return 0;
   const int threads = 256;
-  const unsigned blocks = static_cast<unsigned>((total + threads - 1) / threads);
-  if (dtype == kF32)
-    swiglu_kernel<float><<<blocks, threads, 0, stream>>>(static_cast<const float*>(gate_up),
-                                                         static_cast<float*>(out), I, total, interleave);
-  else if (dtype == kBF16)
-    swiglu_kernel<bf16_t><<<blocks, threads, 0, stream>>>(static_cast<const bf16_t*>(gate_up),
-                                                          static_cast<bf16_t*>(out), I, total, interleave);
-  else
-    LYP_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+  const bool vec = I % 8 == 0 && reinterpret_cast<uintptr_t>(gate_up) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const size_t work = vec ? total / 8 : total;
+  LYP_REQUIRE((work + threads - 1) / threads <= 2147483647u, "swiglu: too many elements for one launch");
+  const unsigned blocks = static_cast<unsigned>((work + threads - 1) / threads);
+#define LYP_SWIGLU(T)                                                                                         \
+  do {                                                                                                        \
+    if (vec)                                                                                                  \
+      swiglu_vec_kernel<T><<<blocks, threads, 0, stream>>>(static_cast<const T*>(gate_up), static_cast<T*>(out), \
+                                                           I, work, interleave);                              \
+    else                                                                                                      \
+      swiglu_kernel<T><<<blocks, threads, 0, stream>>>(static_cast<const T*>(gate_up), static_cast<T*>(out), I, \
+                                                       total, interleave);                                    \
+  } while (0)
+  if (dtype == kF32) LYP_SWIGLU(float);
+  else if (dtype == kBF16) LYP_SWIGLU(bf16_t);
+  else LYP_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+#undef LYP_SWIGLU
   LYP_LAUNCH_CHECK("swiglu");
   return 0;
 }

@@ -58,10 +58,38 @@ __device__ __forceinline__ int block_count(int c, int* scratch) {
   return total;
 }
 
+// First pass over the logits with the whole chip: the row is cut into
+// kArgmaxChunks pieces, one workgroup each, and every piece leaves its largest
+// value and the first index that has it.
+constexpr int kArgmaxChunks = 32;
+
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, int ld, int V,
+                                                            ArgMax* __restrict__ cand) {
+  __shared__ ArgMax s_arg[4];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int per = (V + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int begin = min(V, chunk * per), end = min(V, begin + per);
+  const float* x = logits + static_cast<size_t>(row) * ld;
+  ArgMax am{LYP_NEG_INF, 0x7fffffff};
+  for (int i = begin + threadIdx.x; i < end; i += 256) am = better(am, ArgMax{x[i], i});
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    ArgMax o{__shfl_xor(am.v, off, kWave), __shfl_xor(am.i, off, kWave)};
+    am = better(am, o);
+  }
+  if (threadIdx.x % kWave == 0) s_arg[threadIdx.x / kWave] = am;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    ArgMax r = s_arg[0];
+    for (int w = 1; w < 4; ++w) r = better(r, s_arg[w]);
+    cand[row * kArgmaxChunks + chunk] = r;
+  }
+}
+
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
-    int32_t* __restrict__ out) {
+    const ArgMax* __restrict__ cand, int32_t* __restrict__ out) {
   __shared__ ArgMax s_arg[kSampleThreads / kWave];
   __shared__ int s_cnt[kSampleThreads / kWave];
   __shared__ float s_f[kSampleThreads / kWave];
@@ -73,7 +101,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const float* x = logits + static_cast<size_t>(row) * ld;
 
   ArgMax am{LYP_NEG_INF, 0x7fffffff};
-  for (int i = tid; i < V; i += kSampleThreads) am = better(am, ArgMax{x[i], i});
+  if (cand) {  // the pieces' winners instead of the whole row
+    if (tid < kArgmaxChunks) am = cand[row * kArgmaxChunks + tid];
+  } else {
+    for (int i = tid; i < V; i += kSampleThreads) am = better(am, ArgMax{x[i], i});
+  }
   am = block_argmax(am, s_arg);
   const float T = temperature[row];
   if (T < 1e-4f) {
@@ -175,13 +207,23 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 using namespace lyp;
 
+// Bytes of workspace lyp_sample wants for this many rows.
+extern "C" long long lyp_sample_workspace(int rows) {
+  return static_cast<long long>(rows) * kArgmaxChunks * sizeof(ArgMax);
+}
+
 // logits [rows, ld] float; temperature, top_k, top_p, uniform: one per row.
+// workspace: lyp_sample_workspace(rows) bytes, or null (then one workgroup per
+// row scans its whole row for the maximum).
 extern "C" int lyp_sample(const float* logits, int ld, int rows, int V, const float* temperature,
-                          const int32_t* top_k, const float* top_p, const float* uniform, int32_t* out,
-                          hipStream_t stream) {
+                          const int32_t* top_k, const float* top_p, const float* uniform, void* workspace,
+                          int32_t* out, hipStream_t stream) {
   LYP_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
   if (rows == 0) return 0;
-  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, out);
+  LYP_REQUIRE(rows <= 65535, "sample: %d rows in one launch", rows);
+  ArgMax* cand = static_cast<ArgMax*>(workspace);
+  if (cand) argmax_chunks_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(logits, ld, V, cand);
+  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, cand, out);
   LYP_LAUNCH_CHECK("sample");
   return 0;
 }

@@ -59,7 +59,9 @@ def core() -> ctypes.CDLL:
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
         lib.lyp_sample.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                   c_void_p]
+                                   c_void_p, c_void_p]
+        lib.lyp_sample_workspace.argtypes = [c_int]
+        lib.lyp_sample_workspace.restype = c_longlong
         _core = lib
     return _core
 
@@ -388,9 +390,15 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
 
 
 # -------------------------------------------------------------------- sampling
+def sample_workspace(rows: int, device) -> torch.Tensor:
+    return torch.empty(max(1, core().lyp_sample_workspace(rows)), dtype=torch.uint8, device=device)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    _dev(logits, temperature, top_k, top_p, uniform, out)
+           uniform: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row of logits.  With a ``workspace`` (``sample_workspace``)
+    the search for each row's maximum is spread over the chip."""
+    _dev(logits, temperature, top_k, top_p, uniform, out, workspace)
     R, V = logits.shape
     if logits.dtype != torch.float32 or temperature.dtype != torch.float32 or top_k.dtype != torch.int32 or \
             top_p.dtype != torch.float32 or uniform.dtype != torch.float32 or out.dtype != torch.int32:
@@ -398,6 +406,8 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if any(t.numel() != R for t in (temperature, top_k, top_p, uniform, out)):
         raise KernelError("sample: one parameter per row")
     lib = core()
-    _check(lib.lyp_sample(_p(logits), V, R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform), _p(out),
-                          _stream()), lib)
+    if workspace is not None and workspace.numel() < lib.lyp_sample_workspace(R):
+        raise KernelError("sample: workspace too small")
+    _check(lib.lyp_sample(_p(logits), V, R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform), _p(workspace),
+                          _p(out), _stream()), lib)
     return out

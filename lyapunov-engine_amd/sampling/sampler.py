@@ -49,6 +49,7 @@ class Sampler:
             self._host = torch.zeros((4, self._cap), dtype=torch.float32).pin_memory()
             self._dev = torch.zeros((4, self._cap), dtype=torch.float32, device=self.device)
             self._out = torch.zeros(self._cap, dtype=torch.int32, device=self.device)
+            self._work = ops.sample_workspace(self._cap, self.device)
             self._greedy_on_device = True   # the device block is all zeros: temperature 0 everywhere
 
     def sample(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> list:
@@ -74,7 +75,7 @@ class Sampler:
             self._greedy_on_device = False
         d = self._dev
         out = self._out[:R]
-        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out)
+        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work)
         return out.tolist()
 
 

@@ -356,7 +356,8 @@ def test_sampler_greedy_and_draws(ops):
     for u_val in (0.0, 0.137, 0.5, 0.77, 0.999):
         u = torch.full((6,), u_val)
         out = torch.empty(6, dtype=torch.int32, device=DEV)
-        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out)
+        work = ops.sample_workspace(6, DEV) if u_val > 0.4 else None   # both ways of finding the maximum
+        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out, work)
         got = out.cpu().tolist()
         assert got[0] == P.greedy(logits[0])
         assert got[1] == 7
