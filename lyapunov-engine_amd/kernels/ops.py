@@ -224,7 +224,7 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, interleave: int) -> torch.Te
             raise KernelError(f"linear_swiglu: weight {w.dtype} against activations {x.dtype}")
         return cast(linear_swiglu(cast(x, torch.float32), w, interleave), x.dtype)
     out = torch.empty((x.shape[0], I), dtype=x.dtype, device=x.device)
-    if interleave == 8 and x.shape[0] <= 64:
+    if interleave == 8 and x.shape[0] <= 64 and not _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
         _dev(x, w)
         lib = core()
         rc = lib.lyp_gemm_swiglu(_p(x), _p(w), _p(out), _code(x.dtype), x.shape[0], w.shape[0], w.shape[1],
@@ -255,6 +255,17 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 # (true 32-bit) and everything when LYAPUNOV_AMD_GEMM=own use the kernels here.
 LIBRARY_GEMM = os.environ.get("LYAPUNOV_AMD_GEMM", "library") != "own"
 LIBRARY_GEMM_MIN_ROWS = 65
+# Between 17 and 64 rows the weight-streaming kernel re-reads the activations
+# once per 16 weight rows, which costs more than the weights themselves when the
+# matrix is large; measured, the library is ahead from this many weights on.
+LIBRARY_GEMM_MID_ROWS = 17
+LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
+
+
+def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+    if not LIBRARY_GEMM or dtype != torch.bfloat16:
+        return False
+    return M >= LIBRARY_GEMM_MIN_ROWS or (M >= LIBRARY_GEMM_MID_ROWS and N * K >= LIBRARY_GEMM_MID_WEIGHTS)
 
 
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
@@ -265,8 +276,7 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
     N = w.shape[0]
     if w.shape[1] != K or tuple(out.shape) != (M, N) or a.dtype != w.dtype:
         raise KernelError(f"gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
-    if LIBRARY_GEMM and a.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and not accumulate \
-            and M >= LIBRARY_GEMM_MIN_ROWS:
+    if out.dtype == torch.bfloat16 and not accumulate and _library_product(M, N, K, a.dtype):
         return torch.matmul(a, w.t(), out=out)
     if accumulate:
         if out.dtype != torch.float32:
@@ -298,7 +308,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
         if w.dtype != torch.float32:
             raise KernelError(f"linear: weight {w.dtype} against activations {x.dtype}")
         x = cast(x, torch.float32)
-    if may_split and x.shape[0] <= 64:
+    if may_split and x.shape[0] <= 64 and not _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
         _dev(x, w)
         lib = core()
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
@@ -308,6 +318,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
             _check(lib.lyp_gemm_nt_parts(_p(x), _p(w), _p(parts), _code(x.dtype), slices, M, N, K, x.stride(0),
                                          w.stride(0), _stream()), lib)
             return parts
+    if out_dtype == torch.float32 and _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
+        # the library writes the operands' type; the float result is a cast of it
+        y = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+        return cast(gemm_nt(x, w, y), torch.float32)
     if out_dtype in (x.dtype, torch.float32):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
         return gemm_nt(x, w, out)
