@@ -571,6 +571,356 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   }
 }
 
+#if LYP_HEAD_DIM % 32 == 0
+// ------------------------------------------------- prefill, bfloat16, wide steps
+// The same work with the 16x16x32 matrix instruction (head sizes that are
+// multiples of 32), more waves per workgroup and loads that run further ahead:
+// NW waves, wave w takes head w % GH and the 16 tokens of sub-block w / GH, so
+// a workgroup covers (NW / GH) * 16 tokens (a unit).  The page size must be a
+// multiple of 16, so that a 16-key block never straddles two pages.
+//   * A lane holds eight consecutive values of the inner dimension.  For P.V the
+//     inner dimension is the key: the score tiles leave lane group j with keys
+//     4 j + {0..3} of two neighbouring 16-key blocks, so the value tile is
+//     stored in LDS with its columns in that order (key 32 w + 16 h + 4 j + i at
+//     column 32 w + 8 j + 4 h + i) and a lane reads its eight values in one piece.
+//   * Tiles travel memory -> registers -> LDS two tiles ahead of their use: two
+//     sets of registers, two LDS buffers.  Every round of the loop asks for
+//     exactly the same loads (past the end of the keys the addresses are clamped
+//     and the data is dropped), which lets the waits for them be counted exactly.
+//   * When `paired`, a workgroup takes two units one after the other, number b
+//     from the heavy end of the host's list and number b from the light end, so
+//     that with a causal mask every workgroup has the same amount of work.
+//   * The exponent is formed as fma(score, scale, -maximum); the accumulators are rescaled only
+//     when a maximum grew; the sum of the probabilities is one more row of the P.V product.
+struct WideTile {
+  static constexpr int kKeys = HD <= 64 ? 64 : 32;
+  static constexpr int kKLd = HD + 8;     // rows stay 16-byte aligned and skewed by four banks
+  static constexpr int kVLd = kKeys + 8;
+  static constexpr int kElems = kKeys * kKLd + HD * kVLd;
+  static constexpr int kBufs = 2 * kElems * 2 <= 64 * 1024 ? 2 : 1;
+  static constexpr int kVecs = kKeys * HD / 8;  // 16-byte pieces of a key tile (and of a value tile)
+};
+
+// The maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in every one of them, with the two
+// row-swap instructions of this chip (no trip through LDS).  v_permlane16_swap exchanges the odd
+// 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap the upper
+// half of the first with the lower half of the second; fed with two copies of a value, the two
+// results hold it and its neighbour's.
+__device__ __forceinline__ float lane_groups_max(float m) {
+  float a = m, b = m;
+  asm volatile(
+      "s_nop 1\n\t"
+      "v_permlane16_swap_b32 %0, %1\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32 %0, %0, %1\n\t"
+      "v_mov_b32 %1, %0\n\t"
+      "s_nop 1\n\t"
+      "v_permlane32_swap_b32 %0, %1\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32 %0, %0, %1"
+      : "+v"(a), "+v"(b));
+  return a;
+}
+
+// The scores of one tile (s[u]: rows = keys kb0 + 16 u + 4 (l / 16) + i, column l % 16): update
+// the running maximum `m_run` (base-2 domain), rescale the accumulators when some column's
+// maximum grew (o: the output; lacc: the sum of the probabilities, which the matrix unit adds up
+// with a row of ones), and return the probabilities as the column operand of the P.V product.
+template <bool MASKED, int NB>
+__device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[NB / 2], float scale_log2, int kb0,
+                                             int pos, int window, int hi, float& m_run, f32x4& lacc,
+                                             f32x4 (&o)[kSteps], int lane) {
+  bool vis[NB][4];
+  float mx = LYP_NEG_INF;
+#pragma unroll
+  for (int u = 0; u < NB; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if constexpr (MASKED) {
+        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
+        vis[u][i] = key <= pos && key < hi && (window == 0 || key > pos - window);
+        mx = fmaxf(mx, vis[u][i] ? s[u][i] : LYP_NEG_INF);
+      } else {
+        vis[u][i] = true;
+        mx = fmaxf(mx, s[u][i]);
+      }
+    }
+  mx = lane_groups_max(mx);
+  const float m_new = fmaxf(m_run, mx * scale_log2);  // the scale is positive
+  if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+    const float alpha = fast_exp2(m_run - (m_new == LYP_NEG_INF ? 0.f : m_new));  // 0 while nothing was seen
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lacc[i] *= alpha;
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
+  }
+  const float m_safe = m_run == LYP_NEG_INF ? 0.f : m_run;
+#pragma unroll
+  for (int u = 0; u < NB; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float p = fast_exp2(__builtin_fmaf(s[u][i], scale_log2, -m_safe));
+      if constexpr (MASKED) p = vis[u][i] ? p : 0.f;
+      pw[u / 2][4 * (u % 2) + i] = from_f32<bf16_t>(p);
+    }
+}
+
+// One thread's share of a tile on its way from memory to LDS.
+template <int PER>
+struct TileRegs {
+  bf16x8 k[PER], v[PER];
+  bool lost[PER];  // the table had no page for the piece's block
+};
+
+template <int GH, int NW>
+__global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide_kernel(
+    const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride, const void* kpool,
+    const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
+    int bs, int window, float scale_log2, int paired) {
+  using T = bf16_t;
+  using WT = WideTile;
+  using MMA = Mma16Wide<bf16_t>;
+  constexpr int KT = WT::kKeys, NB = KT / 16, NWIDE = KT / 32, DSTEPS = HD / 32;
+  constexpr int THREADS = NW * kWave;
+  constexpr int PER = (WT::kVecs + THREADS - 1) / THREADS;
+  constexpr int QW = (NW / GH) * 16;  // new tokens per unit
+  constexpr int kSubs = 64 / QW;      // units per 64-token tile of the host's list
+  static_assert(NW % GH == 0 && QW <= 64 && 64 % QW == 0, "a unit is a whole fraction of a 64-token tile");
+  __shared__ __attribute__((aligned(16))) T lds[WT::kBufs * WT::kElems];
+
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int col = lane % 16, grp = lane / 16;
+  const int g = nh / nkv;
+  const int head_groups = (g + GH - 1) / GH;
+  const int kvh = blockIdx.y / head_groups;
+  const int hsub = (blockIdx.y % head_groups) * GH;
+  const int hw = hsub + wave % GH;
+  const int head = kvh * g + (hw < g ? hw : 0);
+  const T* kp = static_cast<const T*>(kpool);
+  const T* vp = static_cast<const T*>(vpool);
+  const size_t page_stride = static_cast<size_t>(nkv) * bs * HD;  // of both pools, in elements
+  const size_t head_base = static_cast<size_t>(kvh) * bs * HD;
+  const int step_blk = KT / bs, step_off = KT % bs;
+
+  // Where this thread's pieces of a tile lie (the same for every tile).  Piece n is 16 bytes of
+  // the keys and 16 bytes of the values of one 16-key block of the tile, so of one page.
+  // A thread beyond the tile's pieces asks for some piece all the same (every thread issues the
+  // same loads) and only leaves out the store to LDS.
+  int p_blk[PER], p_key[PER], p_vkey[PER], k_off[PER], v_off[PER], k_lds[PER], v_lds[PER];
+  bool p_live[PER];
+#pragma unroll
+  for (int n = 0; n < PER; ++n) {
+    p_live[n] = tid + n * THREADS < WT::kVecs;
+    const int v = (tid + n * THREADS) % WT::kVecs;
+    const int k_row = v / (HD / 8), k_d0 = (v % (HD / 8)) * 8;
+    const int v_d = (v % (HD * 2)) / 2, v_c = (v % 2) * 8;
+    p_blk[n] = v / (HD * 2);                // the 16-key block, the same for both halves
+    p_key[n] = k_row;                       // the key of the tile that the key piece belongs to
+    p_vkey[n] = 16 * p_blk[n] + v_c;        // the first of the eight keys of the value piece
+    k_off[n] = (k_row % 16) * HD + k_d0;    // from the block's first key, in the key pool
+    v_off[n] = v_d * bs + v_c;              // the same in the value pool
+    k_lds[n] = k_row * WT::kKLd + k_d0;
+    // keys 16 blk + c .. + 7 (c = 0 or 8) are lane groups c / 4 and c / 4 + 1 of half blk % 2
+    v_lds[n] = v_d * WT::kVLd + 32 * (p_blk[n] / 2) + 8 * (v_c / 4) + 4 * (p_blk[n] % 2);
+  }
+  auto zero_vec = [] {
+    bf16x8 z;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) z[e] = from_f32<T>(0.f);
+    return z;
+  };
+
+  const int n_units = n_tiles * kSubs;
+  for (int round = 0; round < (paired ? 2 : 1); ++round) {
+    // the host lists tiles in rising order of position
+    int unit = n_units - 1 - static_cast<int>(blockIdx.x);
+    if (round == 1) {
+      if (2 * static_cast<int>(blockIdx.x) >= n_units - 1) break;  // the middle unit has no partner
+      unit = blockIdx.x;
+    }
+    const int tile = unit / kSubs;
+    const int seq = tile_seq[tile];
+    const int tok0 = q_start[seq];
+    const int q_len = q_start[seq + 1] - tok0;
+    const int ctx = ctx_len[seq];
+    const int q0_wg = tile_q0[tile] + (unit % kSubs) * QW;
+    if (q0_wg >= q_len) continue;  // the whole workgroup
+    const int pos_first = ctx - q_len + q0_wg;
+    const int pos_last_wg = pos_first + min(QW, q_len - q0_wg) - 1;
+    const int lo_wg = window > 0 ? max(0, pos_first - window + 1) : 0;
+    const int hi_wg = pos_last_wg + 1;
+
+    // this wave's tokens
+    const int q0_w = q0_wg + (wave / GH) * 16;
+    const bool wave_active = hw < g && q0_w < q_len;
+    const bool col_valid = wave_active && q0_w + col < q_len;
+    const int pos0 = ctx - q_len + q0_w;
+    const int pos_last_w = min(pos_last_wg, pos0 + 15);
+    bf16x8 qf[DSTEPS];
+    {
+      const T* row = q + (static_cast<size_t>(tok0) + q0_w + col) * q_stride + static_cast<size_t>(head) * HD + 8 * grp;
+#pragma unroll
+      for (int s = 0; s < DSTEPS; ++s) qf[s] = col_valid ? *reinterpret_cast<const bf16x8*>(row + 32 * s) : zero_vec();
+    }
+    f32x4 o[kSteps];
+#pragma unroll
+    for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = LYP_NEG_INF;
+    f32x4 lacc = f32x4{0.f, 0.f, 0.f, 0.f};  // every row: the running sum of this column's probabilities
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ones[e] = from_f32<T>(1.f);
+
+    // ---- bringing tiles in.  A thread follows the block of each of its pieces from tile to
+    // tile (index into the table and place in the page, without a division); the table entry is
+    // read one tile ahead of the data, the data two tiles ahead of its use.  Past the last block
+    // that holds a key of interest the table may hold anything, so the index is clamped there.
+    const int32_t* table = block_tables + static_cast<size_t>(seq) * max_blocks;
+    const int blk_last = (hi_wg - 1) / bs;
+    const int kt_first = (lo_wg / KT) * KT;
+    int w_blk[PER], w_off[PER];      // the walk: the block of the tile whose table entry is read next
+    int page[PER], page_off[PER];    // for the tile whose data is asked for next
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      const int x = kt_first + 16 * p_blk[n];
+      w_blk[n] = x / bs;
+      w_off[n] = x - w_blk[n] * bs;
+    }
+    auto read_table = [&](int (&pg)[PER], int (&po)[PER]) {  // for the tile of the walk, which moves on
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        pg[n] = table[min(w_blk[n], blk_last)];
+        po[n] = w_off[n];
+        w_blk[n] += step_blk;
+        w_off[n] += step_off;
+        if (w_off[n] >= bs) {
+          w_off[n] -= bs;
+          w_blk[n] += 1;
+        }
+      }
+    };
+    auto ask = [&](TileRegs<PER>& r, const int (&pg)[PER], const int (&po)[PER]) {
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        r.lost[n] = pg[n] < 0;
+        const size_t base = static_cast<size_t>(max(pg[n], 0)) * page_stride + head_base;
+        r.k[n] = *reinterpret_cast<const bf16x8*>(kp + base + (po[n] * HD + k_off[n]));
+        r.v[n] = *reinterpret_cast<const bf16x8*>(vp + base + (po[n] + v_off[n]));
+      }
+    };
+    // Keys outside [lo_wg, hi_wg) are stored as zeros: a page that was never written, or that
+    // belongs to someone else by now, may hold any bit pattern.
+    auto stash = [&](const TileRegs<PER>& r, int buf, int kt0) {
+      T* ks = lds + buf * WT::kElems;
+      T* vs = ks + KT * WT::kKLd;
+      const bool inside = kt0 >= lo_wg && kt0 + KT <= hi_wg;
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        bf16x8 kx = r.k[n], vx = r.v[n];
+        if (!inside || r.lost[n]) {
+          const int key = kt0 + p_key[n];
+          if (key < lo_wg || key >= hi_wg || r.lost[n]) kx = zero_vec();
+          const int key0 = kt0 + p_vkey[n];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (key0 + e < lo_wg || key0 + e >= hi_wg || r.lost[n]) vx[e] = from_f32<T>(0.f);
+        }
+        if (!p_live[n]) continue;
+        *reinterpret_cast<bf16x8*>(ks + k_lds[n]) = kx;
+        bf16x4 lo_h, hi_h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo_h[e] = vx[e];
+          hi_h[e] = vx[e + 4];
+        }
+        *reinterpret_cast<bf16x4*>(vs + v_lds[n]) = lo_h;
+        *reinterpret_cast<bf16x4*>(vs + v_lds[n] + 8) = hi_h;
+      }
+    };
+
+    // ---- one tile's worth of work for this wave
+    auto compute = [&](int buf, int kt0) {
+      const T* ks = lds + buf * WT::kElems;
+      const T* vs = ks + KT * WT::kKLd;
+      f32x4 sc[NB];
+#pragma unroll
+      for (int u = 0; u < NB; ++u) {
+        const T* krow = ks + (16 * u + col) * WT::kKLd + 8 * grp;
+        sc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DSTEPS; ++s)
+          sc[u] = MMA::mma(*reinterpret_cast<const bf16x8*>(krow + 32 * s), qf[s], sc[u]);
+      }
+      bf16x8 pw[NWIDE];
+      const bool full = kt0 + KT - 1 <= pos0 && kt0 >= lo_wg && pos0 + 15 <= pos_last_wg &&
+                        (window == 0 || kt0 > pos0 + 15 - window);
+      if (full)
+        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, hi_wg, m_run, lacc, o, lane);
+      else
+        softmax_wide<true, NB>(sc, pw, scale_log2, kt0, col_valid ? pos0 + col : -1, window, hi_wg, m_run, lacc, o,
+                               lane);
+#pragma unroll
+      for (int w = 0; w < NWIDE; ++w) {
+        lacc = MMA::mma(ones, pw[w], lacc);
+        const T* vrow = vs + col * WT::kVLd + 32 * w + 8 * grp;
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db)
+          o[db] = MMA::mma(*reinterpret_cast<const bf16x8*>(vrow + db * 16 * WT::kVLd), pw[w], o[db]);
+      }
+    };
+
+    // One round of the loop: tile kt0 is in LDS buffer `buf`, tile kt0 + KT in `ready`; the
+    // loads of tile kt0 + 2 KT are started into `filling`, whose last content is in LDS already.
+    auto step = [&](int kt0, int buf, TileRegs<PER>& filling, const TileRegs<PER>& ready) {
+      int page_n[PER], page_off_n[PER];
+      read_table(page_n, page_off_n);      // for the tile at kt0 + 3 KT
+      ask(filling, page, page_off);        // the tile at kt0 + 2 KT
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        page[n] = page_n[n];
+        page_off[n] = page_off_n[n];
+      }
+      if (wave_active && kt0 <= pos_last_w) compute(buf, kt0);
+      if (WT::kBufs == 1) __syncthreads();  // everyone is done with the only buffer before it is overwritten
+      if (kt0 + KT < hi_wg) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KT);
+      __syncthreads();
+    };
+
+    TileRegs<PER> ra, rb;
+    read_table(page, page_off);
+    ask(ra, page, page_off);     // the first tile
+    read_table(page, page_off);
+    ask(rb, page, page_off);     // the second
+    read_table(page, page_off);  // for the third
+    stash(ra, 0, kt_first);
+    __syncthreads();
+    for (int kt0 = kt_first; kt0 < hi_wg; kt0 += 2 * KT) {
+      step(kt0, 0, ra, rb);
+      if (kt0 + KT >= hi_wg) break;
+      step(kt0 + KT, WT::kBufs == 2 ? 1 : 0, rb, ra);
+    }
+
+    if (col_valid) {
+      const float inv = lacc[0] > 0.f ? 1.0f / lacc[0] : 0.f;
+      T* orow = out + (static_cast<size_t>(tok0) + q0_w + col) * out_stride + static_cast<size_t>(head) * HD + 4 * grp;
+#pragma unroll
+      for (int db = 0; db < kSteps; ++db) {
+        bf16x4 f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = from_f32<T>(o[db][i] * inv);
+        *reinterpret_cast<bf16x4*>(orow + db * 16) = f;
+      }
+    }
+  }
+}
+#endif
+
 // ---------------------------------------------------------------------- decode
 // grid (partitions, nkv * column_groups, requests); kDecodeWaves waves.  A
 // workgroup takes one partition of kDecodeWaves * keys_per_wave keys and merges
@@ -736,6 +1086,20 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   }
 }
 
+// Compute units of the current device (asked once per process).
+static int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
 static int check_common(const char* name, int nh, int nkv, int bs, int max_blocks, int q_stride,
                         int out_stride, int window) {
   LYP_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: %d query heads over %d key/value heads", name, nh, nkv);
@@ -778,7 +1142,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
                      const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* tile_seq,
                      const int32_t* tile_q0, int n_tiles, int nh, int nkv, int bs, int window, float scale,
-                     hipStream_t stream) {
+                     int pair, hipStream_t stream) {
   if (check_common("attn_prefill", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
   LYP_REQUIRE(n_tiles >= 0, "attn_prefill: %d tiles", n_tiles);
   if (n_tiles == 0) return 0;
@@ -804,6 +1168,30 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     else LYP_PREFILL(T, 1, 1);              \
   } while (0)
   constexpr int kQB4 = LYP_PREFILL_QB;
+#if LYP_HEAD_DIM % 32 == 0 && !defined(LYP_PREFILL_NARROW)
+  if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0) {
+    // `pair` is the caller's word on whether the tiles differ much in the keys they see (0: no).
+    // Units (workgroups before pairing) beyond one per compute unit share compute units anyway;
+    // pairing then evens out the causal mask's triangle of work.
+#define LYP_PREFILL_WIDE(GH, NW)                                                                              \
+  do {                                                                                                        \
+    constexpr int kQW = (NW / GH) * 16;                                                                       \
+    const int units = n_tiles * (64 / kQW);                                                                   \
+    const int paired = pair != 0 && static_cast<long long>(units) * nkv * head_groups > compute_units();     \
+    dim3 grid(paired ? (units + 1) / 2 : units, nkv * head_groups);                                           \
+    attn_prefill_wide_kernel<GH, NW><<<grid, NW * kWave, 0, stream>>>(                                        \
+        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,         \
+        block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,          \
+        scale_log2, paired);                                                                                  \
+  } while (0)
+    if (gh == 4) LYP_PREFILL_WIDE(4, 8);
+    else if (gh == 2) LYP_PREFILL_WIDE(2, 8);
+    else LYP_PREFILL_WIDE(1, 4);
+#undef LYP_PREFILL_WIDE
+    LYP_LAUNCH_CHECK("attn_prefill");
+    return 0;
+  }
+#endif
   if (dtype == kF32) LYP_PREFILL_T(float);
   else if (dtype == kBF16) LYP_PREFILL_T(bf16_t);
   else LYP_REQUIRE(false, "attn_prefill: unknown dtype %d", dtype);

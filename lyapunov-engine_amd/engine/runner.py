@@ -100,15 +100,18 @@ class ModelRunner:
         slots = np.asarray([self.cache.state_slot(e.seq_id) for e in entries], dtype=np.int32)
         rows = np.asarray([q_start[b] + w for b, e in enumerate(entries) for w in e.want], dtype=np.int32)
 
-        tile_seq, tile_q0, dec = [], [], []
+        tiles, dec = [], []   # tiles: (keys up to the tile's last token, request, first token)
         for b, e in enumerate(entries):
             n = len(e.tokens)
             if n == 1:
                 dec.append(b)
             else:
                 for q0 in range(0, n, PREFILL_TILE):
-                    tile_seq.append(b)
-                    tile_q0.append(q0)
+                    tiles.append((e.start + min(n, q0 + PREFILL_TILE), b, q0))
+        tiles.sort()          # the attention kernel starts (or pairs) tiles by the work they are
+        tile_seq = [t[1] for t in tiles]
+        tile_q0 = [t[2] for t in tiles]
+        tile_keys = (tiles[0][0], tiles[-1][0]) if tiles else (0, 0)
         max_ctx_dec = max((int(ctx_len[b]) for b in dec), default=0)
 
         sections = [token_ids, positions, np.asarray(q_start, dtype=np.int32), ctx_len, slots, rows,
@@ -150,7 +153,8 @@ class ModelRunner:
         return StepContext(
             device=self.device, dtype=self.dtype, T=T, B=B, token_ids=view(0), positions=view(1), q_start=view(2),
             ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=int(rows.size), groups=groups,
-            tile_seq=view(6), tile_q0=view(7), n_tiles=len(tile_seq), dec_seqs=view(8) if dec else None,
+            tile_seq=view(6), tile_q0=view(7), n_tiles=len(tile_seq), tile_keys=tile_keys,
+            dec_seqs=view(8) if dec else None,
             n_dec=len(dec), max_ctx_dec=max_ctx_dec, q_start_host=q_start, ctx_len_host=ctx_len.tolist(),
             state_slots_host=slots.tolist(), workspace=self.workspace)
 

@@ -73,8 +73,11 @@ class PagedAttention(Mixer):
         common = dict(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                       window=self.window, scale=self.scale)
         if ctx.n_tiles:
+            # Tiles come in rising order of the keys they see; when the first sees less than half
+            # of what the last does, a workgroup may take one from each end.
+            few, many = (min(k, self.window + 64) if self.window else k for k in ctx.tile_keys)
             ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.tile_seq,
-                             ctx.tile_q0, ctx.n_tiles, **common)
+                             ctx.tile_q0, ctx.n_tiles, pair=2 * few <= many, **common)
         if ctx.n_dec:
             part = ops.attn_decode_plan(ctx.n_dec, ctx.max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
             max_parts = max(1, (ctx.max_ctx_dec + part - 1) // part)

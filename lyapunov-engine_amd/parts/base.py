@@ -143,6 +143,7 @@ class StepContext:
     ctx_len_host: list = field(default_factory=list)
     state_slots_host: list = field(default_factory=list)
     workspace: dict = field(default_factory=dict)   # scratch tensors shared by the layers of a step
+    tile_keys: tuple = (0, 0)             # keys up to the last token of the first and of the last tile
 
     def scratch(self, key: str, numel: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
         t = self.workspace.get(key)

@@ -256,6 +256,11 @@ PREFILL_CASES = [
     (4, 2, 32, 4, 9, [(50, 50), (33, 6), (20, 2)]),
     (2, 1, 64, 16, 40, [(200, 100), (41, 3)]),
     (16, 1, 16, 2, 0, [(23, 11)]),  # a page size that is no multiple of 4: the scalar load path
+    # enough work that a workgroup takes a heavy and a light run of tokens, one after the other
+    (32, 8, 64, 16, 0, [(2065, 2065)]),
+    (16, 8, 32, 16, 300, [(1500, 1500), (900, 500), (65, 65), (64, 64)]),
+    (8, 8, 128, 16, 0, [(2100, 2100)]),
+    (2, 1, 256, 16, 0, [(100, 100), (40, 3)]),
 ]
 
 
