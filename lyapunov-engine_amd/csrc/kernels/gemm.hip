@@ -145,14 +145,39 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
 //
 // Epilogues: store in the operands' type; store float; SiLU-gate (rows 0-7 of
 // the tile are gate features, rows 8-15 the matching up features: the output
-// has half as many columns); or float partial sums per slice, [slice][M][N],
-// which the consumer adds up (the RMSNorm kernels do).
-enum SkinnyEpilogue : int { kEpiAct = 0, kEpiF32 = 1, kEpiSwiglu = 2, kEpiParts = 3 };
+// has half as many columns); float partial sums per slice, [slice][M][N],
+// which the consumer adds up (the RMSNorm kernels do); or the whole tail of a
+// fused q/k/v projection: rotate query and key heads by position and put keys
+// and values into their pages.
+enum SkinnyEpilogue : int { kEpiAct = 0, kEpiF32 = 1, kEpiSwiglu = 2, kEpiParts = 3, kEpiRope = 4 };
+
+// What the rotating epilogue needs.  W's rows are heads of `hd` features: nh
+// query heads, then (has_kv) nkv key heads and nkv value heads.  In the first
+// `rot` features of a query or key head, feature i < rot / 2 is rotated with
+// feature i + rot / 2 (rope_kv_kernel has the formula); a workgroup of such a
+// region therefore does not take 16 neighbouring rows of W but features
+// 8 t .. 8 t + 7 and their partners, so that both halves of a pair meet in it.
+struct RopeTail {
+  const int32_t* positions;  // [M]
+  const float* cos_sin;      // [max_pos][rot]: cosines, then sines; unused when rot == 0
+  const int32_t* slots;      // [M] page * bs + offset of the token's key and value, -1: not stored
+  void* kpool;               // [page][nkv][bs][hd]
+  void* vpool;               // [page][nkv][hd][bs]
+  int nh, nkv, hd, rot, bs, has_kv;
+};
+
+// The feature (row of W, column of the output) that row r of the 16-row tile at n0 stands for.
+__device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
+  const int head = n0 / t.hd, blk = (n0 % t.hd) / 16;
+  const bool rotated = head < t.nh + (t.has_kv ? t.nkv : 0) && blk < t.rot / 16;
+  const int f = rotated ? (r < 8 ? 8 * blk + r : t.rot / 2 + 8 * blk + (r - 8)) : 16 * blk + r;
+  return head * t.hd + f;
+}
 
 template <typename T, int MB, int EPI>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
-                                                           int ldw, int ldc) {
+                                                           int ldw, int ldc, RopeTail tail) {
   using MM = Mma16Wide<T>;
   using Frag = typename MM::Frag;
   constexpr int NF = 16 / MM::kElems;  // fragments per lane per 64 values of K
@@ -162,7 +187,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   const int nwaves = blockDim.x / kWave;
   const int n0 = blockIdx.x * 16;
   const int r = lane % 16, j = lane / 16;
-  const int wrow = min(n0 + r, N - 1);  // rows past the end read the last row and are not stored
+  int wrow = min(n0 + r, N - 1);  // rows past the end read the last row and are not stored
+  if constexpr (EPI == kEpiRope) wrow = rope_feature(tail, n0, r);  // N is a multiple of 16 here
 
   const int chunks = K / 64;
   const int per_slice = (chunks + gridDim.y - 1) / gridDim.y;
@@ -210,7 +236,42 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     const int row = 4 * (l / 16) + i;
     const int m = b * 16 + l % 16, n = n0 + row;
     if (m >= M || n >= N) continue;
-    if constexpr (EPI == kEpiSwiglu) {
+    if constexpr (EPI == kEpiRope) {
+      const int head = n0 / tail.hd, blk = (n0 % tail.hd) / 16;
+      const bool is_q = head < tail.nh, is_k = !is_q && head < tail.nh + tail.nkv;
+      const bool rotated = (is_q || is_k) && blk < tail.rot / 16;
+      if (rotated && row >= 8) continue;  // done by the thread of the partner
+      // as two kernels would do it: the product rounded to the activations' type, then rotated
+      T y0 = from_f32<T>(total(e)), y1 = y0;
+      int f0 = 16 * blk + row, f1 = f0;
+      if (rotated) {
+        const int half = tail.rot / 2, fi = 8 * blk + row;
+        const float* cs = tail.cos_sin + static_cast<size_t>(tail.positions[m]) * tail.rot;
+        const float c = cs[fi], sn = cs[half + fi];
+        const float x0 = to_f32(y0), x1 = to_f32(from_f32<T>(total(e + 128)));  // the same token, row + 8
+        y0 = from_f32<T>(x0 * c - x1 * sn);
+        y1 = from_f32<T>(x1 * c + x0 * sn);
+        f0 = fi;
+        f1 = fi + half;
+      }
+      if (is_q) {
+        T* orow = static_cast<T*>(Cv) + static_cast<size_t>(m) * ldc + head * tail.hd;
+        orow[f0] = y0;
+        if (rotated) orow[f1] = y1;
+        continue;
+      }
+      const int slot = tail.slots[m];
+      if (slot < 0) continue;
+      const size_t page = slot / tail.bs, off = slot % tail.bs;
+      if (is_k) {
+        T* krow = static_cast<T*>(tail.kpool) + ((page * tail.nkv + (head - tail.nh)) * tail.bs + off) * tail.hd;
+        krow[f0] = y0;
+        if (rotated) krow[f1] = y1;
+      } else {
+        T* vhead = static_cast<T*>(tail.vpool) + (page * tail.nkv + (head - tail.nh - tail.nkv)) * tail.hd * tail.bs;
+        vhead[static_cast<size_t>(f0) * tail.bs + off] = y0;
+      }
+    } else if constexpr (EPI == kEpiSwiglu) {
       if (row >= 8) continue;
       const float gate = total(e), up = total(e + 128);  // the same token, row + 8
       static_cast<T*>(Cv)[static_cast<size_t>(m) * ldc + (n0 / 2 + row)] =
@@ -252,13 +313,13 @@ static int skinny_waves(int N, int K, int MB, int slices) {
 
 template <typename T, int EPI>
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
-                          int slices, hipStream_t stream) {
+                          int slices, hipStream_t stream, const RopeTail& tail = RopeTail{}) {
   const int MB = (M + 15) / 16;
   const int waves = skinny_waves(N, K, MB, slices);
   const dim3 grid((N + 15) / 16, slices), block(waves * kWave);
   const size_t lds = static_cast<size_t>(waves) * MB * 256 * sizeof(float);
 #define LYP_SKINNY(MBV) \
-  gemm_skinny_kernel<T, MBV, EPI><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc)
+  gemm_skinny_kernel<T, MBV, EPI><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, tail)
   if (MB == 1) LYP_SKINNY(1);
   else if (MB == 2) LYP_SKINNY(2);
   else if (MB == 3) LYP_SKINNY(3);
@@ -367,5 +428,35 @@ extern "C" int lyp_gemm_swiglu(const void* A, const void* W, void* out, int dtyp
   else
     LYP_REQUIRE(false, "gemm_swiglu: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gemm_swiglu");
+  return 0;
+}
+
+// The fused q/k/v projection of a step with few rows, finished in one kernel:
+// out[M, nh * hd] receives the query heads, rotated; the key heads, rotated,
+// and the value heads go to the pages that `slots` names (see RopeTail; what
+// lyp_gemm_nt followed by lyp_rope_kv_write does, to the last bit).  W has
+// (nh + 2 nkv) * hd rows, or nh * hd without has_kv.  Returns 1 (and does
+// nothing) when the few-rows kernel does not apply or the rotated part of a
+// head is no multiple of 16.
+extern "C" int lyp_gemm_rope_kv(const void* A, const void* W, void* out, int dtype, int M, int K, int lda, int ldw,
+                                int ldo, const int32_t* positions, const float* cos_sin, const int32_t* slots,
+                                void* kpool, void* vpool, int nh, int nkv, int hd, int rot, int bs, int has_kv,
+                                hipStream_t stream) {
+  LYP_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_rope_kv: %d heads, %d key/value heads of %d", nh,
+              nkv, hd);
+  LYP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "gemm_rope_kv: rotary size %d of head size %d", rot, hd);
+  LYP_REQUIRE(positions && (rot == 0 || cos_sin), "gemm_rope_kv: positions and the rotation table are needed");
+  LYP_REQUIRE(!has_kv || (slots && kpool && vpool && bs > 0 && nkv > 0), "gemm_rope_kv: no pages to store to");
+  const int N = (has_kv ? nh + 2 * nkv : nh) * hd;
+  LYP_REQUIRE(ldo >= nh * hd, "gemm_rope_kv: output stride %d", ldo);
+  if (rot % 16 != 0 || !skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
+  const RopeTail tail{positions, cos_sin, slots, kpool, vpool, nh, nkv, hd, rot, bs, has_kv};
+  if (dtype == kF32)
+    launch_skinny<float, kEpiRope>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiRope>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
+  else
+    LYP_REQUIRE(false, "gemm_rope_kv: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_rope_kv");
   return 0;
 }

@@ -55,6 +55,9 @@ def core() -> ctypes.CDLL:
                                           c_int, c_void_p]
         lib.lyp_gemm_swiglu.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                         c_int, c_void_p]
+        lib.lyp_gemm_rope_kv.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                         c_int, c_int, c_int, c_void_p]
         lib.lyp_cast.argtypes = [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p]
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
@@ -173,16 +176,11 @@ def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Te
     return out
 
 
-def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor | None,
-                  slots: torch.Tensor | None, kpool: torch.Tensor | None, vpool: torch.Tensor | None, *, num_heads: int,
-                  num_kv_heads: int, head_dim: int, page_size: int, has_kv: bool = True) -> None:
-    """Rotate the query (and key) heads of ``qkv`` in place by each token's
-    position and store keys and values in the token's cache slot."""
-    _dev(qkv, positions, cos_sin, slots, kpool, vpool)
-    T = qkv.shape[0]
-    width = (num_heads + 2 * num_kv_heads) * head_dim if has_kv else num_heads * head_dim
-    if qkv.shape[1] != width or positions.numel() != T or positions.dtype != torch.int32:
-        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} against width {width}, positions {tuple(positions.shape)}")
+def _rope_check(T: int, dtype: torch.dtype, positions, cos_sin, slots, kpool, vpool, num_kv_heads: int,
+                head_dim: int, page_size: int, has_kv: bool) -> int:
+    """Checks the operands that the rotation and the page write share; returns the rotary size."""
+    if positions.numel() != T or positions.dtype != torch.int32:
+        raise KernelError(f"rope_kv_write: positions {tuple(positions.shape)} {positions.dtype} for {T} tokens")
     rot = 0
     if cos_sin is not None:
         rot = cos_sin.shape[1]
@@ -193,9 +191,23 @@ def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Ten
         if (slots is None or slots.numel() != T or slots.dtype != torch.int32
                 or tuple(kpool.shape) != (n_pages, num_kv_heads, page_size, head_dim)
                 or tuple(vpool.shape) != (n_pages, num_kv_heads, head_dim, page_size)
-                or kpool.dtype != qkv.dtype or vpool.dtype != qkv.dtype):
+                or kpool.dtype != dtype or vpool.dtype != dtype):
             raise KernelError(f"rope_kv_write: pools {tuple(kpool.shape)} / {tuple(vpool.shape)} {kpool.dtype} do not "
-                              f"fit {num_kv_heads} heads of {head_dim}, pages of {page_size}, dtype {qkv.dtype}")
+                              f"fit {num_kv_heads} heads of {head_dim}, pages of {page_size}, dtype {dtype}")
+    return rot
+
+
+def rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor | None,
+                  slots: torch.Tensor | None, kpool: torch.Tensor | None, vpool: torch.Tensor | None, *, num_heads: int,
+                  num_kv_heads: int, head_dim: int, page_size: int, has_kv: bool = True) -> None:
+    """Rotate the query (and key) heads of ``qkv`` in place by each token's
+    position and store keys and values in the token's cache slot."""
+    _dev(qkv, positions, cos_sin, slots, kpool, vpool)
+    T = qkv.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim if has_kv else num_heads * head_dim
+    if qkv.shape[1] != width:
+        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} against width {width}")
+    rot = _rope_check(T, qkv.dtype, positions, cos_sin, slots, kpool, vpool, num_kv_heads, head_dim, page_size, has_kv)
     lib = core()
     _check(lib.lyp_rope_kv_write(_p(qkv), _code(qkv.dtype), _p(positions), _p(cos_sin), _p(slots), _p(kpool),
                                  _p(vpool), T, num_heads, num_kv_heads, head_dim, rot, page_size, int(has_kv),
@@ -213,6 +225,40 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleave: int = 0) -> tor
     lib = core()
     _check(lib.lyp_swiglu(_p(gate_up), _p(out), _code(out.dtype), T, I, interleave, _stream()), lib)
     return out
+
+
+def linear_rope_kv(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, cos_sin: torch.Tensor | None,
+                   slots: torch.Tensor | None, kpool: torch.Tensor | None, vpool: torch.Tensor | None, *,
+                   num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                   has_kv: bool = True) -> torch.Tensor:
+    """The fused q/k/v projection of x (w: query heads, then key heads, then
+    value heads; query heads alone without ``has_kv``), query and key heads
+    rotated by position, keys and values stored in the tokens' cache slots.
+    Returns a tensor whose first ``num_heads * head_dim`` columns are the
+    rotated query heads.  With few rows this is one kernel; its results equal
+    ``linear`` followed by ``rope_kv_write`` bit for bit."""
+    M, K = x.shape
+    N = w.shape[0]
+    width = (num_heads + 2 * num_kv_heads) * head_dim if has_kv else num_heads * head_dim
+    if N != width or w.shape[1] != K:
+        raise KernelError(f"linear_rope_kv: weight {tuple(w.shape)} for {width} features of {K}")
+    if w.dtype == x.dtype and M <= 64 and not _library_product(M, N, K, x.dtype):
+        _dev(x, w, positions, cos_sin, slots, kpool, vpool)
+        rot = _rope_check(M, x.dtype, positions, cos_sin, slots, kpool, vpool, num_kv_heads, head_dim, page_size,
+                          has_kv)
+        out = torch.empty((M, num_heads * head_dim), dtype=x.dtype, device=x.device)
+        lib = core()
+        rc = lib.lyp_gemm_rope_kv(_p(x), _p(w), _p(out), _code(x.dtype), M, K, x.stride(0), w.stride(0),
+                                  out.stride(0), _p(positions), _p(cos_sin), _p(slots), _p(kpool), _p(vpool),
+                                  num_heads, num_kv_heads, head_dim, rot, page_size, int(has_kv), _stream())
+        if rc == 0:
+            return out
+        if rc < 0:
+            _check(rc, lib)
+    qkv = linear(x, w, out_dtype=x.dtype)
+    rope_kv_write(qkv, positions, cos_sin, slots, kpool, vpool, num_heads=num_heads, num_kv_heads=num_kv_heads,
+                  head_dim=head_dim, page_size=page_size, has_kv=has_kv)
+    return qkv
 
 
 def linear_swiglu(x: torch.Tensor, w: torch.Tensor, interleave: int) -> torch.Tensor:

@@ -64,11 +64,10 @@ class PagedAttention(Mixer):
         if cache.writes != self.own_kv:
             raise RuntimeError("a mixer with its own keys must write the cache, one without must not")
         g = cache.group
-        qkv = ops.linear(x, self.qkv_proj, out_dtype=ctx.dtype)
         table = self.position.table if self.position is not None else None
-        ops.rope_kv_write(qkv, ctx.positions, table, g.slot_mapping, cache.k, cache.v, num_heads=self.num_heads,
-                          num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, page_size=g.page_size,
-                          has_kv=self.own_kv)
+        qkv = ops.linear_rope_kv(x, self.qkv_proj, ctx.positions, table, g.slot_mapping, cache.k, cache.v,
+                                 num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+                                 page_size=g.page_size, has_kv=self.own_kv)
         out = torch.empty((ctx.T, self.num_heads * self.head_dim), dtype=ctx.dtype, device=x.device)
         common = dict(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                       window=self.window, scale=self.scale)

@@ -205,6 +205,48 @@ def test_rope_kv_write(ops, dtype, nh, nkv, hd, bs):
     assert int((kp.abs().sum(-1) > 0).sum()) == written * nkv  # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs,T,has_kv", [
+    (32, 8, 64, 64, 16, 8, True), (6, 2, 48, 48, 8, 1, True), (4, 4, 16, 16, 4, 19, True),
+    (3, 1, 128, 32, 16, 64, True),   # only part of a head is rotated
+    (5, 1, 32, 0, 16, 7, True),      # no rotation at all
+    (4, 2, 64, 64, 16, 33, False),   # a layer that reads another layer's keys: query heads only
+    (2, 1, 80, 40, 16, 5, True),     # a rotary size that is no multiple of 16: two kernels
+])
+def test_projection_with_rotation_and_page_write_in_one_kernel(ops, dtype, nh, nkv, hd, rot, bs, T, has_kv):
+    """The fused q/k/v projection gives, bit for bit, what the product followed
+    by the rotation and page-write kernel gives (which has its own test above)."""
+    K, n_pages, max_pos = 192, 9, 300
+    width = (nh + 2 * nkv) * hd if has_kv else nh * hd
+    x = rnd(T, K, dtype=dtype, seed=21).to(DEV)
+    w = (rnd(width, K, dtype=dtype, seed=22) * 0.3).to(DEV)
+    positions = torch.randint(0, max_pos, (T,), generator=torch.Generator().manual_seed(23)).to(torch.int32).to(DEV)
+    table = None
+    if rot:
+        cos, sin = P.rope_cos_sin(torch.arange(max_pos), P.rope_inv_freq(rot, 10000.0))
+        table = torch.cat((cos[:, : rot // 2], sin[:, : rot // 2]), dim=-1).contiguous().to(DEV)
+    slots = torch.randperm(n_pages * bs, generator=torch.Generator().manual_seed(24))[:T].to(torch.int32)
+    slots[T // 2] = -1
+    slots = slots.to(DEV)
+    kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd, page_size=bs, has_kv=has_kv)
+
+    def pools():
+        if not has_kv:
+            return None, None
+        return (torch.full((n_pages, nkv, bs, hd), 7.0, dtype=dtype, device=DEV),
+                torch.full((n_pages, nkv, hd, bs), 7.0, dtype=dtype, device=DEV))
+
+    k1, v1 = pools()
+    two = ops.linear(x, w, out_dtype=dtype)
+    ops.rope_kv_write(two, positions, table, slots if has_kv else None, k1, v1, **kw)
+    k2, v2 = pools()
+    one = ops.linear_rope_kv(x, w, positions, table, slots if has_kv else None, k2, v2, **kw)
+    assert torch.equal(one[:, : nh * hd], two[:, : nh * hd])
+    if has_kv:
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+        assert int((k2 != 7.0).any(-1).sum()) == (T - 1) * nkv  # the token without a slot stored nothing
+
+
 # ------------------------------------------------------------------- attention
 def paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=0, n_pages=None):
     """seqs: list of (ctx_len, q_len).  Random q for the new tokens, k/v for the
