@@ -200,22 +200,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const T* wp = W + static_cast<size_t>(wrow) * ldw + j * 16;
+  // of 64 values of K, fragment f of lane group j holds values 4 E f + E j .. + E - 1 (E = MM::kElems): the
+  // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
+  const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems;
   const T* ap[MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * 16;
+  for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * MM::kElems;
 
 #pragma unroll 4
   for (int c = c_begin; c < c_end; ++c) {
     const int k0 = c * 64;
     Frag wf[NF];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) wf[f] = *reinterpret_cast<const Frag*>(wp + k0 + f * MM::kElems);
+    for (int f = 0; f < NF; ++f) wf[f] = *reinterpret_cast<const Frag*>(wp + k0 + f * 4 * MM::kElems);
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
       Frag xf[NF];
 #pragma unroll
-      for (int f = 0; f < NF; ++f) xf[f] = *reinterpret_cast<const Frag*>(ap[b] + k0 + f * MM::kElems);
+      for (int f = 0; f < NF; ++f) xf[f] = *reinterpret_cast<const Frag*>(ap[b] + k0 + f * 4 * MM::kElems);
 #pragma unroll
       for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[f], xf[f], acc[b]);
     }
