@@ -1,0 +1,129 @@
+"""Times one kernel of the package alone, on random data of a chosen shape.
+
+    python -m lyapunov_engine_amd.utils.kernel_bench attn_prefill --tokens 8192
+    python -m lyapunov_engine_amd.utils.kernel_bench attn_decode --batch 8 --context 8192
+    python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 8 --out-features 16384 --in-features 2048
+
+Prints the time per call and what it means in TFLOP/s or TB/s.  Small enough to
+run under ``rocprofv3 --pmc ...`` when a kernel's counters are wanted; the
+defaults are the Llama-3.2-1B shapes that bench.py runs.
+"""
+from __future__ import annotations
+
+import argparse
+
+import torch
+
+from ..kernels import ops
+
+
+def _time(fn, repeat: int) -> float:
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(repeat):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / repeat * 1e-3
+
+
+def _dtype(name: str) -> torch.dtype:
+    return {"bf16": torch.bfloat16, "fp32": torch.float32}[name]
+
+
+def _pools(pages: int, a) -> tuple:
+    dt, dev = _dtype(a.dtype), a.device
+    k = torch.randn(pages, a.kv_heads, a.page_size, a.head_dim, device=dev, dtype=dt)
+    v = torch.randn(pages, a.kv_heads, a.head_dim, a.page_size, device=dev, dtype=dt)
+    return k, v
+
+
+def attn_prefill(a) -> None:
+    """One request brings ``tokens`` new tokens and ends at ``context`` keys."""
+    dt, dev = _dtype(a.dtype), a.device
+    S, ctx = a.tokens, max(a.context or a.tokens, a.tokens)
+    pages = -(-ctx // a.page_size)
+    k, v = _pools(pages, a)
+    table = torch.arange(pages, dtype=torch.int32, device=dev).view(1, pages)
+    q = torch.randn(S, (a.heads + 2 * a.kv_heads) * a.head_dim, device=dev, dtype=dt)
+    out = torch.empty(S, a.heads * a.head_dim, device=dev, dtype=dt)
+    q_start = torch.tensor([0, S], dtype=torch.int32, device=dev)
+    ctx_len = torch.tensor([ctx], dtype=torch.int32, device=dev)
+    n_tiles = -(-S // 64)
+    tile_seq = torch.zeros(n_tiles, dtype=torch.int32, device=dev)
+    tile_q0 = (torch.arange(n_tiles, dtype=torch.int32) * 64).to(dev)
+    pair = 2 * (ctx - S + 64) <= ctx
+
+    def run():
+        ops.attn_prefill(q, out, k, v, table, q_start, ctx_len, tile_seq, tile_q0, n_tiles, num_heads=a.heads,
+                         num_kv_heads=a.kv_heads, head_dim=a.head_dim, pair=pair)
+
+    t = _time(run, a.repeat)
+    flops = 4 * a.heads * a.head_dim * (S * (ctx - S) + S * S / 2)
+    print(f"attn_prefill tokens={S} context={ctx} heads={a.heads}/{a.kv_heads}x{a.head_dim} {a.dtype}: "
+          f"{t * 1e6:.1f} us  {flops / t / 1e12:.1f} TFLOP/s")
+
+
+def attn_decode(a) -> None:
+    """``batch`` requests with ``context`` keys each bring one token."""
+    dt, dev = _dtype(a.dtype), a.device
+    B, ctx = a.batch, a.context or 8192
+    per = -(-ctx // a.page_size)
+    k, v = _pools(B * per, a)
+    table = torch.arange(B * per, dtype=torch.int32, device=dev).view(B, per)
+    q = torch.randn(B, (a.heads + 2 * a.kv_heads) * a.head_dim, device=dev, dtype=dt)
+    out = torch.empty(B, a.heads * a.head_dim, device=dev, dtype=dt)
+    q_start = torch.arange(B + 1, dtype=torch.int32, device=dev)
+    ctx_len = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    part = ops.attn_decode_plan(B, ctx, a.heads, a.kv_heads, a.head_dim)
+    max_parts = -(-ctx // part)
+    part_o = torch.empty(B * a.heads * max_parts * a.head_dim, device=dev)
+    part_ml = torch.empty(B * a.heads * max_parts * 2, device=dev)
+
+    def run():
+        ops.attn_decode(q, out, k, v, table, q_start, ctx_len, None, B, part_o, part_ml, max_parts, part,
+                        num_heads=a.heads, num_kv_heads=a.kv_heads, head_dim=a.head_dim)
+
+    t = _time(run, a.repeat)
+    nbytes = 2 * B * ctx * a.kv_heads * a.head_dim * k.element_size()
+    print(f"attn_decode batch={B} context={ctx} heads={a.heads}/{a.kv_heads}x{a.head_dim} {a.dtype}: "
+          f"{t * 1e6:.1f} us  {nbytes / t / 1e12:.2f} TB/s of keys and values ({max_parts} partitions of {part})")
+
+
+def linear(a) -> None:
+    dt, dev = _dtype(a.dtype), a.device
+    x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
+    w = torch.randn(a.out_features, a.in_features, device=dev, dtype=dt) * 0.02
+    t = _time(lambda: ops.linear(x, w, may_split=a.may_split), a.repeat)
+    flops = 2.0 * a.rows * a.in_features * a.out_features
+    print(f"linear rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}: {t * 1e6:.1f} us  "
+          f"{flops / t / 1e12:.1f} TFLOP/s  {w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
+
+
+def main(argv=None) -> None:
+    ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--repeat", type=int, default=20)
+    ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--kv-heads", type=int, default=8)
+    ap.add_argument("--head-dim", type=int, default=64)
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--tokens", type=int, default=2048, help="attn_prefill: new tokens of the request")
+    ap.add_argument("--context", type=int, default=0, help="keys per request after the step")
+    ap.add_argument("--batch", type=int, default=8, help="attn_decode: requests")
+    ap.add_argument("--rows", type=int, default=8, help="linear: rows of activations")
+    ap.add_argument("--in-features", type=int, default=2048)
+    ap.add_argument("--out-features", type=int, default=16384)
+    ap.add_argument("--may-split", action="store_true", help="linear: allow partial sums over slices of K")
+    a = ap.parse_args(argv)
+    ops.require_gpu()
+    torch.manual_seed(0)
+    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear}[a.kernel](a)
+
+
+if __name__ == "__main__":
+    main()
