@@ -12,6 +12,8 @@
 // sizes of the product alone (no atomics), so a token's result does not depend
 // on which other tokens are in the batch beyond the choice of kernel, which
 // follows M.
+#include <type_traits>
+
 #include "common.h"
 
 namespace lyp {
@@ -149,7 +151,32 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
 // which the consumer adds up (the RMSNorm kernels do); or the whole tail of a
 // fused q/k/v projection: rotate query and key heads by position and put keys
 // and values into their pages.
-enum SkinnyEpilogue : int { kEpiAct = 0, kEpiF32 = 1, kEpiSwiglu = 2, kEpiParts = 3, kEpiRope = 4 };
+enum SkinnyEpilogue : int {
+  kEpiAct = 0, kEpiF32 = 1, kEpiSwiglu = 2, kEpiParts = 3, kEpiRope = 4,
+  kEpiResidual = 5,  // C is the float residual stream: C += A . W^T
+};
+
+// The residual epilogue's by-products for the RMS norm that follows: with
+// h' = h + A . W^T it also stores xs = h' * next_weight (rounded to the
+// operands' type, not yet divided by the row's rms) and, per workgroup, the
+// sum of h'^2 over the workgroup's features.
+struct ResidualTail {
+  const void* next_w;  // [N] the following norm's weights; null: no by-products
+  int next_w_f32;
+  void* xs;            // [M][ldx]
+  int ldx;
+  float* ssq_part;     // [workgroups][16]: rows past M get zeros
+};
+
+// For a product whose activations are such an xs: the sums are scaled by the
+// row's 1 / sqrt(mean(h'^2) + eps), from the n_parts partial sums of squares
+// (added up in a fixed order), before the epilogue proper.  `width` is the
+// number of features of h'.
+struct NormHead {
+  const float* ssq_part;  // [n_parts][16]
+  int n_parts, width;
+  float eps;
+};
 
 // What the rotating epilogue needs.  W's rows are heads of `hd` features: nh
 // query heads, then (has_kv) nkv key heads and nkv value heads.  In the first
@@ -174,20 +201,25 @@ __device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
   return head * t.hd + f;
 }
 
-template <typename T, int MB, int EPI>
+template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
-                                                           int ldw, int ldc, RopeTail tail) {
+                                                           int ldw, int ldc, RopeTail tail, NormHead head,
+                                                           ResidualTail res) {
   using MM = Mma16Wide<T>;
   using Frag = typename MM::Frag;
   constexpr int NF = 16 / MM::kElems;  // fragments per lane per 64 values of K
-  extern __shared__ float red[];       // [waves][MB][64][4]
+  static_assert(ROWS == 16 || ROWS == 8, "a workgroup owns 16 rows of W, or 8 (the tile's lower half repeats them)");
+  extern __shared__ float red[];       // [waves][MB][64][4], then MB * 16 floats for the epilogues' row values
 
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  // the same in every lane, and said so: the loop over this wave's share of K then has scalar bounds and
+  // can be unrolled, which is what keeps several chunks' loads in flight
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nwaves = blockDim.x / kWave;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * ROWS;
   const int r = lane % 16, j = lane / 16;
-  int wrow = min(n0 + r, N - 1);  // rows past the end read the last row and are not stored
+  int wrow = min(n0 + r % ROWS, N - 1);  // rows past the end read the last row and are not stored
   if constexpr (EPI == kEpiRope) wrow = rope_feature(tail, n0, r);  // N is a multiple of 16 here
 
   const int chunks = K / 64;
@@ -200,44 +232,107 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Small loads that the epilogue needs are started here, ahead of the stream of weights.
+  float* row_val = red + static_cast<size_t>(nwaves) * MB * 256;  // [waves][16]
+  if constexpr (NORMED) {
+    // Every token's sum of squares, from the producer's partial sums [parts][16]: thread t adds up
+    // four tokens (t % 4) over every (threads / 4)-th part, the lanes of a wave meet by shuffles, the
+    // waves in the epilogue (row_val[wave][token]).  The order is fixed by the launch.
+    static_assert(MB == 1, "sums of squares come for at most 16 rows");
+    const f32x4* src = reinterpret_cast<const f32x4*>(head.ssq_part);
+    const int n4 = head.n_parts * 4;  // 16-byte pieces: piece i holds tokens 4 (i % 4) .. + 3 of part i / 4
+    f32x4 sq = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int base = threadIdx.x; base < n4; base += 4 * blockDim.x) {
+      f32x4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * blockDim.x;
+        v[u] = idx < n4 ? src[idx] : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) sq += v[u];
+    }
+#pragma unroll
+    for (int off = 4; off < kWave; off *= 2)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sq[i] += __shfl_xor(sq[i], off, kWave);
+    if (lane < 4) *reinterpret_cast<f32x4*>(row_val + wave * 16 + 4 * lane) = sq;
+  }
+  float h_first = 0.f, nw_first = 0.f;  // kEpiResidual: what the thread's first element adds to and is weighted by
+  if constexpr (EPI == kEpiResidual) {
+    const int e = threadIdx.x, l = (e % 256) / 4, row = 4 * (l / 16) + e % 4;
+    const int m = (e / 256) * 16 + l % 16, n = n0 + row;
+    if (e < MB * 256 && row < ROWS && m < M && n < N) {
+      h_first = static_cast<const float*>(Cv)[static_cast<size_t>(m) * ldc + n];
+      if (res.next_w)
+        nw_first = res.next_w_f32 ? static_cast<const float*>(res.next_w)[n]
+                                  : to_f32(static_cast<const bf16_t*>(res.next_w)[n]);
+    }
+  }
+
   // of 64 values of K, fragment f of lane group j holds values 4 E f + E j .. + E - 1 (E = MM::kElems): the
   // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
   const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems;
-  const T* ap[MB];
+  const T* ap[MB];  // rows past the end read the last row and are not stored
 #pragma unroll
   for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * MM::kElems;
 
-#pragma unroll 4
-  for (int c = c_begin; c < c_end; ++c) {
-    const int k0 = c * 64;
-    Frag wf[NF];
+  // U chunks of 64 values of K at once: all of their loads are asked for before the first product
+  // needs one.  (The matrix instruction counts as a convergent operation, and the compiler does not
+  // unroll a loop of unknown length around one by itself: hence the two loops written out.)
+  auto chunks_at = [&](auto count, int c) {
+    constexpr int U = decltype(count)::value;
+    Frag wf[U][NF];
 #pragma unroll
-    for (int f = 0; f < NF; ++f) wf[f] = *reinterpret_cast<const Frag*>(wp + k0 + f * 4 * MM::kElems);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int f = 0; f < NF; ++f)
+        wf[u][f] = *reinterpret_cast<const Frag*>(wp + (c + u) * 64 + f * 4 * MM::kElems);
+    // the activations come from the cache: four chunks of them at a time are enough
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      Frag xf[NF];
 #pragma unroll
-      for (int f = 0; f < NF; ++f) xf[f] = *reinterpret_cast<const Frag*>(ap[b] + k0 + f * 4 * MM::kElems);
+      for (int u0 = 0; u0 < U; u0 += 4) {
+        constexpr int V = U < 4 ? U : 4;
+        Frag xf[V][NF];
 #pragma unroll
-      for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[f], xf[f], acc[b]);
+        for (int u = 0; u < V; ++u)
+#pragma unroll
+          for (int f = 0; f < NF; ++f)
+            xf[u][f] = *reinterpret_cast<const Frag*>(ap[b] + (c + u0 + u) * 64 + f * 4 * MM::kElems);
+#pragma unroll
+        for (int u = 0; u < V; ++u)
+#pragma unroll
+          for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[u0 + u][f], xf[u][f], acc[b]);
+      }
     }
-  }
+  };
+  int c = c_begin;
+  for (; c + 4 <= c_end; c += 4) chunks_at(std::integral_constant<int, 4>{}, c);
+  for (; c < c_end; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
 
   // acc[b][i]: output feature n0 + 4 j + i, token 16 b + r
   float* mine = red + (static_cast<size_t>(wave) * MB * 64 + lane) * 4;
 #pragma unroll
   for (int b = 0; b < MB; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
   __syncthreads();
+  // The sum over the waves, in order; NORMED: times the row's 1 / rms.
   auto total = [&](int e) {
     float sum = 0.f;
     for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
+    if constexpr (NORMED) {
+      float sq = 0.f;
+      for (int w = 0; w < nwaves; ++w) sq += row_val[w * 16 + ((e % 256) / 4) % 16];
+      sum *= 1.0f / sqrtf(sq / static_cast<float>(head.width) + head.eps);
+    }
     return sum;
   };
+  float* sq_el = row_val + nwaves * 16;  // kEpiResidual with by-products: [256] squares of the new h, by element
   for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
     const int b = e / 256, l = (e % 256) / 4, i = e % 4;
     const int row = 4 * (l / 16) + i;
     const int m = b * 16 + l % 16, n = n0 + row;
-    if (m >= M || n >= N) continue;
+    if (row >= ROWS || m >= M || n >= N) continue;
     if constexpr (EPI == kEpiRope) {
       const int head = n0 / tail.hd, blk = (n0 % tail.hd) / 16;
       const bool is_q = head < tail.nh, is_k = !is_q && head < tail.nh + tail.nkv;
@@ -278,12 +373,38 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
       const float gate = total(e), up = total(e + 128);  // the same token, row + 8
       static_cast<T*>(Cv)[static_cast<size_t>(m) * ldc + (n0 / 2 + row)] =
           from_f32<T>((gate / (1.0f + expf(-gate))) * up);
+    } else if constexpr (EPI == kEpiResidual) {
+      float* hp = static_cast<float*>(Cv) + static_cast<size_t>(m) * ldc + n;
+      const bool first = e == static_cast<int>(threadIdx.x);
+      const float v = (first ? h_first : *hp) + total(e);
+      *hp = v;
+      if (res.next_w) {
+        const float nw = first ? nw_first
+                               : (res.next_w_f32 ? static_cast<const float*>(res.next_w)[n]
+                                                 : to_f32(static_cast<const bf16_t*>(res.next_w)[n]));
+        static_cast<T*>(res.xs)[static_cast<size_t>(m) * res.ldx + n] = from_f32<T>(v * nw);
+        sq_el[e] = v * v;
+      }
     } else if constexpr (EPI == kEpiParts) {
       static_cast<float*>(Cv)[(static_cast<size_t>(blockIdx.y) * M + m) * ldc + n] = total(e);
     } else if constexpr (EPI == kEpiF32) {
       static_cast<float*>(Cv)[static_cast<size_t>(m) * ldc + n] = total(e);
     } else {
       static_cast<T*>(Cv)[static_cast<size_t>(m) * ldc + n] = from_f32<T>(total(e));
+    }
+  }
+  if constexpr (EPI == kEpiResidual) {
+    if (res.next_w) {
+      // A token's squares over this workgroup's features, added up in a fixed order (features past
+      // the end of the matrix left no square behind).
+      __syncthreads();
+      for (int t = threadIdx.x; t < 16; t += blockDim.x) {  // rows that do not exist leave a zero
+        const int m = t;
+        float sq = 0.f;
+        for (int row = 0; row < ROWS && n0 + row < N && m < M; ++row)
+          sq += sq_el[4 * (t % 16 + 16 * (row / 4)) + row % 4];
+        res.ssq_part[static_cast<size_t>(blockIdx.x) * 16 + m] = sq;
+      }
     }
   }
 }
@@ -305,27 +426,34 @@ static int skinny_slices(int N, int K) {
 
 // Waves per workgroup: enough of them over the whole launch to keep every
 // compute unit loading, within what LDS holds for the final sum.
-static int skinny_waves(int N, int K, int MB, int slices) {
-  const int row_blocks = (N + 15) / 16;
+static int skinny_waves(int N, int K, int MB, int slices, int rows = 16) {
+  const int row_blocks = (N + rows - 1) / rows;
   const int chunks = K / 64 / slices;
   int waves = 1;
   while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * slices * waves < 4096 && waves * 2 <= chunks) waves *= 2;
   return waves;
 }
 
-template <typename T, int EPI>
+template <typename T, int EPI, bool NORMED = false, int ROWS = 16>
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
-                          int slices, hipStream_t stream, const RopeTail& tail = RopeTail{}) {
+                          int slices, hipStream_t stream, const RopeTail& tail = RopeTail{},
+                          const NormHead& head = NormHead{}, const ResidualTail& res = ResidualTail{}) {
   const int MB = (M + 15) / 16;
-  const int waves = skinny_waves(N, K, MB, slices);
-  const dim3 grid((N + 15) / 16, slices), block(waves * kWave);
-  const size_t lds = static_cast<size_t>(waves) * MB * 256 * sizeof(float);
-#define LYP_SKINNY(MBV) \
-  gemm_skinny_kernel<T, MBV, EPI><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, tail)
-  if (MB == 1) LYP_SKINNY(1);
-  else if (MB == 2) LYP_SKINNY(2);
-  else if (MB == 3) LYP_SKINNY(3);
-  else LYP_SKINNY(4);
+  const int waves = skinny_waves(N, K, MB, slices, ROWS);
+  const dim3 grid((N + ROWS - 1) / ROWS, slices), block(waves * kWave);
+  const size_t lds = (static_cast<size_t>(waves) * MB * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
+                     sizeof(float);
+#define LYP_SKINNY(MBV)                                                                                      \
+  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, \
+                                                                              tail, head, res)
+  if constexpr (NORMED) {
+    LYP_SKINNY(1);  // at most 16 rows: the callers have checked
+  } else {
+    if (MB == 1) LYP_SKINNY(1);
+    else if (MB == 2) LYP_SKINNY(2);
+    else if (MB == 3) LYP_SKINNY(3);
+    else LYP_SKINNY(4);
+  }
 #undef LYP_SKINNY
 }
 
@@ -460,5 +588,79 @@ extern "C" int lyp_gemm_rope_kv(const void* A, const void* W, void* out, int dty
   else
     LYP_REQUIRE(false, "gemm_rope_kv: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gemm_rope_kv");
+  return 0;
+}
+
+// h[M, N] += A . W^T on the float residual stream, for a step with few rows.
+// With next_w (the weights of the RMS norm that follows) it also
+// stores xs[M, N] = h * next_w in the operands' type and, per workgroup, every
+// row's sum of squares over the workgroup's features: ssq_part[parts][16], with
+// `parts` = lyp_gemm_residual_parts(N) workgroups.  A product normed that way
+// (lyp_gemm_swiglu_normed, lyp_gemm_rope_kv_normed) takes xs and ssq_part in
+// place of the normed activations.  Returns 1 (and does nothing) when the
+// few-rows kernel does not apply.
+extern "C" int lyp_gemm_residual_parts(int N) { return (N + 7) / 8; }
+
+extern "C" int lyp_gemm_residual(const void* A, const void* W, float* h, int dtype, int M, int N, int K, int lda,
+                                 int ldw, int ldh, const void* next_w, int next_w_dtype, void* xs, int ldx,
+                                 float* ssq_part, hipStream_t stream) {
+  LYP_REQUIRE(N > 0 && K > 0 && ldh >= N, "gemm_residual: N=%d K=%d stride %d", N, K, ldh);
+  LYP_REQUIRE(!next_w || (xs && ssq_part && ldx >= N && M <= 16), "gemm_residual: by-products for %d rows", M);
+  if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
+  const ResidualTail res{next_w, next_w_dtype == kF32, xs, ldx, ssq_part};
+  if (dtype == kF32)
+    launch_skinny<float, kEpiResidual, false, 8>(static_cast<const float*>(A), static_cast<const float*>(W), h, M, N, K, lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiResidual, false, 8>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), h, M, N, K, lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res);
+  else
+    LYP_REQUIRE(false, "gemm_residual: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_residual");
+  return 0;
+}
+
+// lyp_gemm_swiglu on activations xs that still lack their rows' 1 / rms (see
+// lyp_gemm_residual): silu(g) * u of (xs / rms) . W^T, `width` being the number
+// of features the sums of squares run over.
+extern "C" int lyp_gemm_swiglu_normed(const void* xs, int ldx, const float* ssq_part, int n_parts, int width,
+                                      float eps, const void* W, void* out, int dtype, int M, int N, int K, int ldw,
+                                      int ldo, hipStream_t stream) {
+  LYP_REQUIRE(N % 16 == 0 && ldo >= N / 2, "gemm_swiglu: %d rows of weights, output stride %d", N, ldo);
+  LYP_REQUIRE(ssq_part && n_parts > 0 && width > 0, "gemm_swiglu: no sums of squares");
+  if (M > 16 || !skinny_ok(M, K, ldx, ldw, xs, W, dtype)) return 1;
+  const NormHead head{ssq_part, n_parts, width, eps};
+  if (dtype == kF32)
+    launch_skinny<float, kEpiSwiglu, true>(static_cast<const float*>(xs), static_cast<const float*>(W), out, M, N, K, ldx, ldw, ldo, 1, stream, RopeTail{}, head);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiSwiglu, true>(static_cast<const bf16_t*>(xs), static_cast<const bf16_t*>(W), out, M, N, K, ldx, ldw, ldo, 1, stream, RopeTail{}, head);
+  else
+    LYP_REQUIRE(false, "gemm_swiglu: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_swiglu_normed");
+  return 0;
+}
+
+// lyp_gemm_rope_kv on such activations.
+extern "C" int lyp_gemm_rope_kv_normed(const void* xs, int ldx, const float* ssq_part, int n_parts, int width,
+                                       float eps, const void* W, void* out, int dtype, int M, int K, int ldw,
+                                       int ldo, const int32_t* positions, const float* cos_sin,
+                                       const int32_t* slots, void* kpool, void* vpool, int nh, int nkv, int hd,
+                                       int rot, int bs, int has_kv, hipStream_t stream) {
+  LYP_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "gemm_rope_kv: %d heads, %d key/value heads of %d", nh,
+              nkv, hd);
+  LYP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "gemm_rope_kv: rotary size %d of head size %d", rot, hd);
+  LYP_REQUIRE(positions && (rot == 0 || cos_sin), "gemm_rope_kv: positions and the rotation table are needed");
+  LYP_REQUIRE(!has_kv || (slots && kpool && vpool && bs > 0 && nkv > 0), "gemm_rope_kv: no pages to store to");
+  LYP_REQUIRE(ssq_part && n_parts > 0 && width > 0, "gemm_rope_kv: no sums of squares");
+  const int N = (has_kv ? nh + 2 * nkv : nh) * hd;
+  LYP_REQUIRE(ldo >= nh * hd, "gemm_rope_kv: output stride %d", ldo);
+  if (M > 16 || rot % 16 != 0 || !skinny_ok(M, K, ldx, ldw, xs, W, dtype)) return 1;
+  const RopeTail tail{positions, cos_sin, slots, kpool, vpool, nh, nkv, hd, rot, bs, has_kv};
+  const NormHead head{ssq_part, n_parts, width, eps};
+  if (dtype == kF32)
+    launch_skinny<float, kEpiRope, true>(static_cast<const float*>(xs), static_cast<const float*>(W), out, M, N, K, ldx, ldw, ldo, 1, stream, tail, head);
+  else if (dtype == kBF16)
+    launch_skinny<bf16_t, kEpiRope, true>(static_cast<const bf16_t*>(xs), static_cast<const bf16_t*>(W), out, M, N, K, ldx, ldw, ldo, 1, stream, tail, head);
+  else
+    LYP_REQUIRE(false, "gemm_rope_kv: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("gemm_rope_kv_normed");
   return 0;
 }

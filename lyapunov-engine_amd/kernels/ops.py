@@ -58,6 +58,15 @@ def core() -> ctypes.CDLL:
         lib.lyp_gemm_rope_kv.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_void_p]
+        lib.lyp_gemm_residual_parts.argtypes = [c_int]
+        lib.lyp_gemm_residual.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p]
+        lib.lyp_gemm_swiglu_normed.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
+                                               c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_gemm_rope_kv_normed.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
+                                                c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                                c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                                c_void_p]
         lib.lyp_cast.argtypes = [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p]
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
@@ -136,11 +145,115 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torc
     return out
 
 
+# ------------------------------------------------- work handed on to a consumer
+# A step with few rows is bound by the number of kernels, so two kinds of work
+# may be passed on as a description for the next kernel to fold in, instead of
+# being run on their own:
+#   PendingLinear  a projection whose output is only ever added to the residual
+#                  stream (``linear(..., pending=True)``): the adding kernel is
+#                  the product itself (``linear_residual``);
+#   PendingNorm    RMS-normed rows of the residual stream (``rmsnorm_pending``):
+#                  the kernel that added to the stream also left the rows times
+#                  the norm's weights and their sums of squares; ``linear_rope_kv``
+#                  and ``linear_swiglu`` multiply those rows and divide by the
+#                  rms at the end.
+# Whoever cannot fold one in calls its ``run()`` and gets the plain tensor.
+PENDING_MAX_ROWS = 8
+
+
+class PendingLinear:
+    def __init__(self, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype):
+        self.x, self.w, self.out_dtype = x, w, out_dtype
+
+    def run(self) -> torch.Tensor:
+        """The product, as ``linear(..., may_split=True)`` gives it."""
+        return linear(self.x, self.w, out_dtype=self.out_dtype, may_split=True)
+
+
+class PendingNorm:
+    """Rows of the residual stream ``h`` (already holding the sum) that are to be
+    RMS-normed.  ``xs`` is h * weight in the activations' type and ``ssq_part``
+    [parts, 16] the rows' sums of squares in parts: what the kernel that
+    added to h left behind for the product that comes next."""
+
+    def __init__(self, h: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype, xs: torch.Tensor,
+                 ssq_part: torch.Tensor):
+        self.h, self.weight, self.eps, self.dtype = h, weight, float(eps), dtype
+        self.xs, self.ssq_part = xs, ssq_part
+        self.shape = h.shape
+
+    def run(self) -> torch.Tensor:
+        out = torch.empty(self.h.shape, dtype=self.dtype, device=self.h.device)
+        return rmsnorm(self.h, self.weight, self.eps, out)
+
+
+def as_delta(delta, dtype: torch.dtype):
+    """What a mixer or feed-forward returned, as one plain tensor [T, H] of
+    ``dtype`` (for a norm that adds it by itself)."""
+    if delta is None:
+        return None
+    if isinstance(delta, PendingLinear):
+        delta = delta.run()
+    return sum_parts(delta, dtype)
+
+
+def _few_rows_product(M: int, w: torch.Tensor, act_dtype: torch.dtype) -> bool:
+    """Whether x [M, K] @ w.T runs in the weight-streaming kernel of this package."""
+    return (M <= 64 and w.dtype == act_dtype and w.shape[1] % 64 == 0 and w.stride(1) == 1
+            and not _library_product(M, w.shape[0], w.shape[1], act_dtype))
+
+
+def linear_residual(h: torch.Tensor, p: PendingLinear, next_weight: torch.Tensor | None = None):
+    """h += p.x @ p.w.T on the float residual stream, in the product's kernel.
+    With ``next_weight`` (the weights of the RMS norm that follows) the kernel
+    also leaves what a PendingNorm carries, and (xs, ssq_part) is returned;
+    without it, True.  False (nothing done) when that kernel does not apply."""
+    x, w = p.x, p.w
+    M, K = x.shape
+    N = w.shape[0]
+    if h.dtype != torch.float32 or tuple(h.shape) != (M, N) or w.shape[1] != K or not _few_rows_product(M, w, x.dtype):
+        return False
+    _dev(h, x, w, next_weight)
+    lib = core()
+    xs = ssq = None
+    if next_weight is not None:
+        if M > PENDING_MAX_ROWS or next_weight.numel() != N:
+            return False
+        xs = torch.empty((M, N), dtype=x.dtype, device=h.device)
+        ssq = torch.empty((lib.lyp_gemm_residual_parts(N), 16), dtype=torch.float32, device=h.device)
+    rc = lib.lyp_gemm_residual(_p(x), _p(w), _p(h), _code(x.dtype), M, N, K, x.stride(0), w.stride(0), h.stride(0),
+                               _p(next_weight), _code(next_weight.dtype) if next_weight is not None else 0, _p(xs), N,
+                               _p(ssq), _stream())
+    if rc < 0:
+        _check(rc, lib)
+    if rc != 0:
+        return False
+    return (xs, ssq) if next_weight is not None else True
+
+
+def rmsnorm_pending(h: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype, delta=None):
+    """Add ``delta`` to h and describe the normed rows instead of computing
+    them.  Returns (PendingNorm, None), or (None, delta) when the rows had
+    better be normed by ``rmsnorm``: ``delta`` is then what still has to be
+    added.  Only a delta that is a product still to be run can be folded: its
+    kernel is the one that prepares the norm."""
+    if (not isinstance(delta, PendingLinear) or h.shape[0] > PENDING_MAX_ROWS or h.dtype != torch.float32
+            or delta.x.dtype != dtype):
+        return None, delta
+    done = linear_residual(h, delta, weight)
+    if done is False:
+        return None, delta
+    return PendingNorm(h, weight, eps, dtype, *done), None
+
+
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, delta: torch.Tensor | None = None,
             rows: torch.Tensor | None = None) -> torch.Tensor:
     """out = rmsnorm(h [+ delta]) * weight.  h is the float residual stream and
     takes the sum, unless ``rows`` picks the rows to norm.  ``delta`` is [T, H]
-    in out's dtype, or float partial sums [S, T, H] (see ``linear``)."""
+    in out's dtype, float partial sums [S, T, H], or a product still to be run
+    (see ``linear``)."""
+    if isinstance(delta, PendingLinear):
+        delta = delta.run()
     _dev(h, weight, out, delta, rows)
     H = h.shape[1]
     n = out.shape[0]
@@ -242,6 +355,24 @@ def linear_rope_kv(x: torch.Tensor, w: torch.Tensor, positions: torch.Tensor, co
     width = (num_heads + 2 * num_kv_heads) * head_dim if has_kv else num_heads * head_dim
     if N != width or w.shape[1] != K:
         raise KernelError(f"linear_rope_kv: weight {tuple(w.shape)} for {width} features of {K}")
+    if isinstance(x, PendingNorm):
+        p = x
+        if _few_rows_product(M, w, p.dtype):
+            _dev(p.xs, p.ssq_part, w, positions, cos_sin, slots, kpool, vpool)
+            rot = _rope_check(M, p.dtype, positions, cos_sin, slots, kpool, vpool, num_kv_heads, head_dim, page_size,
+                              has_kv)
+            out = torch.empty((M, num_heads * head_dim), dtype=p.dtype, device=w.device)
+            lib = core()
+            rc = lib.lyp_gemm_rope_kv_normed(_p(p.xs), p.xs.stride(0), _p(p.ssq_part), p.ssq_part.shape[0],
+                                             p.h.shape[1], p.eps,
+                                             _p(w), _p(out), _code(p.dtype), M, K, w.stride(0), out.stride(0),
+                                             _p(positions), _p(cos_sin), _p(slots), _p(kpool), _p(vpool), num_heads,
+                                             num_kv_heads, head_dim, rot, page_size, int(has_kv), _stream())
+            if rc == 0:
+                return out
+            if rc < 0:
+                _check(rc, lib)
+        x = p.run()
     if w.dtype == x.dtype and M <= 64 and not _library_product(M, N, K, x.dtype):
         _dev(x, w, positions, cos_sin, slots, kpool, vpool)
         rot = _rope_check(M, x.dtype, positions, cos_sin, slots, kpool, vpool, num_kv_heads, head_dim, page_size,
@@ -265,6 +396,20 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, interleave: int) -> torch.Te
     """silu(x @ Wgate.T) * (x @ Wup.T) for the fused matrix w [2 I, K] laid out
     as ``swiglu`` describes.  With few rows and interleave 8 it is one kernel."""
     I = w.shape[0] // 2
+    if isinstance(x, PendingNorm):
+        p, M = x, x.shape[0]
+        if interleave == 8 and p.h.shape[1] == w.shape[1] and _few_rows_product(M, w, p.dtype):
+            _dev(p.xs, p.ssq_part, w)
+            out = torch.empty((M, I), dtype=p.dtype, device=w.device)
+            lib = core()
+            rc = lib.lyp_gemm_swiglu_normed(_p(p.xs), p.xs.stride(0), _p(p.ssq_part), p.ssq_part.shape[0],
+                                            p.h.shape[1], p.eps, _p(w), _p(out), _code(p.dtype), M, w.shape[0],
+                                            w.shape[1], w.stride(0), I, _stream())
+            if rc == 0:
+                return out
+            if rc < 0:
+                _check(rc, lib)
+        x = p.run()
     if w.dtype != x.dtype:
         if w.dtype != torch.float32:
             raise KernelError(f"linear_swiglu: weight {w.dtype} against activations {x.dtype}")
@@ -340,7 +485,7 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = None,
-           may_split: bool = False) -> torch.Tensor:
+           may_split: bool = False, pending: bool = False):
     """x @ w.T for a projection weight [out_features, in_features].  A weight
     kept in 32-bit is multiplied in 32-bit whatever the activations are.
 
@@ -348,8 +493,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     [S, rows, out_features] instead (few rows, few output features: the inner
     dimension is then cut into S slices so that every compute unit has work);
     ``rmsnorm`` takes such a delta and adds the slices up, ``sum_parts`` does it
-    for any other consumer."""
+    for any other consumer.  With ``pending`` (the result will only be added to
+    the residual stream) a product of few rows is not run at all but handed on
+    as a ``PendingLinear``."""
     out_dtype = out_dtype or x.dtype
+    if pending and x.shape[0] <= PENDING_MAX_ROWS and _few_rows_product(x.shape[0], w, x.dtype):
+        return PendingLinear(x, w, out_dtype)
     if w.dtype != x.dtype:
         if w.dtype != torch.float32:
             raise KernelError(f"linear: weight {w.dtype} against activations {x.dtype}")

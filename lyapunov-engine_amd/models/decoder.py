@@ -144,6 +144,8 @@ class DecoderModel(Part):
             h, delta = self.layers[call.layer].forward(ctx, h, delta, cache)
         if ctx.R == 0:
             return None
+        if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
+            delta = delta.run()
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
         return ops.linear(x, self.lm_head, out_dtype=torch.float32)
 

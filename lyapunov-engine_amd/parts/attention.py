@@ -60,7 +60,9 @@ class PagedAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
-    def forward(self, ctx: StepContext, x: torch.Tensor, cache: LayerCache) -> torch.Tensor:
+    takes_pending_norm = True   # x may be an ops.PendingNorm: the q/k/v product norms on its way in
+
+    def forward(self, ctx: StepContext, x, cache: LayerCache):
         if cache.writes != self.own_kv:
             raise RuntimeError("a mixer with its own keys must write the cache, one without must not")
         g = cache.group
@@ -68,7 +70,7 @@ class PagedAttention(Mixer):
         qkv = ops.linear_rope_kv(x, self.qkv_proj, ctx.positions, table, g.slot_mapping, cache.k, cache.v,
                                  num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                                  page_size=g.page_size, has_kv=self.own_kv)
-        out = torch.empty((ctx.T, self.num_heads * self.head_dim), dtype=ctx.dtype, device=x.device)
+        out = torch.empty((ctx.T, self.num_heads * self.head_dim), dtype=ctx.dtype, device=qkv.device)
         common = dict(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                       window=self.window, scale=self.scale)
         if ctx.n_tiles:
@@ -85,4 +87,4 @@ class PagedAttention(Mixer):
             part_ml = ctx.scratch("attn_part_ml", n * 2)
             ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.dec_seqs,
                             ctx.n_dec, part_o, part_ml, max_parts, part, **common)
-        return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True)
+        return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True, pending=True)

@@ -155,6 +155,14 @@ class StepContext:
 
 # ------------------------------------------------------------------ part kinds
 class Norm(Part):
+    # True: ``forward`` also takes ``lazy`` and a delta that is a product still
+    # to be run (kernels.ops.PendingLinear), and with ``lazy`` may return the
+    # rows undone, as a kernels.ops.PendingNorm.  False: the block resolves such
+    # a delta first; the delta is then a tensor [T, H] in the activations' type
+    # or float partial sums [S, T, H] (kernels.ops.as_delta makes one tensor of
+    # either).
+    can_defer = False
+
     def forward(self, ctx: StepContext, h: torch.Tensor, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Add ``delta`` to ``h`` (in place, 32-bit), norm, return activations.
@@ -171,7 +179,13 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    """Mixes information between the tokens of a request."""
+    """Mixes information between the tokens of a request.  What ``forward``
+    returns is only ever added to the residual stream: a tensor [T, H], float
+    partial sums [S, T, H] or a kernels.ops.PendingLinear."""
+
+    # True: ``x`` may arrive as a kernels.ops.PendingNorm (normed rows not yet
+    # computed), which the part's first product folds in.
+    takes_pending_norm = False
 
     def cache_spec(self) -> Optional[KVCacheSpec]:
         return None
@@ -184,6 +198,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_pending_norm = False   # as for Mixer
+
     def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

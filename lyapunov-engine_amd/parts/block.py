@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from ..config.registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 from ..config.specs import LayerSpec
+from ..kernels import ops
 from .base import Block, LayerCache, StepContext
 
 
@@ -28,7 +29,18 @@ class PreNormBlock(Block):
                 n["ffn"] + ".": self.ffn}
 
     def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
-        x = self.norm1.forward(ctx, h, delta)
+        x = normed(self.norm1, self.mixer, ctx, h, delta)
         a = self.mixer.forward(ctx, x, cache)
-        x = self.norm2.forward(ctx, h, a)
+        x = normed(self.norm2, self.ffn, ctx, h, a)
         return h, self.ffn.forward(ctx, x)
+
+
+def normed(norm, consumer, ctx: StepContext, h, delta):
+    """h += delta; the normed rows for ``consumer``.  A norm that can and a
+    consumer that takes it may pass the rows on unevaluated (ops.PendingNorm);
+    a norm that does not know of pending products gets the product itself."""
+    if getattr(norm, "can_defer", False):
+        return norm.forward(ctx, h, delta, lazy=getattr(consumer, "takes_pending_norm", False))
+    if isinstance(delta, ops.PendingLinear):
+        delta = delta.run()
+    return norm.forward(ctx, h, delta)

@@ -35,6 +35,8 @@ class SwiGLU(FeedForward):
             WeightSpec("down_proj", (WeightSource("down_proj.weight", (self.hidden_size, self.intermediate_size)),)),
         ]
 
-    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+    takes_pending_norm = True   # x may be an ops.PendingNorm: the gate/up product norms on its way in
+
+    def forward(self, ctx: StepContext, x):
         act = ops.linear_swiglu(x, self.gate_up_proj, self.interleave)
-        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype, may_split=True)
+        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype, may_split=True, pending=True)

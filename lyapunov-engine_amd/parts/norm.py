@@ -27,7 +27,15 @@ class RMSNorm(Norm):
     def weight_specs(self):
         return [WeightSpec("weight", (WeightSource("weight", (self.size,)),), init="ones")]
 
-    def forward(self, ctx: StepContext, h, delta=None, rows=None):
+    # With ``lazy`` the norm may add the delta and hand the rows on as an
+    # ops.PendingNorm for the consumer's kernel to norm on its way in.
+    can_defer = True
+
+    def forward(self, ctx: StepContext, h, delta=None, rows=None, lazy=False):
+        if lazy and rows is None:
+            pending, delta = ops.rmsnorm_pending(h, self.weight, self.eps, ctx.dtype, delta)
+            if pending is not None:
+                return pending
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=ctx.dtype, device=h.device)
         return ops.rmsnorm(h, self.weight, self.eps, out, delta=delta, rows=rows)

@@ -32,11 +32,20 @@ TINY_B = dict(
                       original_max_position_embeddings=64),
     tie_word_embeddings=False,
 )
+# A third one whose sizes are multiples of 64, as a real model's are: only then do the steps with
+# few rows take the kernels that a large model takes (the weight-streaming products with their
+# fused epilogues and the norm folded into them).
+TINY_C = dict(
+    architectures=["LlamaForCausalLM"], vocab_size=320, hidden_size=128, intermediate_size=192, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=32, max_position_embeddings=512, rms_norm_eps=1e-5,
+    rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True,
+)
 # init_std is chosen large enough that attention is peaked: with the usual 0.02
 # every score is near 0, the softmax is flat, and a wrong key or a wrong
 # position barely moves the logits.
 TINY = {"A": (TINY_A, dict(seed=0, init_std=0.15, norm_init_std=0.0, block_size=4)),
-        "B": (TINY_B, dict(seed=2, init_std=0.1, norm_init_std=0.1, block_size=16))}
+        "B": (TINY_B, dict(seed=2, init_std=0.1, norm_init_std=0.1, block_size=16)),
+        "C": (TINY_C, dict(seed=5, init_std=0.1, norm_init_std=0.1, block_size=16))}
 
 
 @pytest.fixture(scope="session")

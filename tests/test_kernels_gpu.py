@@ -134,6 +134,81 @@ def test_linear_partial_sums(ops, dtype, M, N, K):
         assert ((y.cpu().double() - want).abs() <= (1e-2 if dtype == torch.bfloat16 else rel) * bound + 1e-30).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (8, 100, 192), (5, 515, 1024)])
+def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N, K):
+    """A projection of few rows handed on instead of run (pending=True) and
+    then added to the float residual stream by the product kernel itself."""
+    a, w = rnd(M, K, dtype=dtype, seed=31), rnd(N, K, dtype=dtype, scale=0.05, seed=32)
+    want = a.double() @ w.double().T
+    bound = a.double().abs() @ w.double().abs().T
+    p = ops.linear(a.to(DEV), w.to(DEV), may_split=True, pending=True)
+    assert isinstance(p, ops.PendingLinear)
+    h0 = rnd(M, N, seed=33)
+    h = h0.to(DEV)
+    assert ops.linear_residual(h, p) is True
+    rel = 2e-6 if dtype == torch.float32 else 1e-5
+    assert (((h.cpu() - h0).double() - want).abs() <= rel * bound + 2e-6 * h0.abs() + 1e-6).all()
+    # whoever cannot fold it in runs it: the same product (rounded to bfloat16 unless it comes in slices)
+    loose = 1e-2 if dtype == torch.bfloat16 and p.run().dim() == 2 else rel
+    assert ((ops.as_delta(p, torch.float32).cpu().double() - want).abs() <= loose * bound + 1e-30).all()
+    # with more rows the product is not handed on
+    big = ops.linear(rnd(ops.PENDING_MAX_ROWS + 1, K, dtype=dtype).to(DEV), w.to(DEV), may_split=True, pending=True)
+    assert isinstance(big, torch.Tensor)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,K", [(1, 2048), (8, 192), (5, 1024), (7, 256)])
+def test_norm_folded_into_the_products_around_it(ops, dtype, M, K):
+    """The product that adds to the residual stream prepares the RMS norm that
+    follows (rmsnorm_pending), and the gate/up and the q/k/v products finish
+    it: against the plain sum, the plain norm and the plain products."""
+    eps, J = 1e-5, 192
+    h0 = rnd(M, K, seed=41) * 3
+    nw = (1 + 0.2 * rnd(K, seed=42)).to(dtype)
+    a, wo = rnd(M, J, dtype=dtype, seed=44), rnd(K, J, dtype=dtype, scale=0.2, seed=45)
+    h64 = h0.double() + a.double() @ wo.double().T
+    x64 = P.rms_norm(h64, nw.double(), eps)
+    h = h0.to(DEV)
+    delta = ops.linear(a.to(DEV), wo.to(DEV), may_split=True, pending=True)
+    pending, left = ops.rmsnorm_pending(h, nw.to(DEV), eps, dtype, delta)
+    assert isinstance(pending, ops.PendingNorm) and left is None
+    torch.testing.assert_close(h.cpu().double(), h64, rtol=1e-5, atol=1e-4 if dtype == torch.float32 else 1e-2)
+    torch.testing.assert_close(pending.ssq_part.sum(0)[:M].cpu().double(), h.cpu().double().pow(2).sum(-1), rtol=1e-5, atol=0)
+    torch.testing.assert_close(pending.run().cpu().double(), x64, **tol(dtype, 1e-5, 2e-2))
+    # gate/up with the SiLU gate
+    I = 48
+    g = torch.Generator().manual_seed(43)
+    wg, wu = (torch.randn(I, K, generator=g) * 0.1).to(dtype), (torch.randn(I, K, generator=g) * 0.1).to(dtype)
+    w = torch.stack([wg.view(-1, 8, K), wu.view(-1, 8, K)], dim=1).reshape(2 * I, K).contiguous().to(DEV)
+    want = P.mlp(x64, wg.double(), wu.double(), torch.eye(I, dtype=torch.float64))
+    got = ops.linear_swiglu(pending, w, 8)
+    torch.testing.assert_close(got.cpu().double(), want, **tol(dtype, 2e-5, 3e-2))
+    # q/k/v with rotation and page write
+    nh, nkv, hd, bs, n_pages, max_pos = 3, 1, 32, 8, 5, 90
+    wq = (torch.randn((nh + 2 * nkv) * hd, K, generator=g) * 0.1).to(dtype)
+    positions = torch.randint(0, max_pos, (M,), generator=g).to(torch.int32)
+    cos_all, sin_all = P.rope_cos_sin(torch.arange(max_pos), P.rope_inv_freq(hd, 10000.0))
+    table = torch.cat((cos_all[:, : hd // 2], sin_all[:, : hd // 2]), dim=-1).contiguous().to(DEV)
+    slots = torch.randperm(n_pages * bs, generator=g)[:M].to(torch.int32)
+    kpool = torch.zeros(n_pages, nkv, bs, hd, dtype=dtype, device=DEV)
+    vpool = torch.zeros(n_pages, nkv, hd, bs, dtype=dtype, device=DEV)
+    q = ops.linear_rope_kv(pending, wq.to(DEV), positions.to(DEV), table, slots.to(DEV), kpool, vpool, num_heads=nh,
+                           num_kv_heads=nkv, head_dim=hd, page_size=bs)
+    assert q.shape == (M, nh * hd)
+    qkv = (x64 @ wq.double().T).view(M, nh + 2 * nkv, hd)
+    cos, sin = P.rope_cos_sin(positions, P.rope_inv_freq(hd, 10000.0))
+    rotated = P.apply_rope(qkv[:, : nh + nkv].transpose(0, 1), cos.double(), sin.double()).transpose(0, 1)
+    t = tol(dtype, 2e-5, 3e-2)
+    torch.testing.assert_close(q.cpu().double().view(M, nh, hd), rotated[:, :nh], **t)
+    for i in range(M):
+        page, off = int(slots[i]) // bs, int(slots[i]) % bs
+        torch.testing.assert_close(kpool[page, :, off, :].cpu().double(), rotated[i, nh:], **t)
+        torch.testing.assert_close(vpool[page, :, :, off].cpu().double(), qkv[i, nh + nkv:], **t)
+    # nothing to fold the norm into: it is not handed on
+    assert ops.rmsnorm_pending(h, nw.to(DEV), eps, dtype, None) == (None, None)
+
+
 # ------------------------------------------------------------------------ gemm
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 96, 64), (7, 172, 96), (33, 256, 172), (130, 1000, 200), (200, 513, 96),

@@ -1,7 +1,7 @@
 """The whole model through the engine's step function, cache and kernels,
 against the plain implementation: whole prompts, decoding token by token,
 portions of changing size, and mixed batches with pages used again; in 32-bit
-and in bfloat16, for both tiny configurations."""
+and in bfloat16, for the tiny configurations."""
 import json
 import os
 import subprocess
@@ -16,7 +16,8 @@ from trace_util import Trace, compare, plain_logits, random_tokens, replay
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": {"a": 5, "b": 17, "c": 33, "d": 70}, "B": {"a": 1, "b": 9, "c": 64, "d": 130}}
+LENGTHS = {"A": {"a": 5, "b": 17, "c": 33, "d": 70}, "B": {"a": 1, "b": 9, "c": 64, "d": 130},
+           "C": {"a": 3, "b": 20, "c": 48, "d": 81}}
 
 
 def requests_for(name, extra=None):
@@ -60,7 +61,7 @@ def test_each_request_alone_and_whole(model_folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_most_in_one_step_then_token_by_token(model_folders, name, dtype):
     reqs = requests_for(name, {"e": 100})
     want = plain_for(model_folders, name, dtype, reqs)
@@ -75,7 +76,7 @@ def test_most_in_one_step_then_token_by_token(model_folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_portions_of_changing_size(model_folders, name, dtype):
     reqs = requests_for(name, {"e": 100})
     want = plain_for(model_folders, name, dtype, reqs)
@@ -114,7 +115,7 @@ def mixed_trace(reqs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_mixed_batches_with_pages_used_again(model_folders, name, dtype):
     reqs = requests_for(name, {"e": 100, "f": 90, "g": 12, "h": 50})
     want = plain_for(model_folders, name, dtype, reqs)
