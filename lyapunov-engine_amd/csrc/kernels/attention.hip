@@ -177,6 +177,27 @@ struct Softmax {
 // results below the normal range may be flushed.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in every one of them, with the two
+// row-swap instructions of this chip (no trip through LDS).  v_permlane16_swap exchanges the odd
+// 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap the upper
+// half of the first with the lower half of the second; fed with two copies of a value, the two
+// results hold it and its neighbour's.
+__device__ __forceinline__ float lane_groups_max(float m) {
+  float a = m, b = m;
+  asm volatile(
+      "s_nop 1\n\t"
+      "v_permlane16_swap_b32 %0, %1\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32 %0, %0, %1\n\t"
+      "v_mov_b32 %1, %0\n\t"
+      "s_nop 1\n\t"
+      "v_permlane32_swap_b32 %0, %1\n\t"
+      "s_nop 1\n\t"
+      "v_max_f32 %0, %0, %1"
+      : "+v"(a), "+v"(b));
+  return a;
+}
+
 // Take the scores of one 16-key block (s: rows = keys kb0 + 4 (l / 16) + i,
 // column = l % 16), update the running state, rescale the output accumulator
 // and return the probabilities as the column operand of the P.V product.
@@ -199,8 +220,7 @@ __device__ __forceinline__ Frag<T> softmax_block(f32x4 s, float scale_log2, int 
     }
     mx = fmaxf(mx, sv[i]);
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  mx = lane_groups_max(mx);
   const float m_new = fmaxf(st.m, mx);
   const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
   const float alpha = fast_exp2(st.m - m_safe);  // 0 while nothing has been seen yet
@@ -243,8 +263,7 @@ __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf
       }
       mx = fmaxf(mx, sv[u][i]);
     }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+  mx = lane_groups_max(mx);
   const float m_new = fmaxf(st.m, mx);
   const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
   const float alpha = fast_exp2(st.m - m_safe);
@@ -269,24 +288,6 @@ __device__ __forceinline__ float lane_groups_sum(float v) {
   v += __shfl_xor(v, 16, kWave);
   v += __shfl_xor(v, 32, kWave);
   return v;
-}
-
-// One 16-key block of keys and values.  FULL: the page size is a multiple of 16
-// and every key of the block is inside the request and visible, so the block
-// lies in one page (`page`, the same for the whole wave), nothing is masked and
-// the addresses are a wave-wide base plus a constant per lane.
-template <typename T>
-__device__ __forceinline__ void load_block_full(Frag<T> (&kf)[kSteps], Frag<T> (&vf)[kSteps], const PagedKV& kv,
-                                                int kb0, int page, int lane) {
-  const int off = kb0 % kv.bs;
-  const size_t head = static_cast<size_t>(page) * kv.nkv + kv.kvh;
-  const T* krow = static_cast<const T*>(kv.kpool) + (head * kv.bs + off) * HD + (lane % 16) * HD + (lane / 16) * kSlice;
-#pragma unroll
-  for (int s = 0; s < kSteps; ++s) kf[s] = *reinterpret_cast<const Frag<T>*>(krow + 4 * s);
-  const T* vrow = static_cast<const T*>(kv.vpool) + head * HD * kv.bs + off + (lane % 16) * kv.bs + 4 * (lane / 16);
-#pragma unroll
-  for (int db = 0; db < kSteps; ++db)
-    vf[db] = *reinterpret_cast<const Frag<T>*>(vrow + static_cast<size_t>(db) * 16 * kv.bs);
 }
 
 // --------------------------------------------------------------------- prefill
@@ -600,27 +601,6 @@ struct WideTile {
   static constexpr int kBufs = 2 * kElems * 2 <= 64 * 1024 ? 2 : 1;
   static constexpr int kVecs = kKeys * HD / 8;  // 16-byte pieces of a key tile (and of a value tile)
 };
-
-// The maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in every one of them, with the two
-// row-swap instructions of this chip (no trip through LDS).  v_permlane16_swap exchanges the odd
-// 16-lane rows of its first operand with the even rows of its second, v_permlane32_swap the upper
-// half of the first with the lower half of the second; fed with two copies of a value, the two
-// results hold it and its neighbour's.
-__device__ __forceinline__ float lane_groups_max(float m) {
-  float a = m, b = m;
-  asm volatile(
-      "s_nop 1\n\t"
-      "v_permlane16_swap_b32 %0, %1\n\t"
-      "s_nop 1\n\t"
-      "v_max_f32 %0, %0, %1\n\t"
-      "v_mov_b32 %1, %0\n\t"
-      "s_nop 1\n\t"
-      "v_permlane32_swap_b32 %0, %1\n\t"
-      "s_nop 1\n\t"
-      "v_max_f32 %0, %0, %1"
-      : "+v"(a), "+v"(b));
-  return a;
-}
 
 // The scores of one tile (s[u]: rows = keys kb0 + 16 u + 4 (l / 16) + i, column l % 16): update
 // the running maximum `m_run` (base-2 domain), rescale the accumulators when some column's
@@ -955,6 +935,14 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
   const int part = blockIdx.x;
   const int block_keys = kDecodeWaves * keys_per_wave;
+  // The table entries of this wave's first blocks are asked for together with the request's length
+  // (the index is clamped to the row; an entry past the request's keys is not used): one trip to
+  // memory less before the first keys can be asked for.
+  const int32_t* table = block_tables + static_cast<size_t>(seq) * max_blocks;
+  const int k_begin = part * block_keys + wave * keys_per_wave;
+  int pg_first[kDecodeDepth];
+#pragma unroll
+  for (int u = 0; u < kDecodeDepth; ++u) pg_first[u] = table[min((k_begin + 16 * u) / bs, max_blocks - 1)];
   const int ctx = ctx_len[seq];
   const int pos = ctx - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
@@ -972,47 +960,83 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   for (int db = 0; db < kSteps; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   Softmax st{LYP_NEG_INF, 0.f};
 
-  PagedKV kv{kpool, vpool, block_tables + static_cast<size_t>(seq) * max_blocks, nkv, bs, kvh, max_blocks};
+  PagedKV kv{kpool, vpool, table, nkv, bs, kvh, max_blocks};
   const bool aligned = bs % 16 == 0;
-  const int k_begin = part * block_keys + wave * keys_per_wave;
   const int k_first = max(k_begin, (lo / 16) * 16);
   const int k_end = min(ctx, k_begin + keys_per_wave);
 
   Frag<T> kf[kDecodeDepth][kSteps], vf[kDecodeDepth][kSteps];
   auto is_full = [&](int kb0) { return aligned && kb0 >= lo && kb0 + 16 <= ctx; };
-  auto load = [&](int u, int kb0) {
-    if (is_full(kb0)) {
-      load_block_full<T>(kf[u], vf[u], kv, kb0, kv.table[kb0 / bs], lane);
+  // kDecodeDepth blocks of 16 keys are taken together: their scores first (after which the key
+  // buffers are refilled for the next group), one maximum, one rescaling and one pass of
+  // exponentials for all of them, then the products with the values (and the value buffers are
+  // refilled).  Keys from k_end on are another wave's, or do not exist: masked.
+  constexpr int GK = 16 * kDecodeDepth;
+  int pg[kDecodeDepth];  // the pages of the group whose blocks are being asked for (blocks that lie in one page)
+  auto load_k_of = [&](int u, int kb0) {
+    if (is_full(kb0) && kb0 + 16 <= k_end) {
+      const T* krow = static_cast<const T*>(kv.kpool) +
+                      ((static_cast<size_t>(pg[u]) * nkv + kvh) * bs + kb0 % bs) * HD + (lane % 16) * HD +
+                      (lane / 16) * kSlice;
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) kf[u][s] = *reinterpret_cast<const Frag<T>*>(krow + 4 * s);
     } else {
-      load_k<T>(kf[u], kv, kb0, lo, ctx, lane);
-      load_v<T>(vf[u], kv, kb0, lo, ctx, lane);
+      load_k<T>(kf[u], kv, kb0, lo, k_end, lane);
     }
   };
-  auto compute = [&](int u, int kb0) {
-    f32x4 s{0.f, 0.f, 0.f, 0.f};
+  auto load_v_of = [&](int u, int kb0) {
+    if (is_full(kb0) && kb0 + 16 <= k_end) {
+      const T* vrow = static_cast<const T*>(kv.vpool) +
+                      (static_cast<size_t>(pg[u]) * nkv + kvh) * HD * bs + kb0 % bs + (lane % 16) * bs +
+                      4 * (lane / 16);
 #pragma unroll
-    for (int k = 0; k < kSteps; ++k) s = Mma16<T>::mma(kf[u][k], qf[k], s);
-    Frag<T> pf;
-    if (is_full(kb0)) pf = softmax_block<T, false>(s, scale_log2, kb0, pos, window, ctx, st, o, lane);
-    else pf = softmax_block<T, true>(s, scale_log2, kb0, col_valid ? pos : -1, window, ctx, st, o, lane);
-#pragma unroll
-    for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf, o[db]);
+      for (int db = 0; db < kSteps; ++db)
+        vf[u][db] = *reinterpret_cast<const Frag<T>*>(vrow + static_cast<size_t>(db) * 16 * bs);
+    } else {
+      load_v<T>(vf[u], kv, kb0, lo, k_end, lane);
+    }
   };
-
-  // kDecodeDepth blocks are on their way at any time: a buffer is refilled for
-  // the block kDecodeDepth ahead as soon as its block has been used.
+  auto pages_of = [&](int kb0) {
 #pragma unroll
-  for (int u = 0; u < kDecodeDepth; ++u)
-    if (k_first + 16 * u < k_end) load(u, k_first + 16 * u);
-  for (int kb0 = k_first; kb0 < k_end; kb0 += 16 * kDecodeDepth) {
+    for (int u = 0; u < kDecodeDepth; ++u) pg[u] = table[min((kb0 + 16 * u) / bs, max_blocks - 1)];
+  };
+  if (k_first == k_begin) {
+#pragma unroll
+    for (int u = 0; u < kDecodeDepth; ++u) pg[u] = pg_first[u];
+  } else {
+    pages_of(k_first);
+  }
+#pragma unroll
+  for (int u = 0; u < kDecodeDepth; ++u) {
+    load_k_of(u, k_first + 16 * u);
+    load_v_of(u, k_first + 16 * u);
+  }
+  for (int kb0 = k_first; kb0 < k_end; kb0 += GK) {
+    const bool more = kb0 + GK < k_end;
+    f32x4 s[kDecodeDepth];
 #pragma unroll
     for (int u = 0; u < kDecodeDepth; ++u) {
-      const int cur = kb0 + 16 * u;
-      if (cur < k_end) {
-        compute(u, cur);
-        const int next = cur + 16 * kDecodeDepth;
-        if (next < k_end) load(u, next);
-      }
+      s[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < kSteps; ++k) s[u] = Mma16<T>::mma(kf[u][k], qf[k], s[u]);
+    }
+    if (more) {
+      pages_of(kb0 + GK);  // the values of the next group, asked for below, lie in the same pages
+#pragma unroll
+      for (int u = 0; u < kDecodeDepth; ++u) load_k_of(u, kb0 + GK + 16 * u);
+    }
+    Frag<T> pf[kDecodeDepth];
+    if (aligned && kb0 >= lo && kb0 + GK <= k_end)
+      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, k_end, st, o, lane);
+    else
+      softmax_group<T, true, kDecodeDepth>(s, pf, scale_log2, kb0, col_valid ? pos : -1, window, k_end, st, o, lane);
+#pragma unroll
+    for (int u = 0; u < kDecodeDepth; ++u)
+#pragma unroll
+      for (int db = 0; db < kSteps; ++db) o[db] = Mma16<T>::mma(vf[u][db], pf[u], o[db]);
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < kDecodeDepth; ++u) load_v_of(u, kb0 + GK + 16 * u);
     }
   }
 
