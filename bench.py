@@ -136,6 +136,30 @@ def measure_prefill(engine, cfg, tokens, repeats=5):
     return times[len(times) // 2]
 
 
+def check_logits(layers=2, tokens=96):
+    """The 32-bit engine against the bfloat16 engine on the same shape (fewer
+    layers) and the same random weights before rounding: the largest difference
+    of the last position's logits, relative to the largest logit."""
+    import torch
+
+    from lyapunov_engine_amd.engine.runner import StepEntry
+
+    prompt = random_prompt(tokens, MODEL["vocab_size"], 6)
+    logits = {}
+    for dtype in ("fp32", "bf16"):
+        engine, _ = build_engine(layers, dtype, num_blocks=64, max_num_seqs=4, block_size=16, budget=2048)
+        core = engine.core
+        core.cache.add(0)
+        core.cache.extend(0, tokens)
+        logits[dtype] = core.step([StepEntry(0, prompt, 0, [tokens - 1])]).float().cpu()
+        core.cache.commit(0, tokens)
+        core.cache.free(0)
+        del engine, core
+        torch.cuda.empty_cache()
+    ref = logits["fp32"]
+    return float((logits["bf16"] - ref).abs().max() / ref.abs().max()), int(ref.argmax() == logits["bf16"].argmax())
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -146,6 +170,7 @@ def main():
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
+    ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -175,6 +200,14 @@ def main():
             s, _ = measure_decode(engine, cfg, b, 2304, min(args.steps, 64), min(args.warmup, 8), seed=20 + b)
             points[f"decode_b{b}_ctx2048"] = round(b / s, 1)
 
+    check = None
+    if not args.skip_check:
+        del engine
+        torch.cuda.empty_cache()
+        rel, same = check_logits()
+        check = {"what": "bf16 against fp32 logits, same weights, 2 layers, 96-token prompt, last position",
+                 "max_diff_over_max_logit": round(rel, 5), "same_argmax": bool(same)}
+
     peak = MFMA_PEAK[args.dtype]
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2048 tokens; % of roofline",
@@ -195,6 +228,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        "logits_check": check,
     }
     print(json.dumps(line))
     return 0
