@@ -106,7 +106,17 @@ def require_gpu() -> None:
         raise KernelError(f"the kernels are built for {build.GPU_ARCH}, this device is {name}")
 
 
+# torch's current stream as a raw handle.  torch.cuda.current_stream() builds a
+# Stream object on every call (several microseconds, a tenth of the host's time
+# in an eager step); the two private accessors below, where this torch has
+# them, give the same handle directly.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> c_void_p:
+    if _raw_stream is not None and _current_device is not None:
+        return c_void_p(_raw_stream(_current_device()))
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
