@@ -1,13 +1,16 @@
 // Attention over the paged cache, on the matrix cores, compiled for one head
 // size (LYP_HEAD_DIM, a multiple of 16) and both element types.
 //
-// Two kernels share the fragment loaders and the online softmax:
+// The kernels share the fragment loaders and the online softmax:
 //   * attn_prefill: a workgroup takes a run of new tokens of one request and up
 //     to four query heads of one key/value head; the keys and values they may
-//     see pass through LDS, shared by its waves (a wave: one head, 16 tokens).
+//     see pass through LDS, shared by its waves (a wave: one head, 16 or 32
+//     tokens).  attn_prefill_wide is the same work for bfloat16 on the
+//     16x16x32 instruction, with eight waves and loads two tiles ahead.
 //   * attn_decode:  a wave takes one request's single new token, all query
-//     heads of one key/value head (as the 16 columns of the tile), and 64 keys
-//     of the context; a workgroup merges its waves, attn_combine the workgroups.
+//     heads of one key/value head (as the 16 columns of the tile), and a
+//     multiple of 64 keys of the context; a workgroup merges its waves,
+//     attn_combine the workgroups.
 // Both read keys and values from pages through the request's block table, and
 // both run after the step's new keys and values have been written, so a
 // prompt portion needs no second source of keys.
@@ -198,52 +201,14 @@ __device__ __forceinline__ float lane_groups_max(float m) {
   return a;
 }
 
-// Take the scores of one 16-key block (s: rows = keys kb0 + 4 (l / 16) + i,
-// column = l % 16), update the running state, rescale the output accumulator
-// and return the probabilities as the column operand of the P.V product.
-// `pos` is the column's absolute position; a key is visible when
-// key <= pos and (window == 0 or key > pos - window).  With MASKED false every
-// key of the block is visible to every column and the tests are skipped.
-template <typename T, bool MASKED = true>
-__device__ __forceinline__ Frag<T> softmax_block(f32x4 s, float scale_log2, int kb0, int pos, int window,
-                                                 int hi, Softmax& st, f32x4 (&o)[kSteps], int lane) {
-  float sv[4];
-  float mx = LYP_NEG_INF;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if constexpr (MASKED) {
-      const int key = kb0 + 4 * (lane / 16) + i;
-      const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window);
-      sv[i] = vis ? s[i] * scale_log2 : LYP_NEG_INF;
-    } else {
-      sv[i] = s[i] * scale_log2;
-    }
-    mx = fmaxf(mx, sv[i]);
-  }
-  mx = lane_groups_max(mx);
-  const float m_new = fmaxf(st.m, mx);
-  const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
-  const float alpha = fast_exp2(st.m - m_safe);  // 0 while nothing has been seen yet
-  float psum = 0.f;
-  Frag<T> pf;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float p = fast_exp2(sv[i] - m_safe);
-    psum += p;
-    pf[i] = from_f32<T>(p);
-  }
-  st.lsum = st.lsum * alpha + psum;
-  st.m = m_new;
-#pragma unroll
-  for (int db = 0; db < kSteps; ++db)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) o[db][i] *= alpha;
-  return pf;
-}
-
-// The same for NB consecutive 16-key blocks at once (s[u]: block kb0 + 16 u):
-// one maximum, one rescaling of the accumulator and one pass of exponentials
-// for all of them, which is most of the arithmetic outside the matrix cores.
+// Take the scores of NB consecutive 16-key blocks (s[u]: rows = keys
+// kb0 + 16 u + 4 (l / 16) + i, column = l % 16), update the running state,
+// rescale the output accumulator and return the probabilities as the column
+// operands of the P.V products: one maximum, one rescaling and one pass of
+// exponentials for all of them, which is most of the arithmetic outside the
+// matrix cores.  `pos` is the column's absolute position; a key is visible when
+// key <= pos, key < hi and (window == 0 or key > pos - window).  With MASKED
+// false every key is visible to every column and the tests are skipped.
 template <typename T, bool MASKED, int NB>
 __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf)[NB], float scale_log2, int kb0,
                                               int pos, int window, int hi, Softmax& st, f32x4 (&o)[kSteps],
