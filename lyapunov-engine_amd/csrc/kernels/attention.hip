@@ -643,8 +643,11 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
   const int col = lane % 16, grp = lane / 16;
   const int g = nh / nkv;
   const int head_groups = (g + GH - 1) / GH;
-  const int kvh = blockIdx.y / head_groups;
-  const int hsub = (blockIdx.y % head_groups) * GH;
+  // grid (key/value heads x head groups, units): workgroups go to the chip's eight dies in turn by
+  // their number in the launch, x fastest, so with eight key/value heads a die only ever sees the
+  // keys and values of one of them and its second-level cache keeps them between tiles.
+  const int kvh = blockIdx.x / head_groups;
+  const int hsub = (blockIdx.x % head_groups) * GH;
   const int hw = hsub + wave % GH;
   const int head = kvh * g + (hw < g ? hw : 0);
   const T* kp = static_cast<const T*>(kpool);
@@ -684,10 +687,10 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
   const int n_units = n_tiles * kSubs;
   for (int round = 0; round < (paired ? 2 : 1); ++round) {
     // the host lists tiles in rising order of position
-    int unit = n_units - 1 - static_cast<int>(blockIdx.x);
+    int unit = n_units - 1 - static_cast<int>(blockIdx.y);
     if (round == 1) {
-      if (2 * static_cast<int>(blockIdx.x) >= n_units - 1) break;  // the middle unit has no partner
-      unit = blockIdx.x;
+      if (2 * static_cast<int>(blockIdx.y) >= n_units - 1) break;  // the middle unit has no partner
+      unit = blockIdx.y;
     }
     const int tile = unit / kSubs;
     const int seq = tile_seq[tile];
@@ -1140,7 +1143,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   // that are left over take further tokens.
   const int gh = g >= 4 ? 4 : (g >= 2 ? 2 : 1);
   const int head_groups = (g + gh - 1) / gh;
-  LYP_REQUIRE(nkv * head_groups <= 65535, "attn_prefill: too many heads for one launch");
+  LYP_REQUIRE(nkv * head_groups <= 65535 && n_tiles <= 16383, "attn_prefill: too many heads or tiles for one launch");
   const float scale_log2 = scale * kLog2e;
 #define LYP_PREFILL(T, GH, QB)                                                                              \
   do {                                                                                                      \
@@ -1167,7 +1170,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     constexpr int kQW = (NW / GH) * 16;                                                                       \
     const int units = n_tiles * (64 / kQW);                                                                   \
     const int paired = pair != 0 && static_cast<long long>(units) * nkv * head_groups > compute_units();     \
-    dim3 grid(paired ? (units + 1) / 2 : units, nkv * head_groups);                                           \
+    dim3 grid(nkv * head_groups, paired ? (units + 1) / 2 : units);                                           \
     attn_prefill_wide_kernel<GH, NW><<<grid, NW * kWave, 0, stream>>>(                                        \
         static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,         \
         block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,          \
