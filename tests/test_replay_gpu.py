@@ -126,6 +126,45 @@ def test_mixed_batches_with_pages_used_again(model_folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_of_few_rows_take_the_folded_kernels(model_folders, dtype, monkeypatch):
+    """Configuration C is there so that decode steps run the kernels a large
+    model's decode steps run: the norm folded into the products around it.  Count
+    how often that happens in a token-by-token replay (and compare, as above)."""
+    from lyapunov_engine_amd.kernels import ops
+
+    taken = {"norm": 0, "qkv": 0, "gate_up": 0}
+    pending, rope_kv, swiglu = ops.rmsnorm_pending, ops.linear_rope_kv, ops.linear_swiglu
+
+    def count_pending(*a, **k):
+        out = pending(*a, **k)
+        taken["norm"] += out[0] is not None
+        return out
+
+    def count_rope_kv(x, *a, **k):
+        taken["qkv"] += isinstance(x, ops.PendingNorm)
+        return rope_kv(x, *a, **k)
+
+    def count_swiglu(x, *a, **k):
+        taken["gate_up"] += isinstance(x, ops.PendingNorm)
+        return swiglu(x, *a, **k)
+
+    monkeypatch.setattr(ops, "rmsnorm_pending", count_pending)
+    monkeypatch.setattr(ops, "linear_rope_kv", count_rope_kv)
+    monkeypatch.setattr(ops, "linear_swiglu", count_swiglu)
+    reqs = {"a": random_tokens(40, TINY["C"][0]["vocab_size"], seed=7)}
+    want = plain_for(model_folders, "C", dtype, reqs)
+    t = Trace(reqs)
+    t.step([("a", 30)], want="last")
+    for _ in range(10):
+        t.step([("a", 1)])
+    compare(t, replay(folder(model_folders, "C", dtype), dtype, t), want, dtype, "folded")
+    layers = TINY["C"][0]["num_hidden_layers"]
+    # per decode step: the norm before every feed-forward and before every attention but the first
+    assert taken["norm"] == 10 * (2 * layers - 1), taken
+    assert taken["gate_up"] == 10 * layers and taken["qkv"] == 10 * (layers - 1), taken
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_folders, dtype):
     name = "B"
     reqs = {"long": random_tokens(400, TINY[name][0]["vocab_size"], seed=9)}
