@@ -466,6 +466,53 @@ def test_attention_finds_one_far_key(ops, dtype, kind):
     torch.testing.assert_close(out.cpu().float(), want, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["prefill", "decode"])
+@pytest.mark.parametrize("window", [48, 50, 64, 129])   # the edge at a page's first slot, inside a page, a tile wide
+def test_attention_at_the_edge_of_the_window(ops, dtype, kind, window):
+    """The last key inside the window and the first one outside both match the
+    query strongly, the outer one more so: the output must be the inner key's
+    value.  A mask that is off by one at the edge gives the other value; random
+    data would change the output by a few hundredths only."""
+    nh, nkv, hd, bs, ctx = 4, 2, 64, 16, 400
+    ql = 1 if kind == "decode" else 3
+    seqs = [(ctx, ql)]
+    s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=6)
+    k, pages = s["ks"][0], s["bt"][0].tolist()
+    s["qs"][0][:] = 0.0
+    out_key = {}
+    for i in range(ql):                      # every new token has an edge of its own
+        pos = ctx - ql + i
+        inner, outer = pos - window + 1, pos - window
+        out_key[i] = inner
+        s["qs"][0][:, i, i] = 8.0            # token i looks at dimension i alone
+        k[:, :, i] = 0.0
+        k[:, inner, i] = 6.0                 # score 8 * 6 / 8 = 6 over zeros elsewhere ... times log-odds of 400 keys
+        k[:, outer, i] = 12.0                # the outer one would win if it were visible
+    for p in range(ctx):
+        s["kpool"][pages[p // bs], :, p % bs, :] = k[:, p]
+    s["q"] = torch.cat([q.transpose(0, 1).reshape(q.shape[1], nh * hd) for q in s["qs"]], dim=0)
+    out = torch.empty((ql, nh * hd), dtype=dtype, device=DEV)
+    args = (s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV), s["q_start"].to(DEV),
+            s["ctx_len"].to(DEV))
+    kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=hd, window=window)
+    if kind == "decode":
+        part = ops.attn_decode_plan(1, ctx, nh, nkv, hd)
+        mp = -(-ctx // part)
+        ops.attn_decode(*args, None, 1, torch.empty(nh * mp * hd, device=DEV), torch.empty(nh * mp * 2, device=DEV),
+                        mp, part, **kw)
+    else:
+        ops.attn_prefill(*args, torch.zeros(1, dtype=torch.int32, device=DEV),
+                         torch.zeros(1, dtype=torch.int32, device=DEV), 1, **kw)
+    want = plain_attention(s, seqs, window)
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+    # and the plain reference itself is dominated by the inner key, not the outer one
+    for i in range(ql):
+        v_in = s["vs"][0][:, out_key[i]].double().repeat_interleave(nh // nkv, dim=0).reshape(-1)
+        v_out = s["vs"][0][:, out_key[i] - 1].double().repeat_interleave(nh // nkv, dim=0).reshape(-1)
+        assert (want[i] - v_in).abs().max() < 0.5 * (want[i] - v_out).abs().max()
+
+
 # --------------------------------------------------------------------- sampler
 def test_sampler_greedy_and_draws(ops):
     V = 1003
