@@ -164,6 +164,42 @@ def test_steps_of_few_rows_take_the_folded_kernels(model_folders, dtype, monkeyp
     assert taken["gate_up"] == 10 * layers and taken["qkv"] == 10 * (layers - 1), taken
 
 
+ODD = dict(architectures=["LlamaForCausalLM"], max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=10000.0,
+           rope_scaling=None, tie_word_embeddings=True, num_hidden_layers=2)
+ODD_SIZES = {
+    # a width that is no multiple of 8, as many key/value heads as query heads, head size 48
+    "wide-heads": dict(ODD, vocab_size=1001, hidden_size=100, intermediate_size=300, num_attention_heads=5,
+                       num_key_value_heads=5, head_dim=48),
+    # nine heads in groups of three, the smallest head size, a separate output head
+    "small-heads": dict(ODD, vocab_size=257, hidden_size=72, intermediate_size=136, num_attention_heads=9,
+                        num_key_value_heads=3, head_dim=16, tie_word_embeddings=False),
+    # one key/value head for twenty query heads (more than a 16-column tile holds), head size 80
+    "one-kv-head": dict(ODD, vocab_size=333, hidden_size=192, intermediate_size=320, num_attention_heads=20,
+                        num_key_value_heads=1, head_dim=80),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", sorted(ODD_SIZES))
+def test_sizes_that_are_no_powers_of_two(tmp_path, name, dtype):
+    """Whole models of awkward sizes, a mixed trace with portions and decoded
+    tokens: every kernel takes them or the engine says why not; never a wrong
+    result."""
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = ODD_SIZES[name]
+    write_random_model(dict(cfg), str(tmp_path), 3, dtype, init_std=0.1, norm_init_std=0.1)
+    reqs = {"a": random_tokens(70, cfg["vocab_size"], 1), "b": random_tokens(9, cfg["vocab_size"], 2)}
+    want = plain_logits(str(tmp_path), reqs)
+    t = Trace(reqs)
+    t.step([("a", 37), ("b", 2)])
+    t.step([("a", 2), ("b", 7)], end=["b"])
+    t.step([("a", 20)])
+    for _ in range(11):
+        t.step([("a", 1)])
+    compare(t, replay(str(tmp_path), dtype, t), want, dtype, name)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_folders, dtype):
     name = "B"
