@@ -63,6 +63,18 @@ def test_what_is_not_implemented_is_refused(bad, match):
         LlamaConfig.from_dict(dict(TINY_A, **bad))
 
 
+@pytest.mark.parametrize("head_dim", [24, 272])
+def test_a_head_size_the_kernels_do_not_take_is_refused_when_the_model_is_built(head_dim):
+    """The configuration is a valid Llama configuration; it is the attention
+    kernels that exist for multiples of 16 up to 256 only, and the part says so."""
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.models.llama import llama_spec
+
+    cfg = LlamaConfig.from_dict(dict(TINY_A, head_dim=head_dim))
+    with pytest.raises(ValueError, match="multiples of 16"):
+        build_model(llama_spec(cfg))
+
+
 def test_round_trip_through_json(tmp_path):
     for raw in (TINY_A, TINY_B, LLAMA_1B):
         cfg = LlamaConfig.from_dict(raw)
