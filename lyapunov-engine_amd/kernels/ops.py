@@ -463,6 +463,9 @@ LIBRARY_GEMM_MID_ROWS = 17
 LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
 
 
+_MM_FLOAT_OUT = True   # torch.mm(..., out_dtype=float32) exists and works (found out at the first use)
+
+
 def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     if not LIBRARY_GEMM or dtype != torch.bfloat16:
         return False
@@ -524,7 +527,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
                                          w.stride(0), _stream()), lib)
             return parts
     if out_dtype == torch.float32 and _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
-        # the library writes the operands' type; the float result is a cast of it
+        global _MM_FLOAT_OUT
+        if _MM_FLOAT_OUT:
+            try:   # the library's float accumulators written out as they are
+                return torch.mm(x, w.t(), out_dtype=torch.float32)
+            except (TypeError, RuntimeError):
+                _MM_FLOAT_OUT = False   # this torch cannot: the operands' type, then a cast
         y = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
         return cast(gemm_nt(x, w, y), torch.float32)
     if out_dtype in (x.dtype, torch.float32):

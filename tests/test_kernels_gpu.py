@@ -233,6 +233,20 @@ def test_gemm(ops, dtype, M, N, K):
     assert (err <= 1e-5 * (bound + acc.double().abs())).all()
 
 
+def test_float_logits_of_many_rows_are_not_rounded_to_bfloat16(ops):
+    """With more rows than the weight-streaming kernel takes the product goes to
+    the vendor's library; asked for float results it must hand out the float
+    sums, not bfloat16 values cast up (which would make near-ties of logits
+    depend on the size of the batch)."""
+    M, N, K = 70, 300, 256
+    a, w = rnd(M, K, dtype=torch.bfloat16, seed=51), rnd(N, K, dtype=torch.bfloat16, scale=0.05, seed=52)
+    want = a.double() @ w.double().T
+    bound = a.double().abs() @ w.double().abs().T
+    y = ops.linear(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    assert y.dtype == torch.float32
+    assert ((y.cpu().double() - want).abs() <= 1e-5 * bound + 1e-30).all()
+
+
 def test_gemm_float_is_true_32_bit(ops):
     """A product whose low bits a reduced-precision matrix mode would drop."""
     K = 64
