@@ -1,8 +1,9 @@
 """Each part of a layer alone against its plain formula, and the generality of
 the frame: a toy architecture, defined here and registered from here, with a
 mixer that keeps state of its own, a windowed attention layer with pages of its
-own, a layer that runs twice and a layer that reads another call's cache.  No
-file of the package knows any of it."""
+own, a layer that runs twice and a layer that reads another call's cache; and a
+second one with a feed-forward that routes tokens to experts and a position
+encoding of its own.  No file of the package knows any of it."""
 import json
 import os
 from dataclasses import dataclass
@@ -138,7 +139,8 @@ class ToyConfig:
 
     @classmethod
     def from_dict(cls, d):
-        return cls(tuple(sorted((k, v) for k, v in d.items() if k != "architectures" and k != "torch_dtype")))
+        return cls(tuple(sorted((k, v) for k, v in d.items() if k != "architectures" and k != "torch_dtype")),
+                   tuple(d.get("architectures", cls.architectures)))
 
     def to_dict(self):
         return dict(self.raw, architectures=list(self.architectures))
@@ -287,3 +289,152 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     finally:
         ARCHITECTURES.unregister("ToyMixForCausalLM")
         MIXERS.unregister("toy_linear_recurrence")
+
+
+# ------------------------------------------- a second toy: routing, other positions
+TOY2 = dict(architectures=["ToyRoutedForCausalLM"], vocab_size=90, hidden_size=64, num_heads=2, num_kv_heads=1,
+            head_dim=32, rotary_dim=16, experts=3, expert_size=48, intermediate_size=80, max_position=128, eps=1e-6,
+            slope=0.37)
+
+
+def register_toy2():
+    """A feed-forward that routes every token to one of several experts, and a
+    position encoding that is neither the package's rope nor its "none": both
+    defined here and registered from here."""
+    from lyapunov_engine_amd.config import (FEED_FORWARDS, POSITION_ENCODINGS, LayerSpec, ModelSpec, PartSpec,
+                                            default_schedule, register_architecture)
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.parts import FeedForward, PositionEncoding, WeightSource, WeightSpec
+
+    class RoutedExperts(FeedForward):
+        """Router logits in 32-bit; a token goes to its best expert alone and its
+        output is weighted by that expert's softmax probability."""
+
+        graph_safe = False   # which rows go where is read on the host
+
+        def __init__(self, hidden_size, expert_size, experts):
+            self.hidden_size, self.expert_size, self.experts = hidden_size, expert_size, experts
+            self.router = None
+
+        def weight_specs(self):
+            E, H = self.expert_size, self.hidden_size
+            specs = [WeightSpec("router", (WeightSource("router.weight", (self.experts, H)),))]
+            for e in range(self.experts):
+                specs.append(WeightSpec(f"gate_up_{e}", (WeightSource(f"experts.{e}.gate_proj.weight", (E, H)),
+                                                         WeightSource(f"experts.{e}.up_proj.weight", (E, H)))))
+                specs.append(WeightSpec(f"down_{e}", (WeightSource(f"experts.{e}.down_proj.weight", (H, E)),)))
+            return specs
+
+        def forward(self, ctx, x):
+            logits = ops.linear(x, self.router, out_dtype=torch.float32)
+            prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            out = torch.zeros((x.shape[0], self.hidden_size), dtype=torch.float32, device=x.device)
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    act = ops.linear_swiglu(x[rows].contiguous(), getattr(self, f"gate_up_{e}"), 0)
+                    y = ops.linear(act, getattr(self, f"down_{e}"), out_dtype=torch.float32)
+                    out[rows] = y * prob[rows, None]
+            return out.to(ctx.dtype)
+
+    class LinearAngles(PositionEncoding):
+        """Rotates the first `dim` features of a head by angles pos * slope / (i + 1)."""
+
+        def __init__(self, dim, slope, max_position):
+            self.rotary_dim, self.slope, self.max_position = dim, slope, max_position
+            self.table = None
+
+        def materialize(self, device, dtype):
+            freq = self.slope / torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32)
+            angles = torch.outer(torch.arange(self.max_position, dtype=torch.float32), freq)
+            self.table = torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous().to(device)
+
+    FEED_FORWARDS.register("toy_routed_experts", RoutedExperts, replace=True)
+    POSITION_ENCODINGS.register("toy_linear_angles", LinearAngles, replace=True)
+
+    def to_spec(cfg: ToyConfig) -> ModelSpec:
+        c = dict(cfg.raw)
+        H = c["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": c["eps"]})
+        pos = PartSpec("toy_linear_angles", {"dim": c["rotary_dim"], "slope": c["slope"],
+                                             "max_position": c["max_position"]})
+        attn = PartSpec("paged_attention", dict(hidden_size=H, num_heads=c["num_heads"],
+                                                num_kv_heads=c["num_kv_heads"], head_dim=c["head_dim"], position=pos))
+        routed = PartSpec("toy_routed_experts", {"hidden_size": H, "expert_size": c["expert_size"],
+                                                 "experts": c["experts"]})
+        dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
+        layers = (LayerSpec("prenorm", attn, routed, norm, norm), LayerSpec("prenorm", attn, dense, norm, norm))
+        return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=default_schedule(2),
+                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"])
+
+    register_architecture("ToyRoutedForCausalLM", ToyConfig, to_spec, replace=True)
+
+
+def toy2_plain(folder, tokens):
+    from safetensors.torch import load_file
+
+    c = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    S, nh, nkv, hd, rot = len(tokens), c["num_heads"], c["num_kv_heads"], c["head_dim"], c["rotary_dim"]
+    pos = torch.arange(S)
+    freq = (c["slope"] / torch.arange(1, rot // 2 + 1, dtype=torch.float32)).double()
+    angles = torch.outer(pos.double(), freq)
+    cos, sin = torch.cat((angles.cos(), angles.cos()), -1), torch.cat((angles.sin(), angles.sin()), -1)
+
+    def rotate(t):   # the first `rot` features of every head, the rest as they are
+        return torch.cat((P.apply_rope(t[..., :rot], cos, sin), t[..., rot:]), dim=-1)
+
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for layer in range(2):
+        p = f"model.layers.{layer}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
+        q = rotate((x @ w[p + "self_attn.q_proj.weight"].T).view(S, nh, hd).transpose(0, 1))
+        k = rotate((x @ w[p + "self_attn.k_proj.weight"].T).view(S, nkv, hd).transpose(0, 1))
+        v = (x @ w[p + "self_attn.v_proj.weight"].T).view(S, nkv, hd).transpose(0, 1)
+        o = P.attention(q, k, v, pos, pos)
+        h = h + o.transpose(0, 1).reshape(S, nh * hd) @ w[p + "self_attn.o_proj.weight"].T
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
+        if layer == 0:
+            prob, choice = torch.softmax(x @ w[p + "mlp.router.weight"].T, dim=-1).max(dim=-1)
+            y = torch.zeros_like(h)
+            for t in range(S):
+                e = int(choice[t])
+                m = f"{p}mlp.experts.{e}."
+                y[t] = prob[t] * P.mlp(x[t:t + 1], w[m + "gate_proj.weight"], w[m + "up_proj.weight"],
+                                       w[m + "down_proj.weight"])[0]
+            h = h + y
+        else:
+            h = h + P.mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_routed_feed_forward_and_another_position_encoding(tmp_path, dtype):
+    from lyapunov_engine_amd.config import ARCHITECTURES, FEED_FORWARDS, POSITION_ENCODINGS
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import compare
+
+    register_toy2()
+    try:
+        folder = str(tmp_path / "toy2")
+        # With this seed every token's best expert leads the second by 0.13 or more (logits up to
+        # 4.4) and every expert gets tokens: near a tie the engine and the plain model, which round
+        # differently, would send a token to different experts, which is no fault of either.
+        write_random_model(dict(TOY2), folder, seed=138, dtype=dtype, init_std=0.15, norm_init_std=0.1)
+        reqs = {"x": random_tokens(50, 90, seed=5), "y": random_tokens(19, 90, seed=6)}
+        want = {k: toy2_plain(folder, v) for k, v in reqs.items()}
+        whole = Trace(reqs)
+        for rid in reqs:
+            whole.step([(rid, len(reqs[rid]))], end=[rid])
+        compare(whole, replay(folder, dtype, whole), want, dtype, "routed whole")
+        cut = Trace(reqs)
+        cut.step([("x", 11), ("y", 3)])
+        cut.step([("x", 2), ("y", 16)], end=["y"])
+        for _ in range(12):
+            cut.step([("x", 1)])
+        cut.step([("x", 25)], end=["x"])
+        compare(cut, replay(folder, dtype, cut), want, dtype, "routed cut")
+    finally:
+        ARCHITECTURES.unregister("ToyRoutedForCausalLM")
+        FEED_FORWARDS.unregister("toy_routed_experts")
+        POSITION_ENCODINGS.unregister("toy_linear_angles")
