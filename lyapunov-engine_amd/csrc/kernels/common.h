@@ -40,6 +40,15 @@ __device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
   return static_cast<bf16_t>(x);  // round to nearest even
 }
 
+// One rotation of a pair of features by an angle with cosine c and sine s:
+// (x1 c - x2 s, x2 c + x1 s).  The roundings are written out (one product
+// rounded, then a fused multiply-add) so that every kernel that rotates gives
+// the same bits, whatever the compiler would contract by itself.
+__device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s, float& y1, float& y2) {
+  y1 = __builtin_fmaf(x1, c, -(x2 * s));
+  y2 = __builtin_fmaf(x2, c, x1 * s);
+}
+
 // ----------------------------------------------------------------- reductions
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -165,9 +165,10 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, const int32_t* __restrict__ 
       const int head = it / half, i = it % half;
       const float c = cs[i], s = cs[half + i];
       T* x = row + head * hd;
-      const float x1 = to_f32(x[i]), x2 = to_f32(x[i + half]);
-      x[i] = from_f32<T>(x1 * c - x2 * s);
-      x[i + half] = from_f32<T>(x2 * c + x1 * s);
+      float y1, y2;
+      rotate_pair(to_f32(x[i]), to_f32(x[i + half]), c, s, y1, y2);
+      x[i] = from_f32<T>(y1);
+      x[i + half] = from_f32<T>(y2);
     }
   }
   if (!has_kv) return;
@@ -181,6 +182,107 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, const int32_t* __restrict__ 
     const int kvh = it / hd, d = it % hd;
     kpool[((page * nkv + kvh) * bs + off) * hd + d] = k[it];
     vpool[((page * nkv + kvh) * hd + d) * bs + off] = v[it];
+  }
+}
+
+// The same with 16-byte accesses and 16 tokens per workgroup: a thread rotates
+// a run of VEC pairs, copies VEC values of a key at a time, and stores one
+// dimension of the values of all 16 tokens at once when their slots are 16
+// neighbouring places of one page (the usual case in a prompt: the value pages
+// are [hd][bs], so a single token's values are 2-byte stores 2 bs bytes apart).
+// Needs hd % VEC == 0, (rot / 2) % VEC == 0 and 16-byte aligned rows (the
+// launcher checks).  The arithmetic, element by element, is that of
+// rope_kv_kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_tile_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                                           const float* __restrict__ cos_sin,
+                                                           const int32_t* __restrict__ slots, T* __restrict__ kpool,
+                                                           T* __restrict__ vpool, int n_tokens, int nh, int nkv, int hd,
+                                                           int rot, int bs, int has_kv) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int TOK = 16;
+  typedef T VecT __attribute__((ext_vector_type(VEC)));
+  __shared__ int s_slot[TOK];
+  __shared__ int s_run;  // 1: the slots are TOK neighbouring places of one page, the first at a multiple of VEC
+  const int t0 = blockIdx.x * TOK;
+  const int n = min(TOK, n_tokens - t0);
+  const int width = has_kv ? (nh + 2 * nkv) * hd : nh * hd;
+  T* rows = qkv + static_cast<size_t>(t0) * width;
+
+  // The heads are dealt out over the workgroups of a tile of tokens (blockIdx.y): query head h
+  // goes to workgroup h % Y, key/value head k to workgroup k % Y, which rotates that key head and
+  // stores its keys and values.
+  const int Y = gridDim.y, y = blockIdx.y;
+  const int my_q = (nh - y + Y - 1) / Y, my_kv = has_kv ? (nkv - y + Y - 1) / Y : 0;
+  if (rot > 0) {
+    const int half = rot / 2, runs = half / VEC, per_token = (my_q + my_kv) * runs;
+    for (int it = threadIdx.x; it < n * per_token; it += blockDim.x) {
+      const int j = it / per_token, rest = it % per_token;
+      const int mine = rest / runs, i0 = (rest % runs) * VEC;
+      const int head = mine < my_q ? y + mine * Y : nh + y + (mine - my_q) * Y;
+      const float* cs = cos_sin + static_cast<size_t>(positions[t0 + j]) * rot;
+      T* x = rows + static_cast<size_t>(j) * width + head * hd + i0;
+      VecT a = *reinterpret_cast<const VecT*>(x), b = *reinterpret_cast<const VecT*>(x + half);
+      VecT ra, rb;
+#pragma unroll
+      for (int q = 0; q < VEC / 4; ++q) {
+        const f32x4 c = *reinterpret_cast<const f32x4*>(cs + i0 + 4 * q);
+        const f32x4 sn = *reinterpret_cast<const f32x4*>(cs + half + i0 + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float y1, y2;
+          rotate_pair(to_f32(a[4 * q + e]), to_f32(b[4 * q + e]), c[e], sn[e], y1, y2);
+          ra[4 * q + e] = from_f32<T>(y1);
+          rb[4 * q + e] = from_f32<T>(y2);
+        }
+      }
+      *reinterpret_cast<VecT*>(x) = ra;
+      *reinterpret_cast<VecT*>(x + half) = rb;
+    }
+  }
+  if (!has_kv) return;
+  if (threadIdx.x < TOK) s_slot[threadIdx.x] = threadIdx.x < n ? slots[t0 + threadIdx.x] : -1;
+  __syncthreads();  // the rotated keys are in place, the slots are known
+  if (threadIdx.x == 0) {
+    const int first = s_slot[0];
+    bool run = n == TOK && first >= 0 && first % bs % VEC == 0 && first % bs + TOK <= bs;
+    for (int j = 1; j < TOK && run; ++j) run = s_slot[j] == first + j;
+    s_run = run;
+  }
+  const int kv_runs = my_kv * hd / VEC;
+  for (int it = threadIdx.x; it < n * kv_runs; it += blockDim.x) {
+    const int j = it / kv_runs, rest = it % kv_runs;
+    const int slot = s_slot[j];
+    if (slot < 0) continue;
+    const size_t page = slot / bs, off = slot % bs;
+    const int kvh = y + (rest * VEC / hd) * Y, d = rest * VEC % hd;
+    *reinterpret_cast<VecT*>(kpool + ((page * nkv + kvh) * bs + off) * hd + d) =
+        *reinterpret_cast<const VecT*>(rows + static_cast<size_t>(j) * width + (nh + kvh) * hd + d);
+  }
+  __syncthreads();  // s_run
+  const T* v0 = rows + (nh + nkv) * hd;
+  if (s_run) {
+    const size_t page = s_slot[0] / bs, off = s_slot[0] % bs;
+    for (int it = threadIdx.x; it < my_kv * hd; it += blockDim.x) {
+      const int kvh = y + (it / hd) * Y, d = it % hd;
+      T* dst = vpool + ((page * nkv + kvh) * hd + d) * bs + off;
+#pragma unroll
+      for (int q = 0; q < TOK / VEC; ++q) {
+        VecT x;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] = v0[static_cast<size_t>(q * VEC + e) * width + kvh * hd + d];
+        *reinterpret_cast<VecT*>(dst + q * VEC) = x;
+      }
+    }
+  } else {
+    for (int it = threadIdx.x; it < n * my_kv * hd; it += blockDim.x) {
+      const int j = it / (my_kv * hd), rest = it % (my_kv * hd);
+      const int slot = s_slot[j];
+      if (slot < 0) continue;
+      const size_t page = slot / bs, off = slot % bs;
+      const int kvh = y + (rest / hd) * Y, d = rest % hd;
+      vpool[((page * nkv + kvh) * hd + d) * bs + off] = v0[static_cast<size_t>(j) * width + kvh * hd + d];
+    }
   }
 }
 
@@ -334,7 +436,24 @@ int lyp_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const floa
   LYP_REQUIRE(!has_kv || (slots && kpool && vpool), "rope_kv_write: cache write without a cache");
   if (T == 0) return 0;
   const int threads = 256;
-  if (dtype == kF32)
+  const int vec = dtype == kF32 ? 4 : 8;
+  const int width = (has_kv ? nh + 2 * nkv : nh) * hd;
+  // With 16 or more tokens: the kernel that takes 16 of them per workgroup, if everything is
+  // aligned for 16-byte accesses (bs % vec: the value pages' rows then are, too).
+  const bool aligned = T >= 16 && hd % vec == 0 && (rot / 2) % vec == 0 && width % vec == 0 && bs % vec == 0 &&
+                       reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(kpool) % 16 == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;
+  const dim3 tiles((T + 15) / 16, 8);
+  if (aligned && dtype == kF32) {
+    rope_kv_tile_kernel<float><<<tiles, threads, 0, stream>>>(static_cast<float*>(qkv), positions, cos_sin, slots,
+                                                              static_cast<float*>(kpool), static_cast<float*>(vpool),
+                                                              T, nh, nkv, hd, rot, bs, has_kv);
+  } else if (aligned && dtype == kBF16) {
+    rope_kv_tile_kernel<bf16_t><<<tiles, threads, 0, stream>>>(static_cast<bf16_t*>(qkv), positions, cos_sin, slots,
+                                                               static_cast<bf16_t*>(kpool),
+                                                               static_cast<bf16_t*>(vpool), T, nh, nkv, hd, rot, bs,
+                                                               has_kv);
+  } else if (dtype == kF32)
     rope_kv_kernel<float><<<T, threads, 0, stream>>>(static_cast<float*>(qkv), positions, cos_sin, slots,
                                                      static_cast<float*>(kpool), static_cast<float*>(vpool),
                                                      nh, nkv, hd, rot, bs, has_kv);

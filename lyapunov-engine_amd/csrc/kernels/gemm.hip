@@ -346,8 +346,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
         const float* cs = tail.cos_sin + static_cast<size_t>(tail.positions[m]) * tail.rot;
         const float c = cs[fi], sn = cs[half + fi];
         const float x0 = to_f32(y0), x1 = to_f32(from_f32<T>(total(e + 128)));  // the same token, row + 8
-        y0 = from_f32<T>(x0 * c - x1 * sn);
-        y1 = from_f32<T>(x1 * c + x0 * sn);
+        float r0, r1;
+        rotate_pair(x0, x1, c, sn, r0, r1);
+        y0 = from_f32<T>(r0);
+        y1 = from_f32<T>(r1);
         f0 = fi;
         f1 = fi + half;
       }

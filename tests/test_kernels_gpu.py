@@ -260,15 +260,22 @@ def test_gemm_float_is_true_32_bit(ops):
 
 # ----------------------------------------------------- rotation and page write
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd,bs", [(6, 2, 48, 8), (4, 4, 16, 4), (3, 1, 128, 16)])
-def test_rope_kv_write(ops, dtype, nh, nkv, hd, bs):
-    T, n_pages, max_pos = 11, 7, 64
+@pytest.mark.parametrize("nh,nkv,hd,bs,T", [(6, 2, 48, 8, 11), (4, 4, 16, 4, 11), (3, 1, 128, 16, 11),
+                                            (8, 2, 64, 16, 75), (6, 2, 48, 8, 40)])
+def test_rope_kv_write(ops, dtype, nh, nkv, hd, bs, T):
+    """Few tokens take the kernel with a workgroup per token, 16 or more the one
+    with 16 tokens per workgroup, which stores values of tokens in neighbouring
+    slots of a page together: tokens 16..47 below are such runs (where the page
+    is long enough), the others lie anywhere."""
+    n_pages, max_pos = (64 + 2 * T) // bs + 2, 64
     qkv = rnd(T, (nh + 2 * nkv) * hd, dtype=dtype, seed=12)
-    positions = torch.tensor([0, 1, 2, 3, 40, 41, 42, 63, 5, 6, 7], dtype=torch.int32)
+    positions = torch.tensor(([0, 1, 2, 3, 40, 41, 42, 63, 5, 6, 7] * 7)[:T], dtype=torch.int32)
     inv_freq = P.rope_inv_freq(hd, 10000.0)
     cos_all, sin_all = P.rope_cos_sin(torch.arange(max_pos), inv_freq)
     table = torch.cat((cos_all[:, : hd // 2], sin_all[:, : hd // 2]), dim=-1).contiguous()
-    slots = torch.randperm(n_pages * bs, generator=torch.Generator().manual_seed(13))[:T].to(torch.int32)
+    slots = torch.randperm(n_pages * bs - 64, generator=torch.Generator().manual_seed(13))[:T].to(torch.int32) + 64
+    if T >= 48:
+        slots[16:48] = torch.arange(16, 48, dtype=torch.int32)   # two runs of 16, page by page when bs is 16
     slots[4] = -1  # "do not store"
     kpool = torch.zeros(n_pages, nkv, bs, hd, dtype=dtype, device=DEV)
     vpool = torch.zeros(n_pages, nkv, hd, bs, dtype=dtype, device=DEV)
