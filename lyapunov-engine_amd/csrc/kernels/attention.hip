@@ -620,8 +620,12 @@ struct TileRegs {
   bool lost[PER];  // the table had no page for the piece's block
 };
 
-template <int GH, int NW>
-__global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide_kernel(
+// KS = 2: two sets of NW waves share a unit; set 0 takes the unit's key tiles 0, 2, 4, ..., set 1 the
+// tiles 1, 3, 5, ..., each through LDS buffers of its own, and the two running results are merged
+// at the end.  Half as many tiles in a row for one unit: for launches with few units, whose time
+// is that of the unit with most keys.
+template <int GH, int NW, int KS>
+__global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride, const void* kpool,
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
@@ -631,15 +635,22 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
   using WT = WideTile;
   using MMA = Mma16Wide<bf16_t>;
   constexpr int KT = WT::kKeys, NB = KT / 16, NWIDE = KT / 32, DSTEPS = HD / 32;
-  constexpr int THREADS = NW * kWave;
+  constexpr int THREADS = NW * kWave;  // of one set
   constexpr int PER = (WT::kVecs + THREADS - 1) / THREADS;
+  constexpr int KSTEP = KS * KT;       // from one tile of a set to its next
   constexpr int QW = (NW / GH) * 16;  // new tokens per unit
   constexpr int kSubs = 64 / QW;      // units per 64-token tile of the host's list
   static_assert(NW % GH == 0 && QW <= 64 && 64 % QW == 0, "a unit is a whole fraction of a 64-token tile");
-  __shared__ __attribute__((aligned(16))) T lds[WT::kBufs * WT::kElems];
+  constexpr int kMergeFloats = 4 * kSteps + 2;  // what a lane of set 1 hands to its partner in set 0
+  static_assert(KS == 1 || (KS == 2 && NW * kMergeFloats * kWave * 4 <= KS * WT::kBufs * WT::kElems * 2),
+                "one or two sets; the hand-over goes through the tile buffers");
+  __shared__ __attribute__((aligned(16))) T lds_all[KS * WT::kBufs * WT::kElems];
 
-  const int tid = threadIdx.x, lane = tid % kWave;
+  const int lane = threadIdx.x % kWave;
+  const int set = KS == 1 ? 0 : __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / THREADS);
+  const int tid = threadIdx.x % THREADS;  // within the set
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  T* lds = lds_all + set * (WT::kBufs * WT::kElems);
   const int col = lane % 16, grp = lane / 16;
   const int g = nh / nkv;
   const int head_groups = (g + GH - 1) / GH;
@@ -654,7 +665,7 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
   const T* vp = static_cast<const T*>(vpool);
   const size_t page_stride = static_cast<size_t>(nkv) * bs * HD;  // of both pools, in elements
   const size_t head_base = static_cast<size_t>(kvh) * bs * HD;
-  const int step_blk = KT / bs, step_off = KT % bs;
+  const int step_blk = KSTEP / bs, step_off = KSTEP % bs;
 
   // Where this thread's pieces of a tile lie (the same for every tile).  Piece n is 16 bytes of
   // the keys and 16 bytes of the values of one 16-key block of the tile, so of one page.
@@ -731,7 +742,8 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
     // that holds a key of interest the table may hold anything, so the index is clamped there.
     const int32_t* table = block_tables + static_cast<size_t>(seq) * max_blocks;
     const int blk_last = (hi_wg - 1) / bs;
-    const int kt_first = (lo_wg / KT) * KT;
+    const int kt_base = (lo_wg / KT) * KT;      // the unit's first tile
+    const int kt_first = kt_base + set * KT;    // this set's first tile
     int w_blk[PER], w_off[PER];      // the walk: the block of the tile whose table entry is read next
     int page[PER], page_off[PER];    // for the tile whose data is asked for next
 #pragma unroll
@@ -823,12 +835,13 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
       }
     };
 
-    // One round of the loop: tile kt0 is in LDS buffer `buf`, tile kt0 + KT in `ready`; the
-    // loads of tile kt0 + 2 KT are started into `filling`, whose last content is in LDS already.
+    // One round of the loop, in tiles of this set: tile kt0 is in LDS buffer `buf`, the next in
+    // `ready`; the loads of the one after that are started into `filling`, whose last content is
+    // in LDS already.  A set whose tile lies past the unit's keys still passes the barriers.
     auto step = [&](int kt0, int buf, TileRegs<PER>& filling, const TileRegs<PER>& ready) {
       int page_n[PER], page_off_n[PER];
-      read_table(page_n, page_off_n);      // for the tile at kt0 + 3 KT
-      ask(filling, page, page_off);        // the tile at kt0 + 2 KT
+      read_table(page_n, page_off_n);      // for the third tile after kt0
+      ask(filling, page, page_off);        // the second after kt0
 #pragma unroll
       for (int n = 0; n < PER; ++n) {
         page[n] = page_n[n];
@@ -836,7 +849,7 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
       }
       if (wave_active && kt0 <= pos_last_w) compute(buf, kt0);
       if (WT::kBufs == 1) __syncthreads();  // everyone is done with the only buffer before it is overwritten
-      if (kt0 + KT < hi_wg) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KT);
+      if (kt0 + KSTEP < hi_wg) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KSTEP);
       __syncthreads();
     };
 
@@ -848,13 +861,40 @@ __global__ __launch_bounds__(NW* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide
     read_table(page, page_off);  // for the third
     stash(ra, 0, kt_first);
     __syncthreads();
-    for (int kt0 = kt_first; kt0 < hi_wg; kt0 += 2 * KT) {
-      step(kt0, 0, ra, rb);
-      if (kt0 + KT >= hi_wg) break;
-      step(kt0 + KT, WT::kBufs == 2 ? 1 : 0, rb, ra);
+    // the bounds are those of set 0, so that every wave passes the same barriers
+    for (int kb = kt_base; kb < hi_wg; kb += 2 * KSTEP) {
+      step(kb + set * KT, 0, ra, rb);
+      if (kb + KSTEP >= hi_wg) break;
+      step(kb + KSTEP + set * KT, WT::kBufs == 2 ? 1 : 0, rb, ra);
     }
 
-    if (col_valid) {
+    if constexpr (KS == 2) {
+      // Set 1 hands its maximum, sum and output to the same wave and lane of set 0.
+      float* hand = reinterpret_cast<float*>(lds_all) + wave * (kMergeFloats * kWave) + lane;
+      if (set == 1) {
+        hand[0] = m_run;
+        hand[kWave] = lacc[0];
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) hand[(2 + 4 * db + i) * kWave] = o[db][i];
+      }
+      __syncthreads();
+      if (set == 0) {
+        const float m_other = hand[0];
+        const float m_new = fmaxf(m_run, m_other);
+        const float m_safe = m_new == LYP_NEG_INF ? 0.f : m_new;
+        const float a0 = fast_exp2(m_run - m_safe), a1 = fast_exp2(m_other - m_safe);  // 0 for a set that saw nothing
+        lacc[0] = lacc[0] * a0 + hand[kWave] * a1;
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[db][i] = o[db][i] * a0 + hand[(2 + 4 * db + i) * kWave] * a1;
+      }
+      __syncthreads();  // the buffers are free for the next unit
+    }
+
+    if (col_valid && set == 0) {
       const float inv = lacc[0] > 0.f ? 1.0f / lacc[0] : 0.f;
       T* orow = out + (static_cast<size_t>(tok0) + q0_w + col) * out_stride + static_cast<size_t>(head) * HD + 4 * grp;
 #pragma unroll
@@ -1162,24 +1202,37 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   constexpr int kQB4 = LYP_PREFILL_QB;
 #if LYP_HEAD_DIM % 32 == 0 && !defined(LYP_PREFILL_NARROW)
   if (dtype == kBF16 && q_stride % 8 == 0 && bs % 16 == 0) {
-    // `pair` is the caller's word on whether the tiles differ much in the keys they see (0: no).
+    // Bit 0 of `pair` is the caller's word on whether the tiles differ much in the keys they see
+    // (0: no); bit 1 forbids the two sets of waves per unit (for tests and measurements).
     // Units (workgroups before pairing) beyond one per compute unit share compute units anyway;
     // pairing then evens out the causal mask's triangle of work.
+#define LYP_PREFILL_WIDE_KS(GH, NW, KS)                                                                       \
+  attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
+      static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
+      block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
+      scale_log2, paired)
+    // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
+    // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
   do {                                                                                                        \
     constexpr int kQW = (NW / GH) * 16;                                                                       \
     const int units = n_tiles * (64 / kQW);                                                                   \
-    const int paired = pair != 0 && static_cast<long long>(units) * nkv * head_groups > compute_units();     \
+    const long long wgs = static_cast<long long>(units) * nkv * head_groups;                                  \
+    const int paired = (pair & 1) != 0 && wgs > compute_units();                                              \
     dim3 grid(nkv * head_groups, paired ? (units + 1) / 2 : units);                                           \
-    attn_prefill_wide_kernel<GH, NW><<<grid, NW * kWave, 0, stream>>>(                                        \
-        static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,         \
-        block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,          \
-        scale_log2, paired);                                                                                  \
+    if (HD <= 64 && split_ok && wgs <= static_cast<long long>(kSplitBelow) * compute_units()) {               \
+      if constexpr (HD <= 64) LYP_PREFILL_WIDE_KS(GH, NW, 2);                                                 \
+    } else {                                                                                                  \
+      LYP_PREFILL_WIDE_KS(GH, NW, 1);                                                                         \
+    }                                                                                                         \
   } while (0)
+    constexpr int kSplitBelow = 2;
+    const bool split_ok = (pair & 2) == 0;
     if (gh == 4) LYP_PREFILL_WIDE(4, 8);
     else if (gh == 2) LYP_PREFILL_WIDE(2, 8);
     else LYP_PREFILL_WIDE(1, 4);
 #undef LYP_PREFILL_WIDE
+#undef LYP_PREFILL_WIDE_KS
     LYP_LAUNCH_CHECK("attn_prefill");
     return 0;
   }

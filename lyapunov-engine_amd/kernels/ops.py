@@ -576,13 +576,16 @@ def _attn_check(q, out, kpool, vpool, block_tables, nh, nkv, hd):
 def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
                  block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor, tile_seq: torch.Tensor,
                  tile_q0: torch.Tensor, n_tiles: int, *, num_heads: int, num_kv_heads: int, head_dim: int,
-                 window: int = 0, scale: float | None = None, pair: bool | None = None) -> torch.Tensor:
+                 window: int = 0, scale: float | None = None, pair: bool | None = None,
+                 split: bool = True) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache (which already
     holds their own keys).  q is a view [T, >= nh * hd] whose first nh * hd
     columns are the query heads; a tile is 64 new tokens of one request, and
     the tiles are best listed in rising order of the keys they see.  ``pair``
     says whether the first tiles see far fewer keys than the last (then a
-    workgroup may take one of each); None leaves it to the kernel's launcher."""
+    workgroup may take one of each); None leaves it to the kernel's launcher.
+    ``split=False`` keeps a small launch from sharing a tile's keys between
+    two sets of waves (a different order of additions, for tests)."""
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
@@ -592,7 +595,7 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
     _check(lib.lyp_attn_prefill(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
                                 _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(tile_seq),
                                 _p(tile_q0), n_tiles, num_heads, num_kv_heads, bs, window, scale,
-                                -1 if pair is None else int(bool(pair)), _stream()), lib)
+                                (1 if pair is None else int(bool(pair))) | (0 if split else 2), _stream()), lib)
     return out
 
 

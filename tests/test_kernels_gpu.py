@@ -402,9 +402,11 @@ PREFILL_CASES = [
 ]
 
 
+@pytest.mark.parametrize("split", [True, False], ids=["split", "whole"])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("case", PREFILL_CASES, ids=[str(c[:5]) for c in PREFILL_CASES])
-def test_attention_prefill(ops, dtype, case):
+def test_attention_prefill(ops, dtype, case, split):
+    """``split``: a small launch may give a tile's keys to two sets of waves in turn."""
     nh, nkv, hd, bs, window, seqs = case
     s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=hd + bs)
     tile_seq, tile_q0 = [], []
@@ -415,7 +417,7 @@ def test_attention_prefill(ops, dtype, case):
     ops.attn_prefill(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
                      s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(tile_seq, dtype=torch.int32, device=DEV),
                      torch.tensor(tile_q0, dtype=torch.int32, device=DEV), len(tile_seq), num_heads=nh,
-                     num_kv_heads=nkv, head_dim=hd, window=window)
+                     num_kv_heads=nkv, head_dim=hd, window=window, split=split)
     want = plain_attention(s, seqs, window)
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
 
