@@ -399,6 +399,11 @@ PREFILL_CASES = [
     (16, 8, 32, 16, 300, [(1500, 1500), (900, 500), (65, 65), (64, 64)]),
     (8, 8, 128, 16, 0, [(2100, 2100)]),
     (2, 1, 256, 16, 0, [(100, 100), (40, 3)]),
+    # three, five, six and seven query heads to a key/value head
+    (24, 8, 128, 16, 0, [(300, 300), (77, 5)]),
+    (5, 1, 64, 16, 0, [(200, 130)]),
+    (12, 2, 64, 16, 50, [(333, 333)]),
+    (7, 1, 32, 16, 0, [(150, 150)]),
 ]
 
 
