@@ -25,10 +25,16 @@ MODEL = dict(  # BASELINE.json configs[2]: Llama 3.2 1B shape
     rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
     rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
                       original_max_position_embeddings=8192))
-FULL_LAYERS = MODEL["num_hidden_layers"]
+# The larger shapes of BASELINE.json (configs[3] and [4]), for measurements beside the headline.
+SHAPES = {
+    "1b": MODEL,
+    "3b": dict(MODEL, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, head_dim=128),
+    "8b": dict(MODEL, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, head_dim=128,
+               tie_word_embeddings=False, rope_scaling=dict(MODEL["rope_scaling"], factor=8.0)),
+}
 
 
-def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget):
+def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget, shape=MODEL):
     import torch
 
     from lyapunov_engine_amd.config import EngineConfig, LlamaConfig
@@ -38,7 +44,7 @@ def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget):
     from lyapunov_engine_amd.models.llama import llama_spec
     from lyapunov_engine_amd.weights import DictSource, load_weights, random_tensors
 
-    cfg = LlamaConfig.from_dict(dict(MODEL, num_hidden_layers=layers))
+    cfg = LlamaConfig.from_dict(dict(shape, num_hidden_layers=layers))
     model = build_model(llama_spec(cfg))
     tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
     tensors = dict(random_tensors(model, 4, tdtype, device="cuda:0"))   # seed 4, N(0, 0.02)
@@ -136,7 +142,7 @@ def measure_prefill(engine, cfg, tokens, repeats=5):
     return times[len(times) // 2]
 
 
-def check_logits(layers=2, tokens=96):
+def check_logits(shape=MODEL, layers=2, tokens=96):
     """The 32-bit engine against the bfloat16 engine on the same shape (fewer
     layers) and the same random weights before rounding: the largest difference
     of the last position's logits, relative to the largest logit."""
@@ -144,10 +150,10 @@ def check_logits(layers=2, tokens=96):
 
     from lyapunov_engine_amd.engine.runner import StepEntry
 
-    prompt = random_prompt(tokens, MODEL["vocab_size"], 6)
+    prompt = random_prompt(tokens, shape["vocab_size"], 6)
     logits = {}
     for dtype in ("fp32", "bf16"):
-        engine, _ = build_engine(layers, dtype, num_blocks=64, max_num_seqs=4, block_size=16, budget=2048)
+        engine, _ = build_engine(layers, dtype, num_blocks=64, max_num_seqs=4, block_size=16, budget=2048, shape=shape)
         core = engine.core
         core.cache.add(0)
         core.cache.extend(0, tokens)
@@ -167,7 +173,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192, help="context length the decode steps run at")
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="1b is the headline configuration")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all of them)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
@@ -182,7 +189,10 @@ def main():
     block_size = 16
     max_batch = 64
     num_blocks = max_batch * (args.context // block_size + 1) + 64
-    engine, cfg = build_engine(args.layers, args.dtype, num_blocks, max_batch, block_size, budget=8192)
+    shape = SHAPES[args.shape]
+    full_layers = shape["num_hidden_layers"]
+    engine, cfg = build_engine(args.layers or full_layers, args.dtype, num_blocks, max_batch, block_size, budget=8192,
+                               shape=shape)
 
     prefill_s = measure_prefill(engine, cfg, 2048)
     step_s, mean_ctx = measure_decode(engine, cfg, args.batch, args.context, args.steps, args.warmup, seed=1)
@@ -204,7 +214,7 @@ def main():
     if not args.skip_check:
         del engine
         torch.cuda.empty_cache()
-        rel, same = check_logits()
+        rel, same = check_logits(shape)
         check = {"what": "bf16 against fp32 logits, same weights, 2 layers, 96-token prompt, last position",
                  "max_diff_over_max_logit": round(rel, 5), "same_argmax": bool(same)}
 
@@ -215,11 +225,12 @@ def main():
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (random weights seed 4, random token ids)",
         "config": {
-            "model": "llama-3.2-1b-shape", "num_hidden_layers": cfg.num_hidden_layers, "full_layers": FULL_LAYERS,
+            "model": f"llama-{args.shape}-shape" if args.shape != "1b" else "llama-3.2-1b-shape",
+            "num_hidden_layers": cfg.num_hidden_layers, "full_layers": full_layers,
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": True,
-            "rope_scaling": "llama3 factor 32", "global_batch": args.batch, "seq_len": int(round(mean_ctx)),
+            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": bool(shape["tie_word_embeddings"]),
+            "rope_scaling": f"llama3 factor {shape['rope_scaling']['factor']:g}", "global_batch": args.batch, "seq_len": int(round(mean_ctx)),
             "context_len": args.context, "kv_block_size": block_size, "prefill_tokens": 2048,
             "parallelism": "single-gpu", "graphs": True,
         },

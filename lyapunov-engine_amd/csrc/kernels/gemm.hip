@@ -201,7 +201,11 @@ __device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
   return head * t.hd + f;
 }
 
-template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16>
+// PAIRED (8 rows of W, at most 8 tokens): the tile's upper half repeats the 8 rows of W and the
+// tile's upper 8 columns the tokens, both 64 values of K further on, so that one matrix instruction
+// does two chunks of K (on the tile's diagonal blocks; the other two are not used) and no load
+// asks for a value twice.
+template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
                                                            int ldw, int ldc, RopeTail tail, NormHead head,
@@ -210,6 +214,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   using Frag = typename MM::Frag;
   constexpr int NF = 16 / MM::kElems;  // fragments per lane per 64 values of K
   static_assert(ROWS == 16 || ROWS == 8, "a workgroup owns 16 rows of W, or 8 (the tile's lower half repeats them)");
+  static_assert(!PAIRED || (ROWS == 8 && MB == 1 && EPI == kEpiResidual), "two chunks per tile: 8 rows, 8 tokens");
+  constexpr int CHUNK = PAIRED ? 128 : 64;  // values of K per step of a wave
   extern __shared__ float red[];       // [waves][MB][64][4], then MB * 16 floats for the epilogues' row values
 
   const int lane = threadIdx.x % kWave;
@@ -222,7 +228,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   int wrow = min(n0 + r % ROWS, N - 1);  // rows past the end read the last row and are not stored
   if constexpr (EPI == kEpiRope) wrow = rope_feature(tail, n0, r);  // N is a multiple of 16 here
 
-  const int chunks = K / 64;
+  const int chunks = K / CHUNK;
   const int per_slice = (chunks + gridDim.y - 1) / gridDim.y;
   const int s_begin = min(chunks, static_cast<int>(blockIdx.y) * per_slice), s_end = min(chunks, s_begin + per_slice);
   const int per_wave = (s_end - s_begin + nwaves - 1) / nwaves;
@@ -272,10 +278,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 
   // of 64 values of K, fragment f of lane group j holds values 4 E f + E j .. + E - 1 (E = MM::kElems): the
   // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
-  const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems;
+  const int second = PAIRED ? (r / 8) * 64 : 0;  // the tile's upper half: the chunk's second 64 values
+  const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems + second;
   const T* ap[MB];  // rows past the end read the last row and are not stored
 #pragma unroll
-  for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * MM::kElems;
+  for (int b = 0; b < MB; ++b)
+    ap[b] = A + static_cast<size_t>(min(PAIRED ? r % 8 : b * 16 + r, M - 1)) * lda + j * MM::kElems + second;
 
   // U chunks of 64 values of K at once: all of their loads are asked for before the first product
   // needs one.  (The matrix instruction counts as a convergent operation, and the compiler does not
@@ -287,7 +295,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int f = 0; f < NF; ++f)
-        wf[u][f] = *reinterpret_cast<const Frag*>(wp + (c + u) * 64 + f * 4 * MM::kElems);
+        wf[u][f] = *reinterpret_cast<const Frag*>(wp + (c + u) * CHUNK + f * 4 * MM::kElems);
     // the activations come from the cache: four chunks of them at a time are enough
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
         for (int u = 0; u < V; ++u)
 #pragma unroll
           for (int f = 0; f < NF; ++f)
-            xf[u][f] = *reinterpret_cast<const Frag*>(ap[b] + (c + u0 + u) * 64 + f * 4 * MM::kElems);
+            xf[u][f] = *reinterpret_cast<const Frag*>(ap[b] + (c + u0 + u) * CHUNK + f * 4 * MM::kElems);
 #pragma unroll
         for (int u = 0; u < V; ++u)
 #pragma unroll
@@ -320,6 +328,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   auto total = [&](int e) {
     float sum = 0.f;
     for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
+    if constexpr (PAIRED) {  // row + 8, token + 8: the chunks' second halves
+      float upper = 0.f;
+      for (int w = 0; w < nwaves; ++w) upper += red[static_cast<size_t>(w) * 256 + e + 160];
+      sum += upper;
+    }
     if constexpr (NORMED) {
       float sq = 0.f;
       for (int w = 0; w < nwaves; ++w) sq += row_val[w * 16 + ((e % 256) / 4) % 16];
@@ -428,27 +441,27 @@ static int skinny_slices(int N, int K) {
 
 // Waves per workgroup: enough of them over the whole launch to keep every
 // compute unit loading, within what LDS holds for the final sum.
-static int skinny_waves(int N, int K, int MB, int slices, int rows = 16) {
+static int skinny_waves(int N, int K, int MB, int slices, int rows = 16, int chunk = 64) {
   const int row_blocks = (N + rows - 1) / rows;
-  const int chunks = K / 64 / slices;
+  const int chunks = K / chunk / slices;
   int waves = 1;
   while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * slices * waves < 4096 && waves * 2 <= chunks) waves *= 2;
   return waves;
 }
 
-template <typename T, int EPI, bool NORMED = false, int ROWS = 16>
+template <typename T, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false>
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                           int slices, hipStream_t stream, const RopeTail& tail = RopeTail{},
                           const NormHead& head = NormHead{}, const ResidualTail& res = ResidualTail{}) {
   const int MB = (M + 15) / 16;
-  const int waves = skinny_waves(N, K, MB, slices, ROWS);
+  const int waves = skinny_waves(N, K, MB, slices, ROWS, PAIRED ? 128 : 64);
   const dim3 grid((N + ROWS - 1) / ROWS, slices), block(waves * kWave);
   const size_t lds = (static_cast<size_t>(waves) * MB * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
                      sizeof(float);
 #define LYP_SKINNY(MBV)                                                                                      \
-  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, \
-                                                                              tail, head, res)
-  if constexpr (NORMED) {
+  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, \
+                                                                                      ldc, tail, head, res)
+  if constexpr (NORMED || PAIRED) {
     LYP_SKINNY(1);  // at most 16 rows: the callers have checked
   } else {
     if (MB == 1) LYP_SKINNY(1);
@@ -610,12 +623,19 @@ extern "C" int lyp_gemm_residual(const void* A, const void* W, float* h, int dty
   LYP_REQUIRE(!next_w || (xs && ssq_part && ldx >= N && M <= 16), "gemm_residual: by-products for %d rows", M);
   if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
   const ResidualTail res{next_w, next_w_dtype == kF32, xs, ldx, ssq_part};
-  if (dtype == kF32)
-    launch_skinny<float, kEpiResidual, false, 8>(static_cast<const float*>(A), static_cast<const float*>(W), h, M, N, K, lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res);
-  else if (dtype == kBF16)
-    launch_skinny<bf16_t, kEpiResidual, false, 8>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), h, M, N, K, lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res);
-  else
+  const bool paired = M <= 8 && K % 128 == 0;  // two chunks of K per matrix instruction
+#define LYP_RESIDUAL(T, PAIRED)                                                                              \
+  launch_skinny<T, kEpiResidual, false, 8, PAIRED>(static_cast<const T*>(A), static_cast<const T*>(W), h, M, N, K, \
+                                                   lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res)
+  if (dtype == kF32) {
+    if (paired) LYP_RESIDUAL(float, true);
+    else LYP_RESIDUAL(float, false);
+  } else if (dtype == kBF16) {
+    if (paired) LYP_RESIDUAL(bf16_t, true);
+    else LYP_RESIDUAL(bf16_t, false);
+  } else
     LYP_REQUIRE(false, "gemm_residual: unknown dtype %d", dtype);
+#undef LYP_RESIDUAL
   LYP_LAUNCH_CHECK("gemm_residual");
   return 0;
 }

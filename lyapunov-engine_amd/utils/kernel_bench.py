@@ -3,6 +3,7 @@
     python -m lyapunov_engine_amd.utils.kernel_bench attn_prefill --tokens 8192
     python -m lyapunov_engine_amd.utils.kernel_bench attn_decode --batch 8 --context 8192
     python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 8 --out-features 16384 --in-features 2048
+    python -m lyapunov_engine_amd.utils.kernel_bench residual --rows 8 --out-features 2048 --in-features 8192
 
 Prints the time per call and what it means in TFLOP/s or TB/s.  Small enough to
 run under ``rocprofv3 --pmc ...`` when a kernel's counters are wanted; the
@@ -102,9 +103,24 @@ def linear(a) -> None:
           f"{flops / t / 1e12:.1f} TFLOP/s  {w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
 
 
+def residual(a) -> None:
+    """The product that adds to the float residual stream and prepares the next norm."""
+    dt, dev = _dtype(a.dtype), a.device
+    x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
+    w = torch.randn(a.out_features, a.in_features, device=dev, dtype=dt) * 0.02
+    h = torch.zeros(a.rows, a.out_features, device=dev)
+    nw = torch.ones(a.out_features, device=dev, dtype=dt)
+    pending = ops.PendingLinear(x, w, dt)
+    if ops.linear_residual(h, pending, nw) is False:
+        raise SystemExit("the few-rows kernel does not take this shape")
+    t = _time(lambda: ops.linear_residual(h, pending, nw), a.repeat)
+    print(f"residual rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}: {t * 1e6:.1f} us  "
+          f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
-    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear"])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--repeat", type=int, default=20)
@@ -122,7 +138,7 @@ def main(argv=None) -> None:
     a = ap.parse_args(argv)
     ops.require_gpu()
     torch.manual_seed(0)
-    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear}[a.kernel](a)
+    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual}[a.kernel](a)
 
 
 if __name__ == "__main__":

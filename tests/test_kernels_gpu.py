@@ -158,12 +158,12 @@ def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,K", [(1, 2048), (8, 192), (5, 1024), (7, 256)])
-def test_norm_folded_into_the_products_around_it(ops, dtype, M, K):
+@pytest.mark.parametrize("M,K,J", [(1, 2048, 192), (8, 192, 192), (5, 1024, 256), (7, 256, 384), (8, 320, 128)])
+def test_norm_folded_into_the_products_around_it(ops, dtype, M, K, J):
     """The product that adds to the residual stream prepares the RMS norm that
     follows (rmsnorm_pending), and the gate/up and the q/k/v products finish
     it: against the plain sum, the plain norm and the plain products."""
-    eps, J = 1e-5, 192
+    eps = 1e-5   # J: the inner dimension of the product that adds to the stream (in pairs of 64 or not)
     h0 = rnd(M, K, seed=41) * 3
     nw = (1 + 0.2 * rnd(K, seed=42)).to(dtype)
     a, wo = rnd(M, J, dtype=dtype, seed=44), rnd(K, J, dtype=dtype, scale=0.2, seed=45)
