@@ -142,6 +142,40 @@ def measure_prefill(engine, cfg, tokens, repeats=5):
     return times[len(times) // 2]
 
 
+def measure_mixed(engine, cfg, requests=64, seed=0):
+    """BASELINE.json configs[3]'s workload: a continuous batch of `requests` requests with prompts
+    of 128 to 4096 random tokens and 128 to 512 output tokens each, prompts taken in portions of at
+    most 512 tokens.  Returns (seconds, prompt tokens, generated tokens, steps)."""
+    import random
+
+    import torch
+
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    ec = engine.config
+    mixed = LLMEngine(engine.core, EngineConfig(dtype=ec.dtype, num_blocks=ec.num_blocks, block_size=ec.block_size,
+                                                max_num_seqs=requests, max_num_batched_tokens=2048, max_chunk=512,
+                                                max_model_len=cfg.max_position_embeddings))
+    rng = random.Random(seed)
+    prompts = [random_prompt(rng.randint(128, 4096), cfg.vocab_size, 100 + i) for i in range(requests)]
+    params = [SamplingParams(temperature=0.0, max_tokens=rng.randint(128, 512), ignore_eos=True) for _ in prompts]
+    for p_, sp in zip(prompts[:4], params[:4]):          # warm-up: libraries, graphs of the small buckets
+        mixed.add_request(p_[:256], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    while mixed.has_unfinished_requests():
+        mixed.step()
+    for p_, sp in zip(prompts, params):
+        mixed.add_request(p_, sp)
+    torch.cuda.synchronize()
+    t0, steps = time.perf_counter(), 0
+    while mixed.has_unfinished_requests():
+        mixed.step()
+        steps += 1
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps
+
+
 def check_logits(shape=MODEL, layers=2, tokens=96):
     """The 32-bit engine against the bfloat16 engine on the same shape (fewer
     layers) and the same random weights before rounding: the largest difference
@@ -176,6 +210,8 @@ def main():
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="1b is the headline configuration")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all of them)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+                    help="mixed: the continuous batch of BASELINE.json configs[3] instead of the headline")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
     args = ap.parse_args()
@@ -193,6 +229,20 @@ def main():
     full_layers = shape["num_hidden_layers"]
     engine, cfg = build_engine(args.layers or full_layers, args.dtype, num_blocks, max_batch, block_size, budget=8192,
                                shape=shape)
+
+    if args.workload == "mixed":
+        secs, n_prompt, n_gen, steps = measure_mixed(engine, cfg)
+        print(json.dumps({
+            "metric": "generated tok/s of a mixed continuous batch", "value": round(n_gen / secs, 1), "unit": "tok/s",
+            "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": round(secs / steps * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+            "data": "synthetic (random weights seed 4, random token ids)",
+            "config": {"model": f"llama-{args.shape}-shape", "num_hidden_layers": cfg.num_hidden_layers,
+                       "full_layers": full_layers, "requests": 64, "prompt_tokens": n_prompt,
+                       "generated_tokens": n_gen, "prompt_portion": 512, "step_token_budget": 2048,
+                       "kv_block_size": block_size, "parallelism": "single-gpu", "graphs": True},
+            "total_tokens_per_s": round((n_prompt + n_gen) / secs, 1)}))
+        return 0
 
     prefill_s = measure_prefill(engine, cfg, 2048)
     step_s, mean_ctx = measure_decode(engine, cfg, args.batch, args.context, args.steps, args.warmup, seed=1)
