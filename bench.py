@@ -244,6 +244,7 @@ def main():
             "total_tokens_per_s": round((n_prompt + n_gen) / secs, 1)}))
         return 0
 
+    lookahead = bool(engine.config.lookahead)
     prefill_s = measure_prefill(engine, cfg, 2048)
     step_s, mean_ctx = measure_decode(engine, cfg, args.batch, args.context, args.steps, args.warmup, seed=1)
     value = args.batch / step_s
@@ -282,7 +283,7 @@ def main():
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "tie_word_embeddings": bool(shape["tie_word_embeddings"]),
             "rope_scaling": f"llama3 factor {shape['rope_scaling']['factor']:g}", "global_batch": args.batch, "seq_len": int(round(mean_ctx)),
             "context_len": args.context, "kv_block_size": block_size, "prefill_tokens": 2048,
-            "parallelism": "single-gpu", "graphs": True,
+            "parallelism": "single-gpu", "graphs": True, "lookahead": lookahead,
         },
         "prefill": {"value": round(2048 / prefill_s, 1), "tokens": 2048, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops(cfg, 2048) / prefill_s / peak, 4)},

@@ -116,6 +116,13 @@ class CacheManager:
         self._rc(self._lib.lyp_cache_export(self._h, seq_ids.ctypes.data, len(seq_ids), group, tables.ctypes.data,
                                             tables.shape[1], slots.ctypes.data if slots is not None else None))
 
+    def reserve(self, seq_ids, new_lens) -> bool:
+        """Pages for positions < new_lens[b] of every request seq_ids[b] (numpy
+        int64 / int32 arrays), all or none: False, and nothing taken, if a
+        group lacks the pages."""
+        return bool(self._rc(self._lib.lyp_cache_reserve(self._h, seq_ids.ctypes.data, new_lens.ctypes.data,
+                                                         len(seq_ids))))
+
     def ref_count(self, group: int, page: int) -> int:
         return self._rc(self._lib.lyp_cache_ref_count(self._h, group, page))
 

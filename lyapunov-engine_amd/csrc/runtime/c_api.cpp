@@ -121,6 +121,23 @@ int lyp_cache_export(void* h, const int64_t* ids, int n, int g, int32_t* tables,
     return 0;
   });
 }
+// Pages for positions < new_lens[b] of every request ids[b], all or none: 1 if they are held now,
+// 0 (and nothing taken) if some group lacks the pages.  For a caller that prepares the step after
+// the one the scheduler planned.
+int lyp_cache_reserve(void* h, const int64_t* ids, const int32_t* new_lens, int n) {
+  return guarded([&] {
+    auto* m = static_cast<CacheManager*>(h);
+    for (int g = 0; g < m->num_groups(); ++g) {
+      long long need = 0;
+      for (int b = 0; b < n; ++b)
+        if (new_lens[b] > m->capacity(ids[b])) need += m->pages_needed(ids[b], g, new_lens[b]);
+      if (need > m->num_free_pages(g)) return 0;
+    }
+    for (int b = 0; b < n; ++b)
+      if (new_lens[b] > m->capacity(ids[b])) m->extend(ids[b], new_lens[b]);
+    return 1;
+  });
+}
 int lyp_cache_ref_count(void* h, int g, int page) {
   return guarded([&] { return static_cast<CacheManager*>(h)->ref_count(g, page); });
 }

@@ -36,6 +36,8 @@ def _bucket(n: int, smallest: int) -> int:
 
 
 class _Captured:
+    TURNS = 3
+
     def __init__(self, runner: ModelRunner, batch: int, ctx_cap: int, pool):
         self.batch, self.ctx_cap = batch, ctx_cap
         cache = runner.cache
@@ -51,15 +53,20 @@ class _Captured:
         for s in self.sizes:
             self.offsets.append(total)
             total += _align4(s)
-        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
+        # Several pinned copies of the table, used in turn: a step may be filled in while the copy
+        # of the one before it to the device has not run yet.
+        self.hosts = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(self.TURNS)]
+        self.turn = 0
         self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
         self.workspace: dict = {}
-        self.h = h = self.host.numpy()
         self._rows = np.arange(B)
-        h[self.offsets[2]:self.offsets[2] + B + 1] = np.arange(B + 1)
-        h[self.offsets[5]:self.offsets[5] + B] = np.arange(B)
+        for host in self.hosts:
+            h = host.numpy()
+            h[self.offsets[2]:self.offsets[2] + B + 1] = np.arange(B + 1)
+            h[self.offsets[5]:self.offsets[5] + B] = np.arange(B)
+        self.h = self.hosts[0].numpy()
         self.fill(runner, np.zeros(0, np.int64), np.zeros(0, np.int32), np.zeros(0, np.int32))
-        self.dev.copy_(self.host)
+        self.dev.copy_(self.hosts[0])
 
         def view(i):
             return self.dev[self.offsets[i]:self.offsets[i] + self.sizes[i]]
@@ -104,9 +111,15 @@ class _Captured:
                 sm[:n] = bt[rows, starts // ps] * ps + starts % ps
             sm[n:] = -1
 
-    def run(self, runner: ModelRunner, ids, starts, tokens) -> torch.Tensor:
+    def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None) -> torch.Tensor:
+        """``tokens_dev``: the token ids as an int32 tensor on the device, for a
+        step whose tokens the host does not know yet (``tokens`` is ignored)."""
+        self.turn = (self.turn + 1) % self.TURNS
+        self.h = self.hosts[self.turn].numpy()
         self.fill(runner, ids, starts, tokens)
-        self.dev.copy_(self.host, non_blocking=True)
+        self.dev.copy_(self.hosts[self.turn], non_blocking=True)
+        if tokens_dev is not None:
+            self.dev[self.offsets[0]:self.offsets[0] + len(ids)].copy_(tokens_dev[:len(ids)])
         self.graph.replay()
         return self.logits[:len(ids)]
 
@@ -130,9 +143,10 @@ class DecodeGraphs:
                                 np.asarray([e.start for e in entries], dtype=np.int32),
                                 np.asarray([e.tokens[0] for e in entries], dtype=np.int32))
 
-    def step_arrays(self, ids, starts, tokens) -> torch.Tensor:
+    def step_arrays(self, ids, starts, tokens, tokens_dev=None) -> torch.Tensor:
         """The same from numpy arrays: request ids (int64), position and id of
-        each request's one new token (int32)."""
+        each request's one new token (int32); or the ids of the tokens as a
+        tensor on the device (``tokens_dev``)."""
         ctx_need = int(starts.max()) + 1
         key = (_bucket(len(ids), 1), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
         cap = self.captured.get(key)
@@ -140,4 +154,4 @@ class DecodeGraphs:
             if self.pool is None:
                 self.pool = torch.cuda.graph_pool_handle()
             cap = self.captured[key] = _Captured(self.runner, key[0], key[1], self.pool)
-        return cap.run(self.runner, ids, starts, tokens)
+        return cap.run(self.runner, ids, starts, tokens, tokens_dev)

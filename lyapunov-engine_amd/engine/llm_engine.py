@@ -14,11 +14,24 @@ One step: the scheduler plans (prompt portions and decoded tokens, pages taken),
 the step function runs the plan as one batch, the sampler picks a token for
 every request whose known tokens are now all in the cache, the scheduler takes
 the tokens and finishes or frees what is done.
+
+Looking ahead: when a step only decodes, through a captured graph, and nothing
+can change the set of requests before the next step (nobody waits, nobody reaches
+its length), the next step is started on the device before this step's tokens
+have reached the host: it reads them from the sampler's device buffer, and its
+pages are taken a step early.  The scheduler is not told; the next call plans as
+ever, and if its plan is the step that is already running, that step's results
+are taken, otherwise (a request ended on an end-of-sequence token, was aborted,
+was added) they are dropped and the plan runs.  A dropped step has only written
+keys and values of its own requests at positions that the plan writes again or
+whose pages were given back; later work on the stream overwrites what it
+reuses before reading it.
 """
 from __future__ import annotations
 
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..config.engine_config import EngineConfig
@@ -52,6 +65,17 @@ class _Request:
         self.outputs: list = []
 
 
+class _Ahead:
+    """A decode step that is running before the scheduler has planned it."""
+    __slots__ = ("ids", "start", "pending")
+
+    def __init__(self, ids, start, pending):
+        self.ids, self.start, self.pending = ids, start, pending
+
+    def is_plan(self, ids, start) -> bool:
+        return len(ids) == len(self.ids) and bool((ids == self.ids).all()) and bool((start == self.start).all())
+
+
 class LLMEngine:
     def __init__(self, model, config: Optional[EngineConfig] = None, **kw):
         """``model`` is an ``EngineCore``, or a model folder (then the core is
@@ -79,6 +103,8 @@ class LLMEngine:
         if config.enable_graphs:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.core.runner, max_batch=config.max_num_seqs)
+        self._ahead: Optional[_Ahead] = None
+        self.steps_taken_ahead = 0    # steps whose results came from a step started ahead
 
     # ---------------------------------------------------------------- requests
     def add_request(self, arg1, arg2=None, arg3=None):
@@ -126,29 +152,39 @@ class LLMEngine:
         part; ``output_tokens`` of an unfinished request is the engine's own
         growing list (copy it to keep a snapshot)."""
         if not self.has_unfinished_requests():
+            self._ahead = None
             return []
         ids, start, count, wants = self.scheduler.schedule_arrays()
+        ahead, self._ahead = self._ahead, None
         n = len(ids)
         if n == 0:
             return []  # everything running was preempted; the next step admits again
         tokens = self.scheduler.plan_tokens()
-        if self.graphs is not None and self.graphs.safe and n <= self.graphs.max_batch and \
-                bool((count == 1).all()) and bool(wants.all()):
-            logits = self.graphs.step_arrays(ids, start, tokens)
-        else:
-            entries, at = [], 0
-            for i in range(n):
-                c = int(count[i])
-                entries.append(StepEntry(int(ids[i]), tokens[at:at + c].tolist(), int(start[i]),
-                                         [c - 1] if wants[i] else []))
-                at += c
-            logits = self.core.step(entries)
         reqs = [self._requests[int(i)] for i in ids]
-        wanting = [r for r, w in zip(reqs, wants) if w]
-        sampled = []
-        if wanting:
-            sampled = self.sampler.sample(logits, [r.params for r in wanting], [r.stream for r in wanting],
-                                          [len(r.outputs) for r in wanting])
+        decoding = self.graphs is not None and self.graphs.safe and n <= self.graphs.max_batch and \
+            bool((count == 1).all()) and bool(wants.all())
+        if ahead is not None and decoding and ahead.is_plan(ids, start):
+            pending = ahead.pending
+            self.steps_taken_ahead += 1
+        else:
+            if decoding:
+                logits = self.graphs.step_arrays(ids, start, tokens)
+            else:
+                entries, at = [], 0
+                for i in range(n):
+                    c = int(count[i])
+                    entries.append(StepEntry(int(ids[i]), tokens[at:at + c].tolist(), int(start[i]),
+                                             [c - 1] if wants[i] else []))
+                    at += c
+                logits = self.core.step(entries)
+            wanting = [r for r, w in zip(reqs, wants) if w]
+            pending = None
+            if wanting:
+                pending = self.sampler.launch(logits, [r.params for r in wanting], [r.stream for r in wanting],
+                                              [len(r.outputs) for r in wanting])
+        if decoding and self.config.lookahead:
+            self._ahead = self._start_ahead(ids, start, reqs, pending)
+        sampled = pending.result() if pending is not None else []
         status = self.scheduler.post_step_status(sampled)
         outputs, k = [], 0
         for i in range(n):
@@ -163,6 +199,23 @@ class LLMEngine:
             if finished:
                 self._drop(int(ids[i]))
         return outputs
+
+    def _start_ahead(self, ids, start, reqs, pending) -> Optional[_Ahead]:
+        """Start the decode step that follows the planned one (same requests, one
+        position on, the tokens that ``pending`` is choosing), if nothing but an
+        end-of-sequence token can keep the next plan from being that step."""
+        if self.scheduler.num_waiting():
+            return None
+        next_start = start + 1
+        if int(next_start.max()) + 1 >= self.max_model_len or \
+                any(len(r.outputs) + 1 >= r.params.max_tokens for r in reqs):
+            return None  # somebody reaches a length in the planned step
+        ids = ids.copy()
+        if not self.core.cache.reserve(ids, next_start + 1):
+            return None  # no pages to take early
+        logits = self.graphs.step_arrays(ids, next_start, np.zeros(len(ids), dtype=np.int32), tokens_dev=pending.tokens)
+        return _Ahead(ids, next_start, self.sampler.launch(logits, [r.params for r in reqs], [r.stream for r in reqs],
+                                                           [len(r.outputs) + 1 for r in reqs]))
 
     def generate(self, prompts: list, params=None) -> list:
         """Run the prompts (lists of token ids) to the end; one RequestOutput

@@ -35,36 +35,60 @@ def uniform(seed: int, stream: int, index: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class PendingSample:
+    """Tokens that the device is still choosing: ``tokens`` is the device
+    tensor they go to (usable by later work on the stream at once), ``result()``
+    waits for the copy to the host and returns them as a list."""
+
+    def __init__(self, tokens: torch.Tensor, host: torch.Tensor, event: torch.cuda.Event):
+        self.tokens, self._host, self._event = tokens, host, event
+
+    def result(self) -> list:
+        self._event.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
+    RING = 4   # sets of buffers in turn: a set is not touched again while its step may still be in flight
+
     def __init__(self, device, seed: int = 0):
         self.device = torch.device(device)
         self.seed = seed
         self._cap = 0
-        self._host = self._dev = self._out = None
+        self._turn = 0
+        self._sets: list = []
 
     def _reserve(self, rows: int) -> None:
         if rows > self._cap:
             self._cap = max(rows, 2 * self._cap, 64)
-            # rows of the parameter block: temperature, top_p, uniform, top_k (as int32 bits)
-            self._host = torch.zeros((4, self._cap), dtype=torch.float32).pin_memory()
+            self._sets = []
+            for _ in range(self.RING):
+                # rows of the parameter block: temperature, top_p, uniform, top_k (as int32 bits)
+                self._sets.append(dict(
+                    host=torch.zeros((4, self._cap), dtype=torch.float32).pin_memory(),
+                    out=torch.zeros(self._cap, dtype=torch.int32, device=self.device),
+                    out_host=torch.zeros(self._cap, dtype=torch.int32).pin_memory(),
+                    event=torch.cuda.Event()))
             self._dev = torch.zeros((4, self._cap), dtype=torch.float32, device=self.device)
-            self._out = torch.zeros(self._cap, dtype=torch.int32, device=self.device)
             self._work = ops.sample_workspace(self._cap, self.device)
             self._greedy_on_device = True   # the device block is all zeros: temperature 0 everywhere
 
-    def sample(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> list:
+    def launch(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> PendingSample:
         """logits [R, vocab] float on the device; one SamplingParams, stream id
-        and output index per row.  Returns R token ids."""
+        and output index per row.  Starts the choice of R token ids and their
+        copy to the host; nothing waits here."""
         R = logits.shape[0]
         if not (len(params) == len(streams) == len(indices) == R):
             raise ValueError("one set of sampling parameters per row of logits")
         self._reserve(R)
+        bufs = self._sets[self._turn]
+        self._turn = (self._turn + 1) % self.RING
         if all(p.temperature < 1e-4 for p in params):
             if not self._greedy_on_device:
                 self._dev.zero_()
                 self._greedy_on_device = True
         else:
-            h = self._host
+            h = bufs["host"]
             hk = h[3].view(torch.int32)
             for r, (p, s, i) in enumerate(zip(params, streams, indices)):
                 h[0, r] = p.temperature
@@ -74,9 +98,16 @@ class Sampler:
             self._dev[:, :R].copy_(h[:, :R], non_blocking=True)
             self._greedy_on_device = False
         d = self._dev
-        out = self._out[:R]
+        out = bufs["out"][:R]
         ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work)
-        return out.tolist()
+        host = bufs["out_host"][:R]
+        host.copy_(out, non_blocking=True)
+        bufs["event"].record()
+        return PendingSample(out, host, bufs["event"])
+
+    def sample(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> list:
+        """The same, waited for: R token ids."""
+        return self.launch(logits, params, streams, indices).result()
 
 
-__all__ = ["Sampler", "SamplingParams", "uniform"]
+__all__ = ["Sampler", "PendingSample", "SamplingParams", "uniform"]

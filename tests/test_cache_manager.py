@@ -44,6 +44,28 @@ def test_growth_by_any_number_of_tokens_and_fifo_reuse():
     m.check()
 
 
+def test_pages_for_several_requests_all_or_none():
+    import numpy as np
+
+    m = CacheManager([GroupConfig(6, 4), GroupConfig(5, 4)], 4)
+    for i in (1, 2, 3):
+        m.add(i)
+        m.extend(i, 4)                  # one page each in both groups: 3 free in the first, 2 in the second
+    ids = np.array([1, 2, 3], dtype=np.int64)
+    assert m.reserve(ids, np.array([4, 3, 1], dtype=np.int32)) and m.num_free_pages(0) == 3   # held already
+    assert not m.reserve(ids, np.array([5, 5, 5], dtype=np.int32))     # the second group has two pages only
+    assert m.num_free_pages(0) == 3 and m.num_free_pages(1) == 2 and m.capacity(1) == 4
+    assert m.reserve(ids, np.array([5, 4, 8], dtype=np.int32))
+    assert m.capacity(1) == 5 and m.capacity(2) == 4 and m.capacity(3) == 8
+    assert m.num_free_pages(0) == 1 and m.num_free_pages(1) == 0
+    assert len(m.table(1)) == 2 and len(m.table(2)) == 1 and len(m.table(3, 1)) == 2
+    m.check()
+    for i in (1, 2, 3):
+        m.free(i)
+    assert m.num_free_pages(0) == 6 and m.num_free_pages(1) == 5
+    m.check()
+
+
 def test_errors():
     m = CacheManager([GroupConfig(4, 4)], 2)
     m.add(7)

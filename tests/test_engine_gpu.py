@@ -81,6 +81,52 @@ def test_portions_preemption_and_graphs_do_not_change_the_tokens(model_folders, 
         check_against_plain(folder, p, done[f"r{i}"].output_tokens, "float32")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_started_ahead_give_the_same_tokens(model_folders, dtype):
+    """Decode steps started before the tokens of the step before them have reached the host
+    (greedy and seeded sampling, end-of-sequence tokens, requests that arrive and end at different
+    times, few pages): the same tokens as without looking ahead, to the last one."""
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    folder = model_folders["B"][dtype]
+    prompts = [random_tokens(n, 515, seed=90 + n) for n in (30, 9, 21, 40, 3)]
+    params = [SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True),
+              SamplingParams(temperature=0.9, top_k=40, max_tokens=25, seed=5, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_tokens=33),
+              SamplingParams(temperature=0.7, top_p=0.9, max_tokens=48, seed=6),
+              SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)]
+    arrive = [0, 0, 3, 10, 30]
+
+    def run(lookahead, eos):
+        engine = LLMEngine(folder, EngineConfig(dtype=dtype, num_blocks=24, block_size=16, max_num_seqs=4,
+                                                max_num_batched_tokens=32, lookahead=lookahead, eos_token_ids=eos))
+        done, steps, added = {}, 0, 0
+        while added < len(prompts) or engine.has_unfinished_requests():
+            while added < len(prompts) and arrive[added] <= steps:
+                engine.add_request(f"r{added}", prompts[added], params[added])
+                added += 1
+            for out in engine.step():
+                if out.finished:
+                    done[out.request_id] = (list(out.output_tokens), out.finish_reason)
+            steps += 1
+            engine.core.cache.check()
+            assert steps < 1000
+        assert engine.core.cache.num_requests() == 0 and engine.core.cache.num_free_pages() == 24
+        return done, engine.steps_taken_ahead
+
+    plain_run, none_ahead = run(False, ())
+    assert none_ahead == 0
+    # tokens that the third and fourth request produce somewhere in the middle end them
+    eos = (plain_run["r2"][0][12], plain_run["r3"][0][20])
+    want, _ = run(False, eos)
+    got, taken_ahead = run(True, eos)
+    assert got == want
+    assert want["r2"][1] == "stop" and len(want["r2"][0]) <= 13
+    assert taken_ahead > 20, "most decode steps were meant to be started ahead"
+
+
 def test_graph_steps_equal_eager_steps(model_folders):
     """The same decode steps through a captured graph, replayed several times
     with other work in between, and eagerly: equal logits every time."""
