@@ -341,11 +341,40 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, siz
 
 static int norm_threads(int H) { return H <= 512 ? 128 : (H >= 4096 ? 512 : 256); }
 
+// A step's table of small integers from pinned host memory (which the device reads through the
+// same address) to its place on the device, in one launch; `n_patch` words from `patch_at` on come
+// from `patch` on the device instead (token ids that only the device knows yet).
+__global__ __launch_bounds__(256) void table_load_kernel(const int32_t* __restrict__ src, int32_t* __restrict__ dst,
+                                                         int n, const int32_t* __restrict__ patch, int patch_at,
+                                                         int n_patch) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int k = i - patch_at;
+  dst[i] = (patch != nullptr && k >= 0 && k < n_patch) ? patch[k] : src[i];
+}
+
 }  // namespace lyp
 
 using namespace lyp;
 
 extern "C" {
+
+// dst[0..n) on the device = src[0..n) in pinned host memory, except dst[patch_at .. patch_at + n_patch)
+// = patch[0..n_patch) (on the device; may be null).
+int lyp_table_load(const int32_t* src, int32_t* dst, int n, const int32_t* patch, int patch_at, int n_patch,
+                   hipStream_t stream) {
+  LYP_REQUIRE(n >= 0 && src && dst, "table_load: %d words", n);
+  LYP_REQUIRE(!patch || (patch_at >= 0 && n_patch >= 0 && patch_at + n_patch <= n), "table_load: patch %d + %d of %d",
+              patch_at, n_patch, n);
+  if (n == 0) return 0;
+  void* mapped = nullptr;  // the device's address of the host memory (the same one, where memory is mapped so)
+  LYP_REQUIRE(hipHostGetDevicePointer(&mapped, const_cast<int32_t*>(src), 0) == hipSuccess && mapped,
+              "table_load: the source is no pinned host memory that the device can read");
+  table_load_kernel<<<(n + 255) / 256, 256, 0, stream>>>(static_cast<const int32_t*>(mapped), dst, n, patch, patch_at,
+                                                         n_patch);
+  LYP_LAUNCH_CHECK("table_load");
+  return 0;
+}
 
 int lyp_embedding(const int32_t* ids, const void* table, int table_dtype, float* out, int T, int H,
                   hipStream_t stream) {

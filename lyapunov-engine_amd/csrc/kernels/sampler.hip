@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restr
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
-    const ArgMax* __restrict__ cand, int32_t* __restrict__ out) {
+    const ArgMax* __restrict__ cand, int32_t* __restrict__ out, int32_t* __restrict__ mirror) {
   __shared__ ArgMax s_arg[kSampleThreads / kWave];
   __shared__ int s_cnt[kSampleThreads / kWave];
   __shared__ float s_f[kSampleThreads / kWave];
@@ -109,7 +109,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   am = block_argmax(am, s_arg);
   const float T = temperature[row];
   if (T < 1e-4f) {
-    if (tid == 0) out[row] = am.i;
+    if (tid == 0) {
+      out[row] = am.i;
+      if (mirror) mirror[row] = am.i;
+    }
     return;
   }
   const float zmax = am.v / T;
@@ -199,7 +202,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
         break;
       }
     }
-    out[row] = token >= 0 ? token : last_kept;
+    const int pick = token >= 0 ? token : last_kept;
+    out[row] = pick;
+    if (mirror) mirror[row] = pick;
   }
 }
 
@@ -214,16 +219,25 @@ extern "C" long long lyp_sample_workspace(int rows) {
 
 // logits [rows, ld] float; temperature, top_k, top_p, uniform: one per row.
 // workspace: lyp_sample_workspace(rows) bytes, or null (then one workgroup per
-// row scans its whole row for the maximum).
+// row scans its whole row for the maximum).  mirror (optional): a second place
+// the tokens are written to, for instance pinned host memory that the host reads
+// once the kernel is done.
 extern "C" int lyp_sample(const float* logits, int ld, int rows, int V, const float* temperature,
                           const int32_t* top_k, const float* top_p, const float* uniform, void* workspace,
-                          int32_t* out, hipStream_t stream) {
+                          int32_t* out, int32_t* mirror, hipStream_t stream) {
   LYP_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
   if (rows == 0) return 0;
   LYP_REQUIRE(rows <= 65535, "sample: %d rows in one launch", rows);
+  if (mirror) {
+    void* mapped = nullptr;
+    LYP_REQUIRE(hipHostGetDevicePointer(&mapped, mirror, 0) == hipSuccess && mapped,
+                "sample: the mirror is no pinned host memory that the device can write");
+    mirror = static_cast<int32_t*>(mapped);
+  }
   ArgMax* cand = static_cast<ArgMax*>(workspace);
   if (cand) argmax_chunks_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(logits, ld, V, cand);
-  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, cand, out);
+  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, cand, out,
+                                                      mirror);
   LYP_LAUNCH_CHECK("sample");
   return 0;
 }

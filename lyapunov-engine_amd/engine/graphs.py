@@ -24,6 +24,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from ..kernels import ops
 from ..parts.base import GroupView, StepContext
 from .runner import ModelRunner, _align4
 
@@ -117,9 +118,9 @@ class _Captured:
         self.turn = (self.turn + 1) % self.TURNS
         self.h = self.hosts[self.turn].numpy()
         self.fill(runner, ids, starts, tokens)
-        self.dev.copy_(self.hosts[self.turn], non_blocking=True)
-        if tokens_dev is not None:
-            self.dev[self.offsets[0]:self.offsets[0] + len(ids)].copy_(tokens_dev[:len(ids)])
+        # one small kernel reads the pinned table (and the device's token ids) into place
+        ops.table_load(self.hosts[self.turn], self.dev, None if tokens_dev is None else tokens_dev[:len(ids)],
+                       self.offsets[0])
         self.graph.replay()
         return self.logits[:len(ids)]
 

@@ -44,6 +44,7 @@ def core() -> ctypes.CDLL:
         lib = _load(build.core_library())
         lib.lyp_last_error.restype = ctypes.c_char_p
         lib.lyp_embedding.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
+        lib.lyp_table_load.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_rmsnorm.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p, c_int, c_void_p,
                                     c_int, c_int, c_float, c_void_p]
         lib.lyp_rmsnorm_act.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p]
@@ -71,7 +72,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
         lib.lyp_sample.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                   c_void_p, c_void_p]
+                                   c_void_p, c_void_p, c_void_p]
         lib.lyp_sample_workspace.argtypes = [c_int]
         lib.lyp_sample_workspace.restype = c_longlong
         _core = lib
@@ -628,11 +629,40 @@ def sample_workspace(rows: int, device) -> torch.Tensor:
     return torch.empty(max(1, core().lyp_sample_workspace(rows)), dtype=torch.uint8, device=device)
 
 
+def _pinned(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
+    if t.is_cuda or not t.is_pinned() or t.dtype != dtype or not t.is_contiguous():
+        raise KernelError(f"{what} must be a contiguous pinned host tensor of {dtype}")
+
+
+def table_load(src: torch.Tensor, dst: torch.Tensor, patch: torch.Tensor | None = None, patch_at: int = 0) -> None:
+    """dst (int32, device) = src (int32, pinned host memory, read by the kernel
+    itself: no copy engine, no second launch); ``patch`` (int32, device)
+    replaces the words from ``patch_at`` on."""
+    _pinned(src, torch.int32, "table_load: the source")
+    _dev(dst, patch)
+    if dst.dtype != torch.int32 or dst.numel() != src.numel() or not dst.is_contiguous():
+        raise KernelError("table_load: the destination must be a contiguous int32 tensor as long as the source")
+    n_patch = 0
+    if patch is not None:
+        n_patch = patch.numel()
+        if patch.dtype != torch.int32 or not patch.is_contiguous() or patch_at < 0 or patch_at + n_patch > dst.numel():
+            raise KernelError("table_load: the patch does not fit")
+    lib = core()
+    _check(lib.lyp_table_load(src.data_ptr(), _p(dst), dst.numel(), _p(patch), patch_at, n_patch, _stream()), lib)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor | None = None) -> torch.Tensor:
+           uniform: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor | None = None,
+           mirror: torch.Tensor | None = None) -> torch.Tensor:
     """One token per row of logits.  With a ``workspace`` (``sample_workspace``)
-    the search for each row's maximum is spread over the chip."""
+    the search for each row's maximum is spread over the chip.  ``mirror``: pinned
+    host memory (int32, a row each) that receives the tokens as well, readable
+    once the work on the stream up to here is done."""
     _dev(logits, temperature, top_k, top_p, uniform, out, workspace)
+    if mirror is not None:
+        _pinned(mirror, torch.int32, "sample: the mirror")
+        if mirror.numel() != out.numel():
+            raise KernelError("sample: one mirrored token per row")
     R, V = logits.shape
     if logits.dtype != torch.float32 or temperature.dtype != torch.float32 or top_k.dtype != torch.int32 or \
             top_p.dtype != torch.float32 or uniform.dtype != torch.float32 or out.dtype != torch.int32:
@@ -643,5 +673,5 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if workspace is not None and workspace.numel() < lib.lyp_sample_workspace(R):
         raise KernelError("sample: workspace too small")
     _check(lib.lyp_sample(_p(logits), V, R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform), _p(workspace),
-                          _p(out), _stream()), lib)
+                          _p(out), mirror.data_ptr() if mirror is not None else None, _stream()), lib)
     return out

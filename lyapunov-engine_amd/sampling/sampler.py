@@ -99,9 +99,9 @@ class Sampler:
             self._greedy_on_device = False
         d = self._dev
         out = bufs["out"][:R]
-        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work)
         host = bufs["out_host"][:R]
-        host.copy_(out, non_blocking=True)
+        # the kernel writes the tokens to the pinned buffer itself: no copy after it
+        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work, mirror=host)
         bufs["event"].record()
         return PendingSample(out, host, bufs["event"])
 

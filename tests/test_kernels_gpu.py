@@ -561,8 +561,10 @@ def test_sampler_greedy_and_draws(ops):
         u = torch.full((6,), u_val)
         out = torch.empty(6, dtype=torch.int32, device=DEV)
         work = ops.sample_workspace(6, DEV) if u_val > 0.4 else None   # both ways of finding the maximum
-        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out, work)
-        got = out.cpu().tolist()
+        mirror = torch.full((6,), -5, dtype=torch.int32).pin_memory() if u_val > 0.1 else None
+        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out, work, mirror=mirror)
+        got = out.cpu().tolist()     # waits for the kernel: the pinned mirror then holds the same tokens
+        assert mirror is None or mirror.tolist() == got
         assert got[0] == P.greedy(logits[0])
         assert got[1] == 7
         for r in range(2, 6):
@@ -571,6 +573,26 @@ def test_sampler_greedy_and_draws(ops):
             cdf = torch.cumsum(probs, 0)
             lo = float(cdf[got[r]] - probs[got[r]])
             assert lo - 1e-5 <= u_val <= float(cdf[got[r]]) + 1e-5, f"row {r}: u={u_val} not in [{lo}, {float(cdf[got[r]])}]"
+
+
+def test_table_from_pinned_memory(ops):
+    """A table of integers read from pinned host memory by the kernel itself, a
+    few words of it replaced by values that only the device holds."""
+    g = torch.Generator().manual_seed(8)
+    src = torch.randint(-5, 10 ** 6, (1000,), generator=g, dtype=torch.int32).pin_memory()
+    dst = torch.full((1000,), -9, dtype=torch.int32, device=DEV)
+    ops.table_load(src, dst)
+    assert torch.equal(dst.cpu(), src)
+    patch = torch.arange(100, 107, dtype=torch.int32, device=DEV)
+    src[:] = src + 1                       # a later step's table in the same buffer
+    ops.table_load(src, dst, patch, 13)
+    want = src.clone()
+    want[13:20] = patch.cpu()
+    assert torch.equal(dst.cpu(), want)
+    with pytest.raises(ops.KernelError, match="pinned"):
+        ops.table_load(torch.zeros(1000, dtype=torch.int32), dst)
+    with pytest.raises(ops.KernelError, match="does not fit"):
+        ops.table_load(src, dst, patch, 995)
 
 
 def test_sampler_top_k_one_is_greedy_and_frequencies(ops):
