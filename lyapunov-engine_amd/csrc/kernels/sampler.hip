@@ -6,9 +6,12 @@
 // top-p drops a token when the probability mass of the tokens before it, in
 // descending order, already exceeds p, and never the first (:54-66), then one
 // draw from the softmax of what is left (:68-69).  The reference sorts; here
-// both cut-offs are found by bisection on the bit pattern of the values, which
-// needs no sort and gives the same set (tokens that tie with the last kept one
-// are all kept).  The draw is the inverse of the cumulative distribution in
+// both cut-offs are found on the bit pattern of the values (through buckets of
+// the distance from the largest value, then by digits within one bucket; by
+// bisection over the row where that does not apply), which needs no sort and
+// gives the same set (tokens that tie with the last kept one are all kept).
+// Values are logits times 1 / T and the exponentials the fast ones, so a
+// probability differs from the reference's in its last bits.  The draw is the inverse of the cumulative distribution in
 // token order at a uniform number the caller supplies, so a request's tokens
 // depend on its own seed and not on what else is in the batch.
 #include "common.h"
@@ -86,6 +89,207 @@ __global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restr
   }
 }
 
+// ---- the cut-offs without 32 passes over the row
+//
+// A token's distance from the row's largest value, in steps of 1/128, is its bucket (the last
+// bucket takes everything from 32 on).  One pass over the row counts the tokens and adds up their
+// mass per bucket; the bucket in which a cut-off falls follows from the running totals; a second
+// pass collects that bucket's keys (a few hundred as a rule) and the cut-off is found among them,
+// exactly, by digits.  Masses are added as integers (2^40 for the largest token), so a sum does not
+// depend on the order in which the threads arrive.  When a bucket holds more keys than the list
+// does, or the cut-off falls into the last bucket, the bisection over the whole row does the work.
+using u64 = unsigned long long;
+constexpr int kBuckets = 4096;
+constexpr float kBucketsPerUnit = 128.f;
+constexpr int kListCap = 8192;
+constexpr int kMaxSegs = 8192;
+constexpr float kFix = 1099511627776.f;  // 2^40
+static_assert(kBuckets == 4 * kSampleThreads, "a thread looks after four buckets");
+
+__device__ __forceinline__ int bucket_of(float zi, float zmax) {
+  const float d = (zmax - zi) * kBucketsPerUnit;  // >= 0: zmax is the row's largest
+  return d < static_cast<float>(kBuckets - 1) ? static_cast<int>(d) : kBuckets - 1;  // -inf and NaN: the last
+}
+__device__ __forceinline__ u64 mass_of(float zi, float zmax) { return static_cast<u64>(__expf(zi - zmax) * kFix); }
+__device__ __forceinline__ float value_of_key(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+__device__ __forceinline__ u64 shfl_up_u64(u64 v, int delta) {
+  const uint32_t lo = __shfl_up(static_cast<uint32_t>(v), delta, kWave);
+  const uint32_t hi = __shfl_up(static_cast<uint32_t>(v >> 32), delta, kWave);
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+__device__ __forceinline__ u64 shfl_u64(u64 v, int src) {
+  const uint32_t lo = __shfl(static_cast<uint32_t>(v), src, kWave);
+  const uint32_t hi = __shfl(static_cast<uint32_t>(v >> 32), src, kWave);
+  return (static_cast<u64>(hi) << 32) | lo;
+}
+// Within a wave: the sum over the lanes before this one, and (every lane) the sum over all.
+__device__ __forceinline__ u64 wave_excl_scan(u64 v, u64& total) {
+  const int lane = threadIdx.x % kWave;
+  u64 incl = v;
+#pragma unroll
+  for (int off = 1; off < kWave; off *= 2) {
+    const u64 t = shfl_up_u64(incl, off);
+    if (lane >= off) incl += t;
+  }
+  total = shfl_u64(incl, kWave - 1);
+  return incl - v;
+}
+// Over the workgroup, in thread order.  scratch: one u64 per wave.
+__device__ __forceinline__ u64 block_excl_scan(u64 v, u64* scratch, u64& total) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  u64 wave_total;
+  const u64 excl = wave_excl_scan(v, wave_total);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = wave_total;
+  __syncthreads();
+  u64 before = 0, all = 0;
+  for (int w = 0; w < kSampleThreads / kWave; ++w) {
+    if (w < wave) before += scratch[w];
+    all += scratch[w];
+  }
+  total = all;
+  return before + excl;
+}
+
+struct Found {
+  int bucket;   // -1: the running total never got there
+  u64 before;   // the total of the buckets before it
+};
+// The first bucket, from the row's largest value on, at which the running total reaches `need`
+// (strict: exceeds it).
+template <typename H>
+__device__ Found find_bucket(const H* hist, u64 need, bool strict, u64* scratch, Found* out) {
+  const int tid = threadIdx.x;
+  u64 loc[4], mine = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    loc[j] = hist[4 * tid + j];
+    mine += loc[j];
+  }
+  if (tid == 0) out->bucket = -1;
+  u64 total;
+  u64 run = block_excl_scan(mine, scratch, total);  // its barriers order the line above and the ones below
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const u64 next = run + loc[j];
+    if (strict ? (run <= need && next > need) : (run < need && next >= need)) {
+      out->bucket = 4 * tid + j;
+      out->before = run;
+    }
+    run = next;
+  }
+  __syncthreads();
+  const Found f = *out;
+  __syncthreads();
+  return f;
+}
+
+// The keys of bucket b into the list; returns how many there are (more than kListCap: too many).
+__device__ int collect_bucket(const float* x, int V, float inv_t, float zmax, int b, uint32_t* list, int* counter) {
+  if (threadIdx.x == 0) *counter = 0;
+  __syncthreads();
+  constexpr int U = 8;  // loads in flight per thread
+  for (int i0 = threadIdx.x; i0 < V; i0 += U * kSampleThreads) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = i0 + u * kSampleThreads < V ? x[i0 + u * kSampleThreads] : 0.f;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float zi = v[u] * inv_t;
+      if (i0 + u * kSampleThreads < V && bucket_of(zi, zmax) == b) {
+        const int at = atomicAdd(counter, 1);
+        if (at < kListCap) list[at] = order_key(zi);
+      }
+    }
+  }
+  __syncthreads();
+  const int n = *counter;
+  __syncthreads();
+  return n;
+}
+
+// The largest key K for which before + (weight of the list's keys >= K, those below `floor_key` left out)
+// reaches `need` (strict: exceeds it).  The weight of a key is 1, or its mass.  The caller knows that the
+// whole list gets there and that `before` alone does not.  By digits of at most 8 bits, from the
+// highest bit in which the list's keys differ.
+template <bool BY_MASS>
+__device__ uint32_t select_in_list(const uint32_t* list, int n, uint32_t floor_key, float zmax, u64 before, u64 need,
+                                   bool strict, u64* hist256, uint32_t* range, Found* out) {
+  const int tid = threadIdx.x, lane = tid % kWave;
+  if (tid == 0) {
+    range[0] = 0xffffffffu;
+    range[1] = 0;
+  }
+  __syncthreads();
+  for (int i = tid; i < n; i += kSampleThreads) {
+    atomicMin(&range[0], list[i]);
+    atomicMax(&range[1], list[i]);
+  }
+  __syncthreads();
+  const uint32_t kmin = range[0], kmax = range[1];
+  __syncthreads();
+  if (kmin == kmax) return kmax;
+  int bits_left = 32 - __clz(kmin ^ kmax);  // the bits above are the same in every key
+  uint32_t prefix = bits_left == 32 ? 0u : (kmax >> bits_left) << bits_left;
+  while (bits_left > 0) {
+    const int nb = bits_left < 8 ? bits_left : 8, shift = bits_left - nb;
+    if (tid < 256) hist256[tid] = 0;
+    __syncthreads();
+    for (int i0 = 0; i0 < n; i0 += kSampleThreads) {
+      const int i = i0 + tid;
+      uint32_t key = 0;
+      bool live = false;
+      if (i < n) {
+        key = list[i];
+        live = key >= floor_key && (bits_left == 32 || (key >> bits_left) == (prefix >> bits_left));
+      }
+      const int digit = (key >> shift) & ((1u << nb) - 1u);
+      const u64 w = !live ? 0 : (BY_MASS ? mass_of(value_of_key(key), zmax) : 1);
+      // when the wave's live keys all have the same digit (the keys of a bucket are close), one add does it
+      const unsigned long long live_mask = __builtin_amdgcn_ballot_w64(live);
+      if (live_mask == 0) continue;
+      const int first = __ffsll(static_cast<long long>(live_mask)) - 1;
+      const int d0 = __shfl(digit, first, kWave);
+      if (__builtin_amdgcn_ballot_w64(live && digit != d0) == 0) {
+        u64 dummy, all;
+        dummy = wave_excl_scan(w, all);
+        (void)dummy;
+        if (lane == first) atomicAdd(&hist256[d0], all);
+      } else if (live) {
+        atomicAdd(&hist256[digit], w);
+      }
+    }
+    __syncthreads();
+    if (tid < kWave) {  // the first wave: lane l looks after digits 255 - 4 l .. 252 - 4 l, from the top down
+      u64 loc[4], mine = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        loc[j] = hist256[255 - 4 * lane - j];
+        mine += loc[j];
+      }
+      u64 all;
+      u64 run = before + wave_excl_scan(mine, all);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u64 next = run + loc[j];
+        if (strict ? (run <= need && next > need) : (run < need && next >= need)) {
+          out->bucket = 255 - 4 * lane - j;
+          out->before = run;
+        }
+        run = next;
+      }
+    }
+    __syncthreads();
+    prefix |= static_cast<uint32_t>(out->bucket) << shift;
+    before = out->before;
+    bits_left = shift;
+    __syncthreads();
+  }
+  return prefix;
+}
+
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
@@ -93,11 +297,18 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   __shared__ ArgMax s_arg[kSampleThreads / kWave];
   __shared__ int s_cnt[kSampleThreads / kWave];
   __shared__ float s_f[kSampleThreads / kWave];
-  __shared__ float s_chunk[kSampleThreads];
-  __shared__ int s_pick;
-  __shared__ float s_prefix;
+  __shared__ u64 s_scan[kSampleThreads / kWave];
+  __shared__ uint32_t s_hist_cnt[kBuckets];
+  __shared__ u64 s_hist_mass[kBuckets];  // later: the segments' sums of the draw (floats)
+  __shared__ uint32_t s_list[kListCap];
+  __shared__ u64 s_hist256[256];
+  __shared__ uint32_t s_range[2];
+  __shared__ Found s_found;
+  __shared__ int s_counter;
+  __shared__ int s_pick, s_last;
+  __shared__ float s_prefix, s_target;
 
-  const int row = blockIdx.x, tid = threadIdx.x;
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const float* x = logits + static_cast<size_t>(row) * ld;
 
   ArgMax am{LYP_NEG_INF, 0x7fffffff};
@@ -115,96 +326,220 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     }
     return;
   }
-  const float zmax = am.v / T;
+  // a token's value is its logit times 1 / T, here and in every pass below
+  const float inv_t = 1.0f / T;
+  const float zmax = am.v * inv_t;
 
   // Smallest order key that survives the cut-offs; 0 keeps everything.
   uint32_t keep = 0;
   const int k = top_k[row];
-  if (k > 0 && k < V) {
-    uint32_t K = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = K | (1u << bit);
-      int c = 0;
-      for (int i = tid; i < V; i += kSampleThreads) c += order_key(x[i] / T) >= cand;
-      if (block_count(c, s_cnt) >= k) K = cand;
-    }
-    keep = K;  // the key of the k-th largest value
-  }
   const float p = top_p[row];
-  if (p < 1.0f) {
-    float z = 0.f;
-    for (int i = tid; i < V; i += kSampleThreads) {
-      const float zi = x[i] / T;
-      if (order_key(zi) >= keep) z += expf(zi - zmax);
+  const bool cut_k = k > 0 && k < V, cut_p = p < 1.0f;
+  bool whole_row = false;  // the cut-offs by bisection over the whole row
+  if (cut_k || cut_p) {
+    for (int b = tid; b < kBuckets; b += kSampleThreads) {
+      s_hist_cnt[b] = 0;
+      s_hist_mass[b] = 0;
     }
-    const float budget = p * block_sum(z, s_f);
-    // Largest key whose strictly-greater mass still exceeds the budget; the
-    // next key is the smallest that is kept.
-    uint32_t K = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t cand = K | (1u << bit);
-      float mass = 0.f;
-      for (int i = tid; i < V; i += kSampleThreads) {
-        const float zi = x[i] / T;
-        const uint32_t key = order_key(zi);
-        if (key > cand && key >= keep) mass += expf(zi - zmax);
+    __syncthreads();
+    constexpr int U = 8;  // loads in flight per thread
+    for (int i0 = tid; i0 < V; i0 += U * kSampleThreads) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = i0 + u * kSampleThreads < V ? x[i0 + u * kSampleThreads] : 0.f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (i0 + u * kSampleThreads >= V) continue;
+        const float zi = v[u] * inv_t;
+        const int b = bucket_of(zi, zmax);
+        if (cut_k) atomicAdd(&s_hist_cnt[b], 1u);
+        if (cut_p) atomicAdd(&s_hist_mass[b], mass_of(zi, zmax));
       }
-      if (block_sum(mass, s_f) > budget) K = cand;
     }
-    if (K + 1 > keep) keep = K + 1;
+    __syncthreads();
+    int bucket_k = -1, n_list = 0;
+    if (cut_k) {
+      const Found f = find_bucket(s_hist_cnt, static_cast<u64>(k), false, s_scan, &s_found);
+      bucket_k = f.bucket;
+      if (f.bucket < 0 || f.bucket == kBuckets - 1) {
+        whole_row = true;
+      } else {
+        n_list = collect_bucket(x, V, inv_t, zmax, f.bucket, s_list, &s_counter);
+        if (n_list > kListCap) whole_row = true;
+        else
+          keep = select_in_list<false>(s_list, n_list, 0u, zmax, f.before, static_cast<u64>(k), false, s_hist256,
+                                       s_range, &s_found);
+      }
+    }
+    if (cut_p && !whole_row) {
+      if (cut_k) {
+        // what top-k dropped leaves the masses: the buckets after its bucket, and of that bucket
+        // the keys below the cut-off
+        u64 kept = 0;
+        for (int i = tid; i < n_list; i += kSampleThreads)
+          if (s_list[i] >= keep) kept += mass_of(value_of_key(s_list[i]), zmax);
+        u64 kept_all;
+        (void)block_excl_scan(kept, s_scan, kept_all);
+        for (int b = tid; b < kBuckets; b += kSampleThreads)
+          if (b > bucket_k) s_hist_mass[b] = 0;
+        if (tid == 0) s_hist_mass[bucket_k] = kept_all;
+        __syncthreads();
+      }
+      u64 mine = 0, total;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) mine += s_hist_mass[4 * tid + j];
+      (void)block_excl_scan(mine, s_scan, total);
+      const u64 budget = static_cast<u64>(static_cast<double>(p) * static_cast<double>(total));
+      const Found f = find_bucket(s_hist_mass, budget, true, s_scan, &s_found);
+      if (f.bucket == kBuckets - 1) {
+        whole_row = true;
+      } else if (f.bucket >= 0) {
+        if (f.bucket != bucket_k) n_list = collect_bucket(x, V, inv_t, zmax, f.bucket, s_list, &s_counter);
+        if (n_list > kListCap) {
+          whole_row = true;
+        } else {
+          const uint32_t keep_p = select_in_list<true>(s_list, n_list, keep, zmax, f.before, budget, true, s_hist256,
+                                                       s_range, &s_found);
+          if (keep_p > keep) keep = keep_p;
+        }
+      }
+    }
+  }
+  if (whole_row) {
+    keep = 0;
+    if (cut_k) {
+      uint32_t K = 0;
+      for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t cand = K | (1u << bit);
+        int c = 0;
+        for (int i = tid; i < V; i += kSampleThreads) c += order_key(x[i] * inv_t) >= cand;
+        if (block_count(c, s_cnt) >= k) K = cand;
+      }
+      keep = K;  // the key of the k-th largest value
+    }
+    if (cut_p) {
+      float z = 0.f;
+      for (int i = tid; i < V; i += kSampleThreads) {
+        const float zi = x[i] * inv_t;
+        if (order_key(zi) >= keep) z += __expf(zi - zmax);
+      }
+      const float budget = p * block_sum(z, s_f);
+      // Largest key whose strictly-greater mass still exceeds the budget; the
+      // next key is the smallest that is kept.
+      uint32_t K = 0;
+      for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t cand = K | (1u << bit);
+        float mass = 0.f;
+        for (int i = tid; i < V; i += kSampleThreads) {
+          const float zi = x[i] * inv_t;
+          const uint32_t key = order_key(zi);
+          if (key > cand && key >= keep) mass += __expf(zi - zmax);
+        }
+        if (block_sum(mass, s_f) > budget) K = cand;
+      }
+      if (K + 1 > keep) keep = K + 1;
+    }
   }
 
-  // Inverse CDF in token order: each thread owns one contiguous run of tokens.
-  const int chunk = (V + kSampleThreads - 1) / kSampleThreads;
-  const int begin = min(V, tid * chunk), end = min(V, begin + chunk);
-  float mine = 0.f;
-  for (int i = begin; i < end; ++i) {
-    const float zi = x[i] / T;
-    if (order_key(zi) >= keep) mine += expf(zi - zmax);
-  }
-  s_chunk[tid] = mine;
+  // The draw: the inverse of the cumulative distribution in token order.  The row in segments of
+  // `seg` tokens (64, more for a vocabulary beyond 64 * kMaxSegs): every wave adds up segments, the
+  // segment that holds the target follows from the running totals, and one wave finds the token in it.
+  float* s_seg = reinterpret_cast<float*>(s_hist_mass);
+  constexpr int kSegBlocks = 8;  // a segment is at least 8 x 64 tokens: one sum across the lanes per 512 tokens
+  const int seg = kWave * max(kSegBlocks, (V + kWave * kMaxSegs - 1) / (kWave * kMaxSegs));
+  const int nseg = (V + seg - 1) / seg;
+  auto weight_of = [&](float v) {
+    const float zi = v * inv_t;
+    return order_key(zi) >= keep ? __expf(zi - zmax) : 0.f;
+  };
+  auto weight = [&](int i) { return i < V ? weight_of(x[i]) : 0.f; };
   __syncthreads();
+  constexpr int kWaves = kSampleThreads / kWave;
+  if (seg == kSegBlocks * kWave) {
+    for (int sg = wave; sg < nseg; sg += kWaves) {
+      float v[kSegBlocks];  // the segment's loads all in flight
+#pragma unroll
+      for (int u = 0; u < kSegBlocks; ++u) {
+        const int i = sg * seg + u * kWave + lane;
+        v[u] = i < V ? x[i] : LYP_NEG_INF;
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int u = 0; u < kSegBlocks; ++u) acc += (sg * seg + u * kWave + lane) < V ? weight_of(v[u]) : 0.f;
+      acc = wave_sum(acc);
+      if (lane == 0) s_seg[sg] = acc;
+    }
+  } else {
+    for (int sg = wave; sg < nseg; sg += kWaves) {
+      float acc = 0.f;
+      for (int j = 0; j < seg; j += kWave) acc += weight(sg * seg + j + lane);
+      acc = wave_sum(acc);
+      if (lane == 0) s_seg[sg] = acc;
+    }
+  }
   if (tid == 0) {
-    float total = 0.f;
-    for (int t = 0; t < kSampleThreads; ++t) total += s_chunk[t];
-    const float target = uniform[row] * total;
-    float prefix = 0.f;
-    int pick = -1, last_nonempty = 0;
-    for (int t = 0; t < kSampleThreads; ++t) {
-      if (s_chunk[t] > 0.f) last_nonempty = t;
-      if (pick < 0 && prefix + s_chunk[t] > target && s_chunk[t] > 0.f) {
-        pick = t;
-        s_prefix = prefix;
-      }
-      if (pick < 0) prefix += s_chunk[t];
-    }
-    if (pick < 0) {  // rounding pushed the target to the total: take the last token that has mass
-      pick = last_nonempty;
-      s_prefix = LYP_NEG_INF;
-    }
-    s_pick = pick;
-    s_chunk[0] = target;
+    s_pick = -1;
+    s_last = 0;
   }
   __syncthreads();
-  if (tid == s_pick) {
-    const float target = s_chunk[0];
-    float run = s_prefix;
-    int token = -1, last_kept = begin;
-    for (int i = begin; i < end; ++i) {
-      const float zi = x[i] / T;
-      if (order_key(zi) < keep) continue;
-      const float e = expf(zi - zmax);
-      if (e <= 0.f) continue;
-      last_kept = i;
-      run += e;
-      if (run > target) {
-        token = i;
-        break;
+  const int per = (nseg + kSampleThreads - 1) / kSampleThreads;
+  const int sg_begin = min(nseg, tid * per), sg_end = min(nseg, sg_begin + per);
+  float mine = 0.f;
+  for (int sg = sg_begin; sg < sg_end; ++sg) mine += s_seg[sg];
+  // running totals over the threads, in thread order: within a wave by shuffles, the waves one after the other
+  float incl = mine;
+#pragma unroll
+  for (int off = 1; off < kWave; off *= 2) {
+    const float t = __shfl_up(incl, off, kWave);
+    if (lane >= off) incl += t;
+  }
+  if (lane == kWave - 1) s_f[wave] = incl;
+  __syncthreads();
+  float before = 0.f, total = 0.f;
+  for (int w = 0; w < kSampleThreads / kWave; ++w) {
+    if (w < wave) before += s_f[w];
+    total += s_f[w];
+  }
+  const float target = uniform[row] * total;
+  float run = before + (incl - mine);
+  for (int sg = sg_begin; sg < sg_end; ++sg) {
+    const float sv = s_seg[sg], next = run + sv;
+    if (sv > 0.f) {
+      atomicMax(&s_last, sg);
+      if (run <= target && next > target) {
+        s_pick = sg;
+        s_prefix = run;
       }
     }
-    const int pick = token >= 0 ? token : last_kept;
-    out[row] = pick;
-    if (mirror) mirror[row] = pick;
+    run = next;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    // rounding may have pushed the target to the total: then the last token that has mass is taken
+    const bool found = s_pick >= 0;
+    const int sg = found ? s_pick : s_last;
+    float run_w = found ? s_prefix : LYP_NEG_INF;
+    int token = -1, last_kept = -1;
+    for (int j = 0; j < seg && token < 0; j += kWave) {
+      const int i = sg * seg + j + lane;
+      const float e = weight(i);
+      float in = e;
+#pragma unroll
+      for (int off = 1; off < kWave; off *= 2) {
+        const float t = __shfl_up(in, off, kWave);
+        if (lane >= off) in += t;
+      }
+      const unsigned long long has = __builtin_amdgcn_ballot_w64(e > 0.f);
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(e > 0.f && run_w + in > target);
+      if (has) last_kept = sg * seg + j + (63 - __clzll(static_cast<long long>(has)));
+      if (hit) token = sg * seg + j + (__ffsll(static_cast<long long>(hit)) - 1);
+      run_w += __shfl(in, kWave - 1, kWave);
+    }
+    if (lane == 0) {
+      const int pick = token >= 0 ? token : (last_kept >= 0 ? last_kept : am.i);
+      out[row] = pick;
+      if (mirror) mirror[row] = pick;
+    }
   }
 }
 

@@ -575,6 +575,57 @@ def test_sampler_greedy_and_draws(ops):
             assert lo - 1e-5 <= u_val <= float(cdf[got[r]]) + 1e-5, f"row {r}: u={u_val} not in [{lo}, {float(cdf[got[r]])}]"
 
 
+def _row(kind, V, g):
+    if kind == "peaked":       # as a trained model's: a few tokens stand out
+        x = torch.randn(V, generator=g) * 2.5
+        x[torch.randperm(V, generator=g)[:20]] += 9.0
+        return x
+    if kind == "flat":         # as random weights give: everything within a few units
+        return torch.randn(V, generator=g) * 0.3
+    if kind == "ties":         # many equal values, also at the cut-offs
+        return torch.randint(0, 6, (V,), generator=g).float() * 0.5
+    if kind == "masked":       # most tokens ruled out beforehand
+        x = torch.randn(V, generator=g)
+        x[torch.rand(V, generator=g) < 0.9] = float("-inf")
+        return x
+    if kind == "far":          # most tokens more than 32 from the largest: the last bucket
+        x = torch.randn(V, generator=g) - 60.0
+        x[torch.randperm(V, generator=g)[:30]] += 60.0
+        return x
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["peaked", "flat", "ties", "masked", "far"])
+@pytest.mark.parametrize("V", [1003, 32000, 128256])
+def test_sampler_cut_offs_against_the_sorted_reference(ops, V, kind):
+    """64 draws at evenly spread uniforms for several (temperature, top-k, top-p): every token must
+    be one that the plain (sorting) filter keeps, and sit where the uniform falls in the plain
+    cumulative distribution.  A kept set that is off by one token shifts that distribution."""
+    g = torch.Generator().manual_seed(V % 1000 + len(kind))
+    x = _row(kind, V, g)
+    n = 64
+    rows = x.expand(n, V).contiguous().to(DEV)
+    u = ((torch.arange(n) + 0.37) / n).float()
+    work = ops.sample_workspace(n, DEV)
+    for temp, tk, tp in [(0.8, -1, 1.0), (1.0, 40, 1.0), (0.7, -1, 0.9), (1.3, 200, 0.6), (1.0, V - 3, 0.999),
+                         (0.9, 1, 0.5), (1.0, 3000, 1.0)]:
+        tk = min(tk, V)
+        if kind == "ties" and tp < 1.0:
+            continue   # which of the equal tokens at the cut-off stay is the sort's whim there; here all of them do
+        out = torch.empty(n, dtype=torch.int32, device=DEV)
+        ops.sample(rows, torch.full((n,), temp).to(DEV), torch.full((n,), tk, dtype=torch.int32).to(DEV),
+                   torch.full((n,), tp).to(DEV), u.to(DEV), out, work)
+        got = out.cpu().tolist()
+        probs = P.sample_filter(x, temp, tk, tp)
+        cdf = torch.cumsum(probs, 0)
+        for r in range(n):
+            t = got[r]
+            assert probs[t] > 0, f"{kind} V={V} T={temp} k={tk} p={tp}: token {t} is not in the kept set"
+            lo, hi = float(cdf[t] - probs[t]), float(cdf[t])
+            assert lo - 2e-5 <= float(u[r]) <= hi + 2e-5, \
+                f"{kind} V={V} T={temp} k={tk} p={tp}: u={float(u[r])} outside [{lo}, {hi}] of token {t}"
+
+
 def test_table_from_pinned_memory(ops):
     """A table of integers read from pinned host memory by the kernel itself, a
     few words of it replaced by values that only the device holds."""
