@@ -620,6 +620,10 @@ struct TileRegs {
   bool lost[PER];  // the table had no page for the piece's block
 };
 
+// n_parts > 1 (grid z): a unit's key tiles are dealt to n_parts workgroups in runs; each leaves its
+// running result (not normalised) in part_o [tile][token of the tile][head][part][hd] and part_ml
+// [...][part][2] = (maximum in the base-2 domain, sum), and attn_merge_parts_kernel puts them together:
+// for few new tokens over many keys, which would otherwise be one long walk on few compute units.
 // KS = 2: two sets of NW waves share a unit; set 0 takes the unit's key tiles 0, 2, 4, ..., set 1 the
 // tiles 1, 3, 5, ..., each through LDS buffers of its own, and the two running results are merged
 // at the end.  Half as many tiles in a row for one unit: for launches with few units, whose time
@@ -630,7 +634,8 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
-    int bs, int window, float scale_log2, int paired) {
+    int bs, int window, float scale_log2, int paired, float* __restrict__ part_o, float* __restrict__ part_ml,
+    int n_parts) {
   using T = bf16_t;
   using WT = WideTile;
   using MMA = Mma16Wide<bf16_t>;
@@ -742,7 +747,13 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     // that holds a key of interest the table may hold anything, so the index is clamped there.
     const int32_t* table = block_tables + static_cast<size_t>(seq) * max_blocks;
     const int blk_last = (hi_wg - 1) / bs;
-    const int kt_base = (lo_wg / KT) * KT;      // the unit's first tile
+    int kt_base = (lo_wg / KT) * KT;            // the first tile of the unit, then of this workgroup's run
+    int kt_end = hi_wg;                         // where the run ends
+    if (n_parts > 1) {
+      const int run = ((hi_wg - kt_base + KT - 1) / KT + n_parts - 1) / n_parts * KT;
+      kt_base += static_cast<int>(blockIdx.z) * run;
+      kt_end = min(hi_wg, kt_base + run);
+    }
     const int kt_first = kt_base + set * KT;    // this set's first tile
     int w_blk[PER], w_off[PER];      // the walk: the block of the tile whose table entry is read next
     int page[PER], page_off[PER];    // for the tile whose data is asked for next
@@ -847,9 +858,9 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
         page[n] = page_n[n];
         page_off[n] = page_off_n[n];
       }
-      if (wave_active && kt0 <= pos_last_w) compute(buf, kt0);
+      if (wave_active && kt0 <= pos_last_w && kt0 < kt_end) compute(buf, kt0);
       if (WT::kBufs == 1) __syncthreads();  // everyone is done with the only buffer before it is overwritten
-      if (kt0 + KSTEP < hi_wg) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KSTEP);
+      if (kt0 + KSTEP < kt_end) stash(ready, WT::kBufs == 2 ? buf ^ 1 : 0, kt0 + KSTEP);
       __syncthreads();
     };
 
@@ -862,9 +873,9 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     stash(ra, 0, kt_first);
     __syncthreads();
     // the bounds are those of set 0, so that every wave passes the same barriers
-    for (int kb = kt_base; kb < hi_wg; kb += 2 * KSTEP) {
+    for (int kb = kt_base; kb < kt_end; kb += 2 * KSTEP) {
       step(kb + set * KT, 0, ra, rb);
-      if (kb + KSTEP >= hi_wg) break;
+      if (kb + KSTEP >= kt_end) break;
       step(kb + KSTEP + set * KT, WT::kBufs == 2 ? 1 : 0, rb, ra);
     }
 
@@ -890,11 +901,24 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
         for (int db = 0; db < kSteps; ++db)
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[db][i] = o[db][i] * a0 + hand[(2 + 4 * db + i) * kWave] * a1;
+        m_run = m_new;  // what the sum and the output are relative to now
       }
       __syncthreads();  // the buffers are free for the next unit
     }
 
-    if (col_valid && set == 0) {
+    if (n_parts > 1) {
+      if (col_valid && set == 0) {
+        const int in_tile = q0_w - tile_q0[tile] + col;
+        const size_t pidx = ((static_cast<size_t>(tile) * 64 + in_tile) * nh + head) * n_parts + blockIdx.z;
+        float* po = part_o + pidx * HD + 4 * grp;
+#pragma unroll
+        for (int db = 0; db < kSteps; ++db) *reinterpret_cast<f32x4*>(po + db * 16) = o[db];
+        if (grp == 0) {
+          part_ml[pidx * 2] = m_run;
+          part_ml[pidx * 2 + 1] = lacc[0];
+        }
+      }
+    } else if (col_valid && set == 0) {
       const float inv = lacc[0] > 0.f ? 1.0f / lacc[0] : 0.f;
       T* orow = out + (static_cast<size_t>(tok0) + q0_w + col) * out_stride + static_cast<size_t>(head) * HD + 4 * grp;
 #pragma unroll
@@ -905,6 +929,33 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
         *reinterpret_cast<bf16x4*>(orow + db * 16) = f;
       }
     }
+  }
+}
+
+// grid (nh, 64, tiles); one wave: the parts of one new token and head, put together.
+template <typename T>
+__global__ __launch_bounds__(64) void attn_merge_parts_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, int n_parts,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0,
+    T* __restrict__ out, int out_stride, int nh) {
+  const int head = blockIdx.x, in_tile = blockIdx.y, tile = blockIdx.z, lane = threadIdx.x;
+  const int seq = tile_seq[tile];
+  const int tok0 = q_start[seq], q_len = q_start[seq + 1] - tok0;
+  const int q = tile_q0[tile] + in_tile;
+  if (q >= q_len) return;
+  const size_t base = ((static_cast<size_t>(tile) * 64 + in_tile) * nh + head) * n_parts;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
+  float m = LYP_NEG_INF;
+  for (int p = 0; p < n_parts; ++p) m = fmaxf(m, ml[p].x);
+  const float m_safe = m == LYP_NEG_INF ? 0.f : m;
+  float l = 0.f;
+  for (int p = 0; p < n_parts; ++p) l += fast_exp2(ml[p].x - m_safe) * ml[p].y;
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  T* orow = out + (static_cast<size_t>(tok0) + q) * out_stride + static_cast<size_t>(head) * HD;
+  for (int d = lane; d < HD; d += kWave) {
+    float acc = 0.f;
+    for (int p = 0; p < n_parts; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+    orow[d] = from_f32<T>(acc * inv);
   }
 }
 #endif
@@ -1118,6 +1169,8 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
   }
 }
 
+constexpr int kPrefillPartsMost = 16;
+
 // Compute units of the current device (asked once per process).
 static int compute_units() {
   static int n = 0;
@@ -1170,13 +1223,36 @@ int lyp_attn_decode_plan(int n_seqs, int max_ctx, int nh, int nkv) {
   return kDecodeWaves * kpw;
 }
 
+// Into how many runs lyp_attn_prefill had better cut every unit's keys (1: not at all), for
+// n_tiles tiles of 64 new tokens of which one sees max_keys keys.  More than one needs a workspace:
+// n_tiles * 64 * nh * parts * hd floats for part_o, n_tiles * 64 * nh * parts * 2 for part_ml.
+int lyp_attn_prefill_plan(int n_tiles, int max_keys, int nh, int nkv, int dtype, int bs) {
+#if LYP_HEAD_DIM % 32 == 0 && !defined(LYP_PREFILL_NARROW)
+  if (dtype != kBF16 || bs <= 0 || bs % 16 != 0 || nkv <= 0 || n_tiles <= 0) return 1;
+  const int g = nh / nkv;
+  const int gh = g >= 4 ? 4 : (g >= 2 ? 2 : 1);
+  const int unit_tokens = ((gh == 1 ? 4 : 8) / gh) * 16;
+  const long long wgs = static_cast<long long>(n_tiles) * (64 / unit_tokens) * nkv * ((g + gh - 1) / gh);
+  const int tiles = (max_keys + WideTile::kKeys - 1) / WideTile::kKeys;
+  int parts = 1;
+  // as measured: up to a workgroup per compute unit, and runs of 8 tiles at least
+  while (parts < kPrefillPartsMost && wgs * parts < compute_units() && tiles / (2 * parts) >= 8) parts *= 2;
+  return parts;
+#else
+  (void)n_tiles, (void)max_keys, (void)nh, (void)nkv, (void)dtype, (void)bs;
+  return 1;
+#endif
+}
+
 int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
                      const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* tile_seq,
                      const int32_t* tile_q0, int n_tiles, int nh, int nkv, int bs, int window, float scale,
-                     int pair, hipStream_t stream) {
+                     int pair, float* part_o, float* part_ml, int n_parts, hipStream_t stream) {
   if (check_common("attn_prefill", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
   LYP_REQUIRE(n_tiles >= 0, "attn_prefill: %d tiles", n_tiles);
+  LYP_REQUIRE(n_parts >= 1 && n_parts <= kPrefillPartsMost && (n_parts == 1 || (part_o && part_ml)),
+              "attn_prefill: %d parts of the keys (at most %d, with a workspace)", n_parts, kPrefillPartsMost);
   if (n_tiles == 0) return 0;
   const int g = nh / nkv;
   // Heads per workgroup: as many of the group as four waves hold; the waves
@@ -1210,16 +1286,16 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
       block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
-      scale_log2, paired)
+      scale_log2, paired, part_o, part_ml, n_parts)
     // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
     // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
   do {                                                                                                        \
     constexpr int kQW = (NW / GH) * 16;                                                                       \
     const int units = n_tiles * (64 / kQW);                                                                   \
-    const long long wgs = static_cast<long long>(units) * nkv * head_groups;                                  \
-    const int paired = (pair & 1) != 0 && wgs > compute_units();                                              \
-    dim3 grid(nkv * head_groups, paired ? (units + 1) / 2 : units);                                           \
+    const long long wgs = static_cast<long long>(units) * nkv * head_groups * n_parts;                        \
+    const int paired = (pair & 1) != 0 && n_parts == 1 && wgs > compute_units();                              \
+    dim3 grid(nkv * head_groups, paired ? (units + 1) / 2 : units, n_parts);                                  \
     if (HD <= 64 && split_ok && wgs <= static_cast<long long>(kSplitBelow) * compute_units()) {               \
       if constexpr (HD <= 64) LYP_PREFILL_WIDE_KS(GH, NW, 2);                                                 \
     } else {                                                                                                  \
@@ -1233,6 +1309,9 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     else LYP_PREFILL_WIDE(1, 4);
 #undef LYP_PREFILL_WIDE
 #undef LYP_PREFILL_WIDE_KS
+    if (n_parts > 1)
+      attn_merge_parts_kernel<bf16_t><<<dim3(nh, 64, n_tiles), 64, 0, stream>>>(
+          part_o, part_ml, n_parts, q_start, tile_seq, tile_q0, static_cast<bf16_t*>(out), out_stride, nh);
     LYP_LAUNCH_CHECK("attn_prefill");
     return 0;
   }

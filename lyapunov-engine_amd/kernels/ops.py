@@ -88,7 +88,8 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
             raise KernelError(f"attention library for head size {head_dim} reports {lib.lyp_attn_head_dim()}")
         lib.lyp_attn_prefill.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                         c_float, c_int, c_void_p]
+                                         c_float, c_int, c_void_p, c_void_p, c_int, c_void_p]
+        lib.lyp_attn_prefill_plan.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
         lib.lyp_attn_decode.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                         c_int, c_int, c_int, c_float, c_void_p]
@@ -560,6 +561,14 @@ def attn_decode_plan(n_seqs: int, max_ctx: int, num_heads: int, num_kv_heads: in
     return attention_lib(head_dim).lyp_attn_decode_plan(n_seqs, max_ctx, num_heads, num_kv_heads)
 
 
+def attn_prefill_plan(n_tiles: int, max_keys: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                      dtype: torch.dtype, page_size: int) -> int:
+    """Into how many runs a prefill launch had better cut every tile's keys
+    (1: not at all) when one of its ``n_tiles`` tiles sees ``max_keys`` keys."""
+    return attention_lib(head_dim).lyp_attn_prefill_plan(n_tiles, max_keys, num_heads, num_kv_heads, _code(dtype),
+                                                         page_size)
+
+
 def _attn_check(q, out, kpool, vpool, block_tables, nh, nkv, hd):
     _dev(out, kpool, vpool, block_tables)
     n_pages, bs = kpool.shape[0], kpool.shape[2]
@@ -578,7 +587,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
                  block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor, tile_seq: torch.Tensor,
                  tile_q0: torch.Tensor, n_tiles: int, *, num_heads: int, num_kv_heads: int, head_dim: int,
                  window: int = 0, scale: float | None = None, pair: bool | None = None,
-                 split: bool = True) -> torch.Tensor:
+                 split: bool = True, parts: int = 1, part_o: torch.Tensor | None = None,
+                 part_ml: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache (which already
     holds their own keys).  q is a view [T, >= nh * hd] whose first nh * hd
     columns are the query heads; a tile is 64 new tokens of one request, and
@@ -586,17 +596,27 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
     says whether the first tiles see far fewer keys than the last (then a
     workgroup may take one of each); None leaves it to the kernel's launcher.
     ``split=False`` keeps a small launch from sharing a tile's keys between
-    two sets of waves (a different order of additions, for tests)."""
+    two sets of waves (a different order of additions, for tests).  ``parts``
+    > 1 (see ``attn_prefill_plan``) cuts every tile's keys into that many runs
+    for workgroups of their own; it needs float workspaces ``part_o`` of
+    n_tiles * 64 * heads * parts * head_dim and ``part_ml`` of n_tiles * 64 *
+    heads * parts * 2 elements."""
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
-    _dev(q_start, ctx_len, tile_seq, tile_q0)
+    _dev(q_start, ctx_len, tile_seq, tile_q0, part_o, part_ml)
+    if parts > 1:
+        need = n_tiles * 64 * num_heads * parts
+        if part_o is None or part_ml is None or part_o.dtype != torch.float32 or part_ml.dtype != torch.float32 or \
+                part_o.numel() < need * head_dim or part_ml.numel() < need * 2:
+            raise KernelError("attention: the workspace for the parts of the keys is missing or too small")
     lib = attention_lib(head_dim)
     scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
     _check(lib.lyp_attn_prefill(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
                                 _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(tile_seq),
                                 _p(tile_q0), n_tiles, num_heads, num_kv_heads, bs, window, scale,
-                                (1 if pair is None else int(bool(pair))) | (0 if split else 2), _stream()), lib)
+                                (1 if pair is None else int(bool(pair))) | (0 if split else 2), _p(part_o),
+                                _p(part_ml), parts, _stream()), lib)
     return out
 
 

@@ -77,8 +77,17 @@ class PagedAttention(Mixer):
             # Tiles come in rising order of the keys they see; when the first sees less than half
             # of what the last does, a workgroup may take one from each end.
             few, many = (min(k, self.window + 64) if self.window else k for k in ctx.tile_keys)
+            # few new tokens over many keys: the keys in runs, for workgroups of their own
+            parts = ops.attn_prefill_plan(ctx.n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim,
+                                          ctx.dtype, g.page_size)
+            part_o = part_ml = None
+            if parts > 1:
+                n = ctx.n_tiles * 64 * self.num_heads * parts
+                part_o = ctx.scratch("attn_part_o", n * self.head_dim)
+                part_ml = ctx.scratch("attn_part_ml", n * 2)
             ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.tile_seq,
-                             ctx.tile_q0, ctx.n_tiles, pair=2 * few <= many, **common)
+                             ctx.tile_q0, ctx.n_tiles, pair=2 * few <= many, parts=parts, part_o=part_o,
+                             part_ml=part_ml, **common)
         if ctx.n_dec:
             part = ops.attn_decode_plan(ctx.n_dec, ctx.max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
             max_parts = max(1, (ctx.max_ctx_dec + part - 1) // part)

@@ -56,15 +56,20 @@ def attn_prefill(a) -> None:
     tile_seq = torch.zeros(n_tiles, dtype=torch.int32, device=dev)
     tile_q0 = (torch.arange(n_tiles, dtype=torch.int32) * 64).to(dev)
     pair = 2 * (ctx - S + 64) <= ctx
+    parts = a.parts or ops.attn_prefill_plan(n_tiles, ctx, a.heads, a.kv_heads, a.head_dim, dt, a.page_size)
+    work = {}
+    if parts > 1:
+        n = n_tiles * 64 * a.heads * parts
+        work = dict(parts=parts, part_o=torch.empty(n * a.head_dim, device=dev), part_ml=torch.empty(n * 2, device=dev))
 
     def run():
         ops.attn_prefill(q, out, k, v, table, q_start, ctx_len, tile_seq, tile_q0, n_tiles, num_heads=a.heads,
-                         num_kv_heads=a.kv_heads, head_dim=a.head_dim, pair=pair)
+                         num_kv_heads=a.kv_heads, head_dim=a.head_dim, pair=pair, **work)
 
     t = _time(run, a.repeat)
     flops = 4 * a.heads * a.head_dim * (S * (ctx - S) + S * S / 2)
     print(f"attn_prefill tokens={S} context={ctx} heads={a.heads}/{a.kv_heads}x{a.head_dim} {a.dtype}: "
-          f"{t * 1e6:.1f} us  {flops / t / 1e12:.1f} TFLOP/s")
+          f"{t * 1e6:.1f} us  {flops / t / 1e12:.1f} TFLOP/s  (keys in {parts} run{'s' if parts > 1 else ''})")
 
 
 def attn_decode(a) -> None:
@@ -130,6 +135,7 @@ def main(argv=None) -> None:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--tokens", type=int, default=2048, help="attn_prefill: new tokens of the request")
     ap.add_argument("--context", type=int, default=0, help="keys per request after the step")
+    ap.add_argument("--parts", type=int, default=0, help="attn_prefill: runs of keys per tile (0: as planned)")
     ap.add_argument("--batch", type=int, default=8, help="attn_decode: requests")
     ap.add_argument("--rows", type=int, default=8, help="linear: rows of activations")
     ap.add_argument("--in-features", type=int, default=2048)

@@ -407,11 +407,13 @@ PREFILL_CASES = [
 ]
 
 
-@pytest.mark.parametrize("split", [True, False], ids=["split", "whole"])
+@pytest.mark.parametrize("split,parts", [(True, 1), (False, 1), (True, 3), (False, 4)],
+                         ids=["split", "whole", "split-3-parts", "4-parts"])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("case", PREFILL_CASES, ids=[str(c[:5]) for c in PREFILL_CASES])
-def test_attention_prefill(ops, dtype, case, split):
-    """``split``: a small launch may give a tile's keys to two sets of waves in turn."""
+def test_attention_prefill(ops, dtype, case, split, parts):
+    """``split``: a small launch may give a tile's keys to two sets of waves in turn.  ``parts``: every
+    tile's keys in that many runs, for workgroups of their own, put together by a second kernel."""
     nh, nkv, hd, bs, window, seqs = case
     s = paged_setup(seqs, nh, nkv, hd, bs, dtype, seed=hd + bs)
     tile_seq, tile_q0 = [], []
@@ -419,12 +421,26 @@ def test_attention_prefill(ops, dtype, case, split):
         for q0 in range(0, ql, 64):
             tile_seq.append(b), tile_q0.append(q0)
     out = torch.full((s["q"].shape[0], nh * hd), float("nan"), dtype=dtype, device=DEV)
+    work = {}
+    if parts > 1:
+        n = len(tile_seq) * 64 * nh * parts
+        work = dict(parts=parts, part_o=torch.full((n * hd,), float("nan"), device=DEV),
+                    part_ml=torch.full((n * 2,), float("nan"), device=DEV))
     ops.attn_prefill(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
                      s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(tile_seq, dtype=torch.int32, device=DEV),
                      torch.tensor(tile_q0, dtype=torch.int32, device=DEV), len(tile_seq), num_heads=nh,
-                     num_kv_heads=nkv, head_dim=hd, window=window, split=split)
+                     num_kv_heads=nkv, head_dim=hd, window=window, split=split, **work)
     want = plain_attention(s, seqs, window)
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+
+
+def test_attention_prefill_plan(ops):
+    plan = lambda tiles, keys, dt=torch.bfloat16, bs=16: ops.attn_prefill_plan(tiles, keys, 32, 8, 64, dt, bs)
+    assert plan(32, 2048) == 1                 # a whole prompt: enough workgroups as it is
+    assert plan(8, 8192) == 2                  # 512 new tokens at the end of 8192
+    assert plan(1, 8192) > plan(8, 8192)       # fewer tokens, more runs
+    assert plan(8, 512) == 1                   # few keys: nothing to cut
+    assert plan(8, 8192, torch.float32) == 1 and plan(8, 8192, bs=4) == 1   # the other kernel has no parts
 
 
 DECODE_CASES = [
