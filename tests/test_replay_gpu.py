@@ -215,6 +215,28 @@ def test_sizes_that_are_no_powers_of_two(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_few_new_tokens_over_many_keys(tmp_path, dtype, monkeypatch):
+    """Portions of a prompt at the end of 1,300 tokens: in bfloat16 the attention kernel then cuts the
+    keys into runs for workgroups of their own (checked), and the logits stay the plain model's."""
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = dict(TINY["C"][0], max_position_embeddings=2048, num_hidden_layers=1)
+    write_random_model(dict(cfg), str(tmp_path), 11, dtype, init_std=0.1, norm_init_std=0.1)
+    reqs = {"a": random_tokens(1300, cfg["vocab_size"], 4), "b": random_tokens(1150, cfg["vocab_size"], 5)}
+    want = plain_logits(str(tmp_path), reqs)
+    seen, plan = [], ops.attn_prefill_plan
+    monkeypatch.setattr(ops, "attn_prefill_plan", lambda *a: seen.append(plan(*a)) or seen[-1])
+    t = Trace(reqs)
+    t.step([("a", 1100), ("b", 1024)], want="last")
+    t.step([("a", 70), ("b", 2)])            # 70 and 2 new tokens over 1,170 and 1,026 keys
+    t.step([("a", 100), ("b", 64)], want="last")
+    t.step([("a", 30), ("b", 60)], end=["a", "b"])
+    compare(t, replay(str(tmp_path), dtype, t), want, dtype, "many keys")
+    assert (max(seen) > 1) == (dtype == "bfloat16"), seen
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_folders, dtype):
     name = "B"
     reqs = {"long": random_tokens(400, TINY[name][0]["vocab_size"], seed=9)}
