@@ -201,7 +201,7 @@ __device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
   return head * t.hd + f;
 }
 
-// PAIRED (8 rows of W, at most 8 tokens): the tile's upper half repeats the 8 rows of W and the
+// PAIRED (8 rows of W, or two tiles of 8; at most 8 tokens): the tile's upper half repeats the 8 rows of W and the
 // tile's upper 8 columns the tokens, both 64 values of K further on, so that one matrix instruction
 // does two chunks of K (on the tile's diagonal blocks; the other two are not used) and no load
 // asks for a value twice.
@@ -214,7 +214,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   using Frag = typename MM::Frag;
   constexpr int NF = 16 / MM::kElems;  // fragments per lane per 64 values of K
   static_assert(ROWS == 16 || ROWS == 8, "a workgroup owns 16 rows of W, or 8 (the tile's lower half repeats them)");
-  static_assert(!PAIRED || (ROWS == 8 && MB == 1 && EPI == kEpiResidual), "two chunks per tile: 8 rows, 8 tokens");
+  // With 16 rows of W a paired wave keeps two tiles, rows 0-7 and 8-15, over the same tokens: MB counts them.
+  static_assert(!PAIRED || (EPI == kEpiResidual && ((ROWS == 8 && MB == 1) || (ROWS == 16 && MB == 2))),
+                "two chunks per tile: 8 rows (or twice 8), 8 tokens");
   constexpr int CHUNK = PAIRED ? 128 : 64;  // values of K per step of a wave
   extern __shared__ float red[];       // [waves][MB][64][4], then MB * 16 floats for the epilogues' row values
 
@@ -225,7 +227,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   const int nwaves = blockDim.x / kWave;
   const int n0 = blockIdx.x * ROWS;
   const int r = lane % 16, j = lane / 16;
-  int wrow = min(n0 + r % ROWS, N - 1);  // rows past the end read the last row and are not stored
+  int wrow = min(n0 + r % (PAIRED ? 8 : ROWS), N - 1);  // rows past the end read the last row and are not stored
   if constexpr (EPI == kEpiRope) wrow = rope_feature(tail, n0, r);  // N is a multiple of 16 here
 
   const int chunks = K / CHUNK;
@@ -266,9 +268,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   }
   float h_first = 0.f, nw_first = 0.f;  // kEpiResidual: what the thread's first element adds to and is weighted by
   if constexpr (EPI == kEpiResidual) {
-    const int e = threadIdx.x, l = (e % 256) / 4, row = 4 * (l / 16) + e % 4;
-    const int m = (e / 256) * 16 + l % 16, n = n0 + row;
-    if (e < MB * 256 && row < ROWS && m < M && n < N) {
+    const int e = threadIdx.x, l = (e % 256) / 4, in_tile = 4 * (l / 16) + e % 4;
+    const int row = PAIRED ? 8 * (e / 256) + in_tile : in_tile;
+    const int m = (PAIRED ? 0 : (e / 256) * 16) + l % 16, n = n0 + row;
+    if (e < MB * 256 && in_tile < (PAIRED ? 8 : ROWS) && m < M && n < N) {
       h_first = static_cast<const float*>(Cv)[static_cast<size_t>(m) * ldc + n];
       if (res.next_w)
         nw_first = res.next_w_f32 ? static_cast<const float*>(res.next_w)[n]
@@ -280,6 +283,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
   const int second = PAIRED ? (r / 8) * 64 : 0;  // the tile's upper half: the chunk's second 64 values
   const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems + second;
+  const T* wp_upper = wp;  // PAIRED with 16 rows: the same lanes' rows 8-15
+  if constexpr (PAIRED && MB == 2) wp_upper = W + static_cast<size_t>(min(n0 + 8 + r % 8, N - 1)) * ldw + j * MM::kElems + second;
   const T* ap[MB];  // rows past the end read the last row and are not stored
 #pragma unroll
   for (int b = 0; b < MB; ++b)
@@ -296,6 +301,24 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
       for (int f = 0; f < NF; ++f)
         wf[u][f] = *reinterpret_cast<const Frag*>(wp + (c + u) * CHUNK + f * 4 * MM::kElems);
+    if constexpr (PAIRED && MB == 2) {  // two tiles of weights over one set of activations
+      Frag wu[U][NF], xf[U][NF];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          wu[u][f] = *reinterpret_cast<const Frag*>(wp_upper + (c + u) * CHUNK + f * 4 * MM::kElems);
+          xf[u][f] = *reinterpret_cast<const Frag*>(ap[0] + (c + u) * CHUNK + f * 4 * MM::kElems);
+        }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) {
+          acc[0] = MM::mma(wf[u][f], xf[u][f], acc[0]);
+          acc[1] = MM::mma(wu[u][f], xf[u][f], acc[1]);
+        }
+      return;
+    }
     // the activations come from the cache: four chunks of them at a time are enough
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
@@ -330,7 +353,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
     if constexpr (PAIRED) {  // row + 8, token + 8: the chunks' second halves
       float upper = 0.f;
-      for (int w = 0; w < nwaves; ++w) upper += red[static_cast<size_t>(w) * 256 + e + 160];
+      for (int w = 0; w < nwaves; ++w) upper += red[static_cast<size_t>(w) * MB * 256 + e + 160];
       sum += upper;
     }
     if constexpr (NORMED) {
@@ -343,9 +366,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   float* sq_el = row_val + nwaves * 16;  // kEpiResidual with by-products: [256] squares of the new h, by element
   for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
     const int b = e / 256, l = (e % 256) / 4, i = e % 4;
-    const int row = 4 * (l / 16) + i;
-    const int m = b * 16 + l % 16, n = n0 + row;
-    if (row >= ROWS || m >= M || n >= N) continue;
+    const int in_tile = 4 * (l / 16) + i;
+    // PAIRED: tile b holds rows 8 b .. 8 b + 7 of W for tokens 0-7; else rows 0-15 for tokens 16 b .. + 15
+    const int row = PAIRED ? 8 * b + in_tile : in_tile;
+    const int m = (PAIRED ? 0 : b * 16) + l % 16, n = n0 + row;
+    if (in_tile >= (PAIRED ? 8 : ROWS) || m >= M || n >= N) continue;
     if constexpr (EPI == kEpiRope) {
       const int head = n0 / tail.hd, blk = (n0 % tail.hd) / 16;
       const bool is_q = head < tail.nh, is_k = !is_q && head < tail.nh + tail.nkv;
@@ -416,8 +441,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
       for (int t = threadIdx.x; t < 16; t += blockDim.x) {  // rows that do not exist leave a zero
         const int m = t;
         float sq = 0.f;
-        for (int row = 0; row < ROWS && n0 + row < N && m < M; ++row)
-          sq += sq_el[4 * (t % 16 + 16 * (row / 4)) + row % 4];
+        for (int row = 0; row < ROWS && n0 + row < N && m < M; ++row) {
+          const int in_tile = PAIRED ? row % 8 : row;
+          sq += sq_el[(PAIRED ? 256 * (row / 8) : 0) + 4 * (t % 16 + 16 * (in_tile / 4)) + in_tile % 4];
+        }
         res.ssq_part[static_cast<size_t>(blockIdx.x) * 16 + m] = sq;
       }
     }
@@ -453,7 +480,7 @@ template <typename T, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED =
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                           int slices, hipStream_t stream, const RopeTail& tail = RopeTail{},
                           const NormHead& head = NormHead{}, const ResidualTail& res = ResidualTail{}) {
-  const int MB = (M + 15) / 16;
+  const int MB = PAIRED ? ROWS / 8 : (M + 15) / 16;  // tiles a wave keeps
   const int waves = skinny_waves(N, K, MB, slices, ROWS, PAIRED ? 128 : 64);
   const dim3 grid((N + ROWS - 1) / ROWS, slices), block(waves * kWave);
   const size_t lds = (static_cast<size_t>(waves) * MB * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
@@ -461,7 +488,9 @@ static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, 
 #define LYP_SKINNY(MBV)                                                                                      \
   gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, \
                                                                                       ldc, tail, head, res)
-  if constexpr (NORMED || PAIRED) {
+  if constexpr (PAIRED && ROWS == 16) {
+    LYP_SKINNY(2);
+  } else if constexpr (NORMED || PAIRED) {
     LYP_SKINNY(1);  // at most 16 rows: the callers have checked
   } else {
     if (MB == 1) LYP_SKINNY(1);
@@ -610,11 +639,19 @@ extern "C" int lyp_gemm_rope_kv(const void* A, const void* W, void* out, int dty
 // With next_w (the weights of the RMS norm that follows) it also
 // stores xs[M, N] = h * next_w in the operands' type and, per workgroup, every
 // row's sum of squares over the workgroup's features: ssq_part[parts][16], with
-// `parts` = lyp_gemm_residual_parts(N) workgroups.  A product normed that way
+// `parts` = lyp_gemm_residual_parts(M, N, K) workgroups.  A product normed that way
 // (lyp_gemm_swiglu_normed, lyp_gemm_rope_kv_normed) takes xs and ssq_part in
 // place of the normed activations.  Returns 1 (and does nothing) when the
 // few-rows kernel does not apply.
-extern "C" int lyp_gemm_residual_parts(int N) { return (N + 7) / 8; }
+// Weight rows per workgroup: 8, so that a matrix of 2,048 rows gives every compute unit a
+// workgroup; 16 (as two paired tiles, the activations loaded once for both) from 3,072 rows on,
+// where that was measured ahead.
+static int residual_rows(int M, int N, int K) { return M <= 8 && K % 128 == 0 && N >= 3072 ? 16 : 8; }
+
+extern "C" int lyp_gemm_residual_parts(int M, int N, int K) {
+  const int rows = residual_rows(M, N, K);
+  return (N + rows - 1) / rows;
+}
 
 extern "C" int lyp_gemm_residual(const void* A, const void* W, float* h, int dtype, int M, int N, int K, int lda,
                                  int ldw, int ldh, const void* next_w, int next_w_dtype, void* xs, int ldx,
@@ -624,15 +661,18 @@ extern "C" int lyp_gemm_residual(const void* A, const void* W, float* h, int dty
   if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
   const ResidualTail res{next_w, next_w_dtype == kF32, xs, ldx, ssq_part};
   const bool paired = M <= 8 && K % 128 == 0;  // two chunks of K per matrix instruction
-#define LYP_RESIDUAL(T, PAIRED)                                                                              \
-  launch_skinny<T, kEpiResidual, false, 8, PAIRED>(static_cast<const T*>(A), static_cast<const T*>(W), h, M, N, K, \
-                                                   lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res)
+  const bool wide = residual_rows(M, N, K) == 16;
+#define LYP_RESIDUAL(T, ROWS, PAIRED)                                                                           \
+  launch_skinny<T, kEpiResidual, false, ROWS, PAIRED>(static_cast<const T*>(A), static_cast<const T*>(W), h, M, N, \
+                                                      K, lda, ldw, ldh, 1, stream, RopeTail{}, NormHead{}, res)
   if (dtype == kF32) {
-    if (paired) LYP_RESIDUAL(float, true);
-    else LYP_RESIDUAL(float, false);
+    if (wide) LYP_RESIDUAL(float, 16, true);
+    else if (paired) LYP_RESIDUAL(float, 8, true);
+    else LYP_RESIDUAL(float, 8, false);
   } else if (dtype == kBF16) {
-    if (paired) LYP_RESIDUAL(bf16_t, true);
-    else LYP_RESIDUAL(bf16_t, false);
+    if (wide) LYP_RESIDUAL(bf16_t, 16, true);
+    else if (paired) LYP_RESIDUAL(bf16_t, 8, true);
+    else LYP_RESIDUAL(bf16_t, 8, false);
   } else
     LYP_REQUIRE(false, "gemm_residual: unknown dtype %d", dtype);
 #undef LYP_RESIDUAL

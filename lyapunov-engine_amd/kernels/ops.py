@@ -59,7 +59,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_gemm_rope_kv.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_void_p]
-        lib.lyp_gemm_residual_parts.argtypes = [c_int]
+        lib.lyp_gemm_residual_parts.argtypes = [c_int, c_int, c_int]
         lib.lyp_gemm_residual.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                           c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p]
         lib.lyp_gemm_swiglu_normed.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p, c_void_p,
@@ -232,7 +232,7 @@ def linear_residual(h: torch.Tensor, p: PendingLinear, next_weight: torch.Tensor
         if M > PENDING_MAX_ROWS or next_weight.numel() != N:
             return False
         xs = torch.empty((M, N), dtype=x.dtype, device=h.device)
-        ssq = torch.empty((lib.lyp_gemm_residual_parts(N), 16), dtype=torch.float32, device=h.device)
+        ssq = torch.empty((lib.lyp_gemm_residual_parts(M, N, K), 16), dtype=torch.float32, device=h.device)
     rc = lib.lyp_gemm_residual(_p(x), _p(w), _p(h), _code(x.dtype), M, N, K, x.stride(0), w.stride(0), h.stride(0),
                                _p(next_weight), _code(next_weight.dtype) if next_weight is not None else 0, _p(xs), N,
                                _p(ssq), _stream())

@@ -135,7 +135,8 @@ def test_linear_partial_sums(ops, dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (8, 100, 192), (5, 515, 1024)])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (8, 100, 192), (5, 515, 1024), (8, 4096, 1024),
+                                   (3, 4101, 384), (7, 3072, 256)])
 def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N, K):
     """A projection of few rows handed on instead of run (pending=True) and
     then added to the float residual stream by the product kernel itself."""
@@ -158,7 +159,7 @@ def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,K,J", [(1, 2048, 192), (8, 192, 192), (5, 1024, 256), (7, 256, 384), (8, 320, 128)])
+@pytest.mark.parametrize("M,K,J", [(1, 2048, 192), (8, 192, 192), (5, 1024, 256), (7, 256, 384), (8, 320, 128), (6, 4096, 256)])
 def test_norm_folded_into_the_products_around_it(ops, dtype, M, K, J):
     """The product that adds to the residual stream prepares the RMS norm that
     follows (rmsnorm_pending), and the gate/up and the q/k/v products finish
