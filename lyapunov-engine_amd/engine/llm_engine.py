@@ -25,7 +25,8 @@ are taken, otherwise (a request ended on an end-of-sequence token, was aborted,
 was added) they are dropped and the plan runs.  A dropped step has only written
 keys and values of its own requests at positions that the plan writes again or
 whose pages were given back; later work on the stream overwrites what it
-reuses before reading it.
+reuses before reading it.  A model with per-request state of its own (which a
+step changes in place) does not look ahead.
 """
 from __future__ import annotations
 
@@ -103,6 +104,9 @@ class LLMEngine:
         if config.enable_graphs:
             from .graphs import DecodeGraphs
             self.graphs = DecodeGraphs(self.core.runner, max_batch=config.max_num_seqs)
+        # A step that is dropped is run again: harmless for keys and values (the same values to the
+        # same slots), not for a mixer's own state, which the step changes in place.
+        self._look_ahead = bool(config.lookahead) and not self.core.pools.state
         self._ahead: Optional[_Ahead] = None
         self.steps_taken_ahead = 0    # steps whose results came from a step started ahead
 
@@ -182,7 +186,7 @@ class LLMEngine:
             if wanting:
                 pending = self.sampler.launch(logits, [r.params for r in wanting], [r.stream for r in wanting],
                                               [len(r.outputs) for r in wanting])
-        if decoding and self.config.lookahead:
+        if decoding and self._look_ahead:
             self._ahead = self._start_ahead(ids, start, reqs, pending)
         sampled = pending.result() if pending is not None else []
         status = self.scheduler.post_step_status(sampled)

@@ -286,6 +286,22 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
             cut.step([("x", 1), ("z", 1)])
         cut.step([("x", 42), ("z", 2)], end=["x", "z"])
         compare(cut, replay(folder, dtype, cut), want, dtype, "toy cut")
+
+        # through the generating engine: greedy tokens are the plain model's; with a state that a step
+        # changes in place no step is started ahead (one that had to be dropped could not be run again)
+        import lyapunov_engine_amd as L
+        llm = L.LLM(folder, dtype=dtype, num_blocks=64, block_size=4, max_num_seqs=4)
+        assert llm.engine._look_ahead is False
+        prompt = reqs["y"][:9]
+        got = llm.generate([prompt], L.SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))[0].output_tokens
+        toks = list(prompt)
+        for i in range(6):
+            logits = toy_plain(folder, toks)[-1]
+            top = torch.topk(logits, 2).values
+            if got[i] != int(logits.argmax()):
+                assert dtype == "bfloat16" and float(top[0] - top[1]) < 0.25, (i, got)
+                break
+            toks.append(got[i])
     finally:
         ARCHITECTURES.unregister("ToyMixForCausalLM")
         MIXERS.unregister("toy_linear_recurrence")
