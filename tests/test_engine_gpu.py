@@ -127,6 +127,39 @@ def test_steps_started_ahead_give_the_same_tokens(model_folders, dtype):
     assert taken_ahead > 20, "most decode steps were meant to be started ahead"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_across_the_graphs_context_buckets(model_folders, dtype):
+    """Three requests decode from under 256 tokens to over 256 (a new graph is captured while a step
+    started ahead is still running) and one of them on to 500: the tokens are those of the engine
+    without graphs, and in 32-bit those of the plain model at the places checked."""
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    folder = model_folders["B"][dtype]
+    prompts = [random_tokens(n, 515, seed=30 + n) for n in (200, 90, 250)]
+    lengths = [290, 200, 40]
+
+    def run(graphs):
+        engine = LLMEngine(folder, EngineConfig(dtype=dtype, num_blocks=80, block_size=16, max_num_seqs=4,
+                                                enable_graphs=graphs))
+        for i, p in enumerate(prompts):
+            engine.add_request(i, p, SamplingParams(temperature=0.0, max_tokens=lengths[i], ignore_eos=True))
+        done = {}
+        while engine.has_unfinished_requests():
+            for out in engine.step():
+                if out.finished:
+                    done[out.request_id] = list(out.output_tokens)
+        return done, engine
+
+    with_graphs, engine = run(True)
+    assert len({key[1] for key in engine.graphs.captured}) >= 2 and engine.steps_taken_ahead > 200
+    eager, _ = run(False)
+    assert with_graphs == eager
+    if dtype == "float32":
+        check_against_plain(folder, prompts[2], with_graphs[2], dtype)
+
+
 def test_graph_steps_equal_eager_steps(model_folders):
     """The same decode steps through a captured graph, replayed several times
     with other work in between, and eagerly: equal logits every time."""
