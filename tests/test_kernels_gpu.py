@@ -400,6 +400,11 @@ PREFILL_CASES = [
     (16, 8, 32, 16, 300, [(1500, 1500), (900, 500), (65, 65), (64, 64)]),
     (8, 8, 128, 16, 0, [(2100, 2100)]),
     (2, 1, 256, 16, 0, [(100, 100), (40, 3)]),
+    # larger pages: 32, 64 and 128 slots
+    (8, 2, 64, 32, 0, [(700, 300), (33, 33)]),
+    (4, 1, 128, 64, 0, [(500, 500), (70, 3)]),
+    (8, 4, 64, 128, 200, [(900, 400)]),
+    (4, 2, 32, 64, 0, [(300, 300)]),
     # three, five, six and seven query heads to a key/value head
     (24, 8, 128, 16, 0, [(300, 300), (77, 5)]),
     (5, 1, 64, 16, 0, [(200, 130)]),
@@ -454,6 +459,9 @@ DECODE_CASES = [
     (4, 2, 32, 4, 9, [50, 5, 9, 10]),
     (2, 1, 64, 16, 100, [700, 64]),
     (16, 1, 16, 2, 0, [23]),
+    (8, 2, 64, 32, 0, [700, 33]),     # larger pages
+    (4, 1, 128, 64, 0, [500, 1]),
+    (8, 4, 64, 128, 200, [900, 129]),
 ]
 
 
