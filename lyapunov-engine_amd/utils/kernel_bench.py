@@ -4,6 +4,7 @@
     python -m lyapunov_engine_amd.utils.kernel_bench attn_decode --batch 8 --context 8192
     python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 8 --out-features 16384 --in-features 2048
     python -m lyapunov_engine_amd.utils.kernel_bench residual --rows 8 --out-features 2048 --in-features 8192
+    python -m lyapunov_engine_amd.utils.kernel_bench sample --rows 8 --vocab 128256 --top-k 50 --top-p 0.9
 
 Prints the time per call and what it means in TFLOP/s or TB/s.  Small enough to
 run under ``rocprofv3 --pmc ...`` when a kernel's counters are wanted; the
@@ -123,9 +124,24 @@ def residual(a) -> None:
           f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
 
 
+def sample(a) -> None:
+    """The sampler's two kernels on ``rows`` rows of random logits (temperature 0: greedy)."""
+    dev = a.device
+    logits = torch.randn(a.rows, a.vocab, device=dev) * 2
+    temperature = torch.full((a.rows,), a.temperature, device=dev)
+    top_k = torch.full((a.rows,), a.top_k, dtype=torch.int32, device=dev)
+    top_p = torch.full((a.rows,), a.top_p, device=dev)
+    u = torch.full((a.rows,), 0.5, device=dev)
+    out = torch.empty(a.rows, dtype=torch.int32, device=dev)
+    work = ops.sample_workspace(a.rows, dev)
+    t = _time(lambda: ops.sample(logits, temperature, top_k, top_p, u, out, work), a.repeat)
+    print(f"sample rows={a.rows} vocab={a.vocab} temperature={a.temperature} top_k={a.top_k} top_p={a.top_p}: "
+          f"{t * 1e6:.1f} us")
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
-    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual"])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--repeat", type=int, default=20)
@@ -139,12 +155,17 @@ def main(argv=None) -> None:
     ap.add_argument("--batch", type=int, default=8, help="attn_decode: requests")
     ap.add_argument("--rows", type=int, default=8, help="linear: rows of activations")
     ap.add_argument("--in-features", type=int, default=2048)
+    ap.add_argument("--vocab", type=int, default=128256, help="sample: width of a row of logits")
+    ap.add_argument("--temperature", type=float, default=0.8)
+    ap.add_argument("--top-k", type=int, default=-1)
+    ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--out-features", type=int, default=16384)
     ap.add_argument("--may-split", action="store_true", help="linear: allow partial sums over slices of K")
     a = ap.parse_args(argv)
     ops.require_gpu()
     torch.manual_seed(0)
-    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual}[a.kernel](a)
+    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual,
+     "sample": sample}[a.kernel](a)
 
 
 if __name__ == "__main__":
