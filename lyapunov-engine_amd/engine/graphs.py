@@ -3,8 +3,10 @@
 A step in which every request brings exactly one token launches some hundred
 small kernels; launched one by one from Python, the launches cost more than the
 kernels.  Such steps are captured once per (batch bucket, context bucket) and
-replayed: the step's tables are copied into fixed device buffers, the graph
-runs, the logits are read from a fixed tensor.
+replayed: a small kernel reads the step's tables from pinned host memory into
+fixed device buffers (the token ids from the sampler's device buffer when the
+host does not know them yet), the graph runs, the logits are read from a fixed
+tensor.
 
 The reference buckets by batch size {1, 2, 4, ... 64}, takes the smallest bucket
 that fits, pads with zeros and slices the result

@@ -2,8 +2,9 @@
 
 What is computed is the reference's sample_next_tokens
 (python/lyapunov_engine/engine/sampling.py:15-72); it runs there row by row with
-a host round trip per row (``.item()``), here as one kernel launch for the
-batch and one copy of the chosen tokens back.
+a host round trip per row (``.item()``), here as one launch for the batch
+whose kernel writes the chosen tokens to the device (for a step that is started
+before the host has them) and to pinned host memory (read behind an event).
 
 The uniform number behind a draw comes from (engine seed, request seed, index of
 the output token) through a counter-based generator, so it is the same whatever
