@@ -116,6 +116,17 @@ class CacheManager:
         self._rc(self._lib.lyp_cache_export(self._h, seq_ids.ctypes.data, len(seq_ids), group, tables.ctypes.data,
                                             tables.shape[1], slots.ctypes.data if slots is not None else None))
 
+    def step_tables(self, seq_ids, start, count, group: int, tables, slot_map, slots=None) -> None:
+        """The tables of one step, checked and written into int32 numpy arrays.
+        Request ``seq_ids[b]`` (int64) continues at ``start[b]`` with
+        ``count[b]`` new tokens (int32): it must hold exactly ``start[b]``
+        tokens and have pages for the new ones.  Row b of ``tables`` gets its
+        block table (-1 past its end), ``slot_map`` the page slot of every new
+        token in order, ``slots`` the state slots."""
+        self._rc(self._lib.lyp_cache_step_tables(self._h, seq_ids.ctypes.data, start.ctypes.data, count.ctypes.data,
+                                                 len(seq_ids), group, tables.ctypes.data, tables.shape[1],
+                                                 slot_map.ctypes.data, slots.ctypes.data if slots is not None else None))
+
     def reserve(self, seq_ids, new_lens) -> bool:
         """Pages for positions < new_lens[b] of every request seq_ids[b] (numpy
         int64 / int32 arrays), all or none: False, and nothing taken, if a

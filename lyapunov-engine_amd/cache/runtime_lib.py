@@ -38,6 +38,8 @@ def lib() -> ctypes.CDLL:
     L.lyp_cache_table.argtypes = [c_void_p, c_int64, c_int, i32p, c_int]
     L.lyp_cache_export.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p]
     L.lyp_cache_reserve.argtypes = [c_void_p, c_void_p, c_void_p, c_int]
+    L.lyp_cache_step_tables.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p,
+                                        c_void_p]
     L.lyp_cache_ref_count.argtypes = [c_void_p, c_int, c_int]
     L.lyp_cache_check.argtypes = [c_void_p]
     L.lyp_cache_counters.argtypes = [c_void_p, i64p]

@@ -121,6 +121,50 @@ int lyp_cache_export(void* h, const int64_t* ids, int n, int g, int32_t* tables,
     return 0;
   });
 }
+// The tables of one step.  Request ids[b] continues at position start[b] with
+// count[b] new tokens: it must be known, hold exactly start[b] tokens and have
+// pages for start[b] + count[b].  Row b of `tables` (`width` entries a row, at
+// least as many as the longest request needs after the step) gets the block
+// table in group g, -1 past its end; slot_map, for each new token in order, the
+// page slot (page * page size + offset) its key and value go to; `slots`, if
+// given, the state slots.
+int lyp_cache_step_tables(void* h, const int64_t* ids, const int32_t* start, const int32_t* count, int n, int g,
+                          int32_t* tables, int width, int32_t* slot_map, int32_t* slots) {
+  return guarded([&] {
+    auto* m = static_cast<CacheManager*>(h);
+    const int ps = m->group(g).page_size;
+    size_t at = 0;
+    for (int b = 0; b < n; ++b) {
+      const std::string who = "request " + std::to_string(ids[b]);
+      if (!m->has(ids[b])) throw std::runtime_error(who + " is not known to the cache manager");
+      if (count[b] < 1) throw std::runtime_error(who + " brings no tokens");
+      if (start[b] != m->length(ids[b]))
+        throw std::runtime_error(who + " continues at " + std::to_string(start[b]) + " but its cache holds " +
+                                 std::to_string(m->length(ids[b])) + " tokens");
+      const int end = start[b] + count[b];
+      if (end > m->capacity(ids[b]))
+        throw std::runtime_error(who + " has pages for " + std::to_string(m->capacity(ids[b])) +
+                                 " tokens, the step needs " + std::to_string(end));
+      const auto& t = m->table(ids[b], g);
+      const int need = (end + ps - 1) / ps;
+      if (need > width || need > static_cast<int>(t.size()))
+        throw std::runtime_error(who + ": a block table row of " + std::to_string(width) + " entries for " +
+                                 std::to_string(need) + " pages");
+      int32_t* row = tables + static_cast<size_t>(b) * width;
+      const int have = std::min(width, static_cast<int>(t.size()));
+      std::memcpy(row, t.data(), sizeof(int32_t) * static_cast<size_t>(have));
+      for (int i = have; i < width; ++i) row[i] = -1;
+      for (int pos = start[b]; pos < end; ++pos) {
+        const int32_t page = row[pos / ps];
+        if (page < 0)
+          throw std::runtime_error(who + " has no page for one of its new tokens in cache group " + std::to_string(g));
+        slot_map[at++] = page * ps + pos % ps;
+      }
+      if (slots) slots[b] = m->state_slot(ids[b]);
+    }
+    return 0;
+  });
+}
 // Pages for positions < new_lens[b] of every request ids[b], all or none: 1 if they are held now,
 // 0 (and nothing taken) if some group lacks the pages.  For a caller that prepares the step after
 // the one the scheduler planned.

@@ -39,7 +39,6 @@ from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .core import EngineCore
-from .runner import StepEntry
 from .scheduler import FINISH_REASON, STATUS, Scheduler
 
 
@@ -174,13 +173,8 @@ class LLMEngine:
             if decoding:
                 logits = self.graphs.step_arrays(ids, start, tokens)
             else:
-                entries, at = [], 0
-                for i in range(n):
-                    c = int(count[i])
-                    entries.append(StepEntry(int(ids[i]), tokens[at:at + c].tolist(), int(start[i]),
-                                             [c - 1] if wants[i] else []))
-                    at += c
-                logits = self.core.step(entries)
+                rows = (np.cumsum(count, dtype=np.int32) - 1)[wants != 0]   # the last token of each request that wants
+                logits = self.core.runner.step_arrays(ids, start, count, tokens, rows)
             wanting = [r for r, w in zip(reqs, wants) if w]
             pending = None
             if wanting:

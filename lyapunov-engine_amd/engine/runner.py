@@ -20,7 +20,7 @@ from typing import Optional
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, CachePools
+from ..cache.manager import CacheError, CacheManager, CachePools
 from ..kernels import ops
 from ..models.decoder import DecoderModel
 from ..parts.base import GroupView, LayerCache, StepContext
@@ -66,71 +66,82 @@ class ModelRunner:
     def build_context(self, entries: list) -> StepContext:
         if not entries:
             raise StepError("a step needs at least one entry")
-        B = len(entries)
-        seen = set()
-        q_start = [0]
         for e in entries:
-            n = len(e.tokens)
-            if n == 0:
+            if len(e.tokens) == 0:
                 raise StepError(f"request {e.seq_id} brings no tokens")
-            if e.seq_id in seen:
-                raise StepError(f"request {e.seq_id} appears twice in one step")
-            seen.add(e.seq_id)
-            if not self.cache.has(e.seq_id):
-                raise StepError(f"request {e.seq_id} is not known to the cache manager")
-            if e.start != self.cache.length(e.seq_id):
-                raise StepError(f"request {e.seq_id} continues at {e.start} but its cache holds "
-                                f"{self.cache.length(e.seq_id)} tokens")
-            if e.start + n > self.cache.capacity(e.seq_id):
-                raise StepError(f"request {e.seq_id} has pages for {self.cache.capacity(e.seq_id)} tokens, "
-                                f"the step needs {e.start + n}")
-            if e.start + n > self.max_position:
-                raise StepError(f"request {e.seq_id} would reach position {e.start + n - 1}, beyond the model's "
-                                f"{self.max_position}")
-            if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size:
-                raise StepError(f"request {e.seq_id} has a token outside the vocabulary of {self.vocab_size}")
-            if any(w < 0 or w >= n for w in e.want):
+            if any(w < 0 or w >= len(e.tokens) for w in e.want):
                 raise StepError(f"request {e.seq_id} wants logits at a place it does not bring")
-            q_start.append(q_start[-1] + n)
-        T = q_start[-1]
+        ids = np.asarray([e.seq_id for e in entries], dtype=np.int64)
+        start = np.asarray([e.start for e in entries], dtype=np.int32)
+        count = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+        at, rows = 0, []
+        for e in entries:
+            rows += [at + w for w in e.want]
+            at += len(e.tokens)
+        return self.build_context_arrays(ids, start, count, tokens, np.asarray(rows, dtype=np.int32))
 
-        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-        positions = np.concatenate([np.arange(e.start, e.start + len(e.tokens), dtype=np.int32) for e in entries])
-        ctx_len = np.asarray([e.start + len(e.tokens) for e in entries], dtype=np.int32)
-        slots = np.asarray([self.cache.state_slot(e.seq_id) for e in entries], dtype=np.int32)
-        rows = np.asarray([q_start[b] + w for b, e in enumerate(entries) for w in e.want], dtype=np.int32)
+    def build_context_arrays(self, ids, start, count, tokens, rows) -> StepContext:
+        """The same from numpy arrays: request ids (int64); the position of each
+        request's first new token and the number of its new tokens (int32); all
+        new tokens in the order of the requests (int32); the rows (indices into
+        ``tokens``) whose logits are wanted (int32)."""
+        B = len(ids)
+        if B == 0:
+            raise StepError("a step needs at least one entry")
+        if len(np.unique(ids)) != B:
+            raise StepError(f"a request appears twice in one step: {ids.tolist()}")
+        if int(count.min()) < 1:
+            raise StepError(f"request {int(ids[int(count.argmin())])} brings no tokens")
+        q_start = np.zeros(B + 1, dtype=np.int32)
+        np.cumsum(count, out=q_start[1:])
+        T = int(q_start[-1])
+        ctx_len = start + count
+        if tokens.size != T:
+            raise StepError(f"{tokens.size} tokens for requests that bring {T}")
+        if int(ctx_len.max()) > self.max_position:
+            b = int(ctx_len.argmax())
+            raise StepError(f"request {int(ids[b])} would reach position {int(ctx_len[b]) - 1}, beyond the model's "
+                            f"{self.max_position}")
+        if int(tokens.min()) < 0 or int(tokens.max()) >= self.vocab_size:
+            bad = int(np.flatnonzero((tokens < 0) | (tokens >= self.vocab_size))[0])
+            b = int(np.searchsorted(q_start, bad, side="right")) - 1
+            raise StepError(f"request {int(ids[b])} has a token outside the vocabulary of {self.vocab_size}")
+        if rows.size and (int(rows.min()) < 0 or int(rows.max()) >= T):
+            raise StepError("logits are wanted at a place the step does not bring")
+        positions = np.arange(T, dtype=np.int32) + np.repeat(start - q_start[:-1], count)
+        slots = np.empty(B, dtype=np.int32)
 
-        tiles, dec = [], []   # tiles: (keys up to the tile's last token, request, first token)
-        for b, e in enumerate(entries):
-            n = len(e.tokens)
-            if n == 1:
-                dec.append(b)
-            else:
-                for q0 in range(0, n, PREFILL_TILE):
-                    tiles.append((e.start + min(n, q0 + PREFILL_TILE), b, q0))
-        tiles.sort()          # the attention kernel starts (or pairs) tiles by the work they are
-        tile_seq = [t[1] for t in tiles]
-        tile_q0 = [t[2] for t in tiles]
-        tile_keys = (tiles[0][0], tiles[-1][0]) if tiles else (0, 0)
-        max_ctx_dec = max((int(ctx_len[b]) for b in dec), default=0)
+        # Attention work: tiles of PREFILL_TILE new tokens of requests that bring several, sorted by
+        # (keys up to the tile's last token, request, first token): the attention kernel starts (or
+        # pairs) tiles by the work they are; and the requests with one new token.
+        several = np.flatnonzero(count > 1)
+        dec = np.flatnonzero(count == 1).astype(np.int32)
+        if several.size:
+            per = (count[several] + PREFILL_TILE - 1) // PREFILL_TILE
+            tile_b = np.repeat(several, per).astype(np.int32)
+            first = np.cumsum(per) - per
+            tile_q0 = ((np.arange(int(per.sum())) - np.repeat(first, per)) * PREFILL_TILE).astype(np.int32)
+            keys = start[tile_b] + np.minimum(count[tile_b], tile_q0 + PREFILL_TILE)
+            order = np.lexsort((tile_q0, tile_b, keys))
+            tile_seq, tile_q0, keys = tile_b[order], tile_q0[order], keys[order]
+            tile_keys = (int(keys[0]), int(keys[-1]))
+        else:
+            tile_seq = tile_q0 = np.zeros(0, dtype=np.int32)
+            tile_keys = (0, 0)
+        max_ctx_dec = int(ctx_len[dec].max()) if dec.size else 0
 
-        sections = [token_ids, positions, np.asarray(q_start, dtype=np.int32), ctx_len, slots, rows,
-                    np.asarray(tile_seq, dtype=np.int32), np.asarray(tile_q0, dtype=np.int32),
-                    np.asarray(dec, dtype=np.int32)]
+        sections = [tokens, positions, q_start, ctx_len, slots, rows, tile_seq, tile_q0, dec]
         group_meta = []
         for g, gc in enumerate(self.cache.groups):
-            tables = [self.cache.table(e.seq_id, g) for e in entries]
-            width = max(1, max(len(t) for t in tables))
-            bt = np.full((B, width), -1, dtype=np.int32)
-            slot_map = np.empty(T, dtype=np.int32)
             ps = gc.page_size
-            for b, (e, t) in enumerate(zip(entries, tables)):
-                bt[b, :len(t)] = t
-                pos = positions[q_start[b]:q_start[b + 1]]
-                pages = np.asarray(t, dtype=np.int32)[pos // ps]
-                if (pages < 0).any():
-                    raise StepError(f"request {e.seq_id} has no page for one of its new tokens in cache group {g}")
-                slot_map[q_start[b]:q_start[b + 1]] = pages * ps + pos % ps
+            width = max(1, -(-int(ctx_len.max()) // ps))
+            bt = np.empty((B, width), dtype=np.int32)
+            slot_map = np.empty(T, dtype=np.int32)
+            try:
+                self.cache.step_tables(ids, start, count, g, bt, slot_map, slots if g == 0 else None)
+            except CacheError as err:
+                raise StepError(str(err)) from None
             sections += [slot_map, bt.reshape(-1)]
             group_meta.append((ps, width, gc.window))
 
@@ -153,9 +164,9 @@ class ModelRunner:
         return StepContext(
             device=self.device, dtype=self.dtype, T=T, B=B, token_ids=view(0), positions=view(1), q_start=view(2),
             ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=int(rows.size), groups=groups,
-            tile_seq=view(6), tile_q0=view(7), n_tiles=len(tile_seq), tile_keys=tile_keys,
-            dec_seqs=view(8) if dec else None,
-            n_dec=len(dec), max_ctx_dec=max_ctx_dec, q_start_host=q_start, ctx_len_host=ctx_len.tolist(),
+            tile_seq=view(6), tile_q0=view(7), n_tiles=int(tile_seq.size), tile_keys=tile_keys,
+            dec_seqs=view(8) if dec.size else None,
+            n_dec=int(dec.size), max_ctx_dec=max_ctx_dec, q_start_host=q_start.tolist(), ctx_len_host=ctx_len.tolist(),
             state_slots_host=slots.tolist(), workspace=self.workspace)
 
     def layer_caches(self, ctx: StepContext) -> list:
@@ -168,4 +179,9 @@ class ModelRunner:
         ``want`` lists, or None when nothing is wanted.  The cache is written
         for every token of the step either way."""
         ctx = self.build_context(entries)
+        return self.model.forward(ctx, self.layer_caches(ctx))
+
+    def step_arrays(self, ids, start, count, tokens, rows) -> Optional[torch.Tensor]:
+        """``step`` from numpy arrays (see ``build_context_arrays``)."""
+        ctx = self.build_context_arrays(ids, start, count, tokens, rows)
         return self.model.forward(ctx, self.layer_caches(ctx))

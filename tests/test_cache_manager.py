@@ -183,3 +183,40 @@ def test_random_orders_keep_every_invariant(seed):
     assert c["pages_taken"] == c["pages_returned"] and c["high_water"] > 0
     m.reset()
     assert m.num_free_slots() == slots
+
+
+def test_tables_of_a_step_are_checked_and_filled():
+    import numpy as np
+
+    m = CacheManager([GroupConfig(8, 4), GroupConfig(8, 4, window=4)], 4)
+    m.add(7), m.add(9)
+    m.extend(7, 12)                      # pages 0, 1, 2
+    m.commit(7, 8)                       # the window group has given its first page back
+    m.extend(9, 3)                       # page 3
+    ids = np.array([7, 9], dtype=np.int64)
+    start, count = np.array([8, 0], dtype=np.int32), np.array([3, 2], dtype=np.int32)
+
+    def tables(g, width=4, ids=ids, start=start, count=count):
+        bt = np.full((len(ids), width), 99, dtype=np.int32)
+        slot_map, slots = np.full(int(count.sum()), 99, dtype=np.int32), np.full(len(ids), 99, dtype=np.int32)
+        m.step_tables(ids, start, count, g, bt, slot_map, slots)
+        return bt.tolist(), slot_map.tolist(), slots.tolist()
+
+    bt, slot_map, slots = tables(0)
+    assert bt == [[0, 1, 2, -1], [3, -1, -1, -1]]                 # -1 past a table's end
+    assert slot_map == [2 * 4 + 0, 2 * 4 + 1, 2 * 4 + 2, 3 * 4 + 0, 3 * 4 + 1]
+    assert slots == [m.state_slot(7), m.state_slot(9)]
+    bt, slot_map, _ = tables(1, width=3)
+    assert bt == [[-1, 1, 2], [3, -1, -1]] and slot_map[:3] == [8, 9, 10]   # a page the window has passed stays -1
+
+    one = lambda v, t: np.array([v], dtype=t)
+    for kw, words in [
+        (dict(ids=one(5, np.int64), start=one(0, np.int32), count=one(1, np.int32)), "request 5 is not known"),
+        (dict(ids=one(7, np.int64), start=one(5, np.int32), count=one(1, np.int32)), "continues at 5 but its cache holds 8"),
+        (dict(ids=one(7, np.int64), start=one(8, np.int32), count=one(5, np.int32)), "has pages for 12 tokens, the step needs 13"),
+        (dict(ids=one(7, np.int64), start=one(8, np.int32), count=one(0, np.int32)), "brings no tokens"),
+        (dict(width=2), "row of 2 entries for 3 pages"),
+    ]:
+        with pytest.raises(CacheError, match=words):
+            tables(0, **kw)
+    m.check()

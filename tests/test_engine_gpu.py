@@ -160,6 +160,36 @@ def test_decoding_across_the_graphs_context_buckets(model_folders, dtype):
         check_against_plain(folder, prompts[2], with_graphs[2], dtype)
 
 
+def test_a_step_that_does_not_fit_the_cache_is_refused(model_folders):
+    """What the step function will not run, with the reason: a request the
+    cache does not know, a gap or an overlap in its positions, tokens without
+    pages, a token outside the vocabulary, a position beyond the model's,
+    logits at a place the step does not bring, a request twice."""
+    from lyapunov_engine_amd.engine.core import EngineCore, StepEntry
+    from lyapunov_engine_amd.engine.runner import StepError
+
+    core = EngineCore.from_folder(model_folders["A"]["float32"], dtype="float32", num_blocks=80, block_size=4)
+    core.cache.add(0)
+    core.cache.extend(0, 8)
+    for entries, words in [
+        ([], "at least one entry"),
+        ([StepEntry(3, [1, 2], 0, [])], "request 3 is not known"),
+        ([StepEntry(0, [], 0, [])], "brings no tokens"),
+        ([StepEntry(0, [1, 2], 1, [])], "continues at 1 but its cache holds 0"),
+        ([StepEntry(0, list(range(9)), 0, [])], "has pages for 8 tokens, the step needs 9"),
+        ([StepEntry(0, [1, 256], 0, [])], "outside the vocabulary of 256"),
+        ([StepEntry(0, [1, 2], 0, [2])], "wants logits at a place it does not bring"),
+        ([StepEntry(0, [1], 0, []), StepEntry(0, [2], 1, [])], "twice"),
+    ]:
+        with pytest.raises(StepError, match=words):
+            core.step(entries)
+    core.cache.extend(0, 300)
+    with pytest.raises(StepError, match="beyond the model's 256"):
+        core.step([StepEntry(0, [1] * 257, 0, [])])
+    logits = core.step([StepEntry(0, [1, 2, 3], 0, [2])])       # and what fits still runs
+    assert tuple(logits.shape) == (1, 256) and bool(torch.isfinite(logits).all())
+
+
 def test_graph_steps_equal_eager_steps(model_folders):
     """The same decode steps through a captured graph, replayed several times
     with other work in between, and eagerly: equal logits every time."""
