@@ -2,8 +2,8 @@
 
 There is one library of kernels whose sizes are run-time values (``core``), one
 attention library per head size (``attn_hd<N>``; the head size is a compile-time
-constant there), and one library of host code (``runtime``: cache manager and
-scheduler).  A library's file name carries a hash of its sources and flags, so a
+constant there), one of host code around the vendor's GEMM library (``blas``),
+and one library of host code (``runtime``: cache manager and scheduler).  A library's file name carries a hash of its sources and flags, so a
 changed source is never served by an old binary; what is missing is compiled on
 first use, with a progress line now and then.
 
@@ -38,6 +38,7 @@ CXX_FLAGS = ["-O2", "-std=c++20", "-fPIC", "-Wall", "-Wextra"]
 
 CORE_SOURCES = ["kernels/errors.hip", "kernels/elementwise.hip", "kernels/gemm.hip", "kernels/sampler.hip"]
 ATTN_SOURCES = ["kernels/errors.hip", "kernels/attention.hip"]
+BLAS_SOURCES = ["kernels/errors.hip", "kernels/library_gemm.hip"]   # host code around the vendor's GEMM library
 RUNTIME_SOURCES = ["runtime/cache_manager.cpp", "runtime/scheduler.cpp", "runtime/c_api.cpp"]
 
 # Head sizes compiled ahead of time by build_all(); any other multiple of 16 up
@@ -132,7 +133,7 @@ def _run_with_progress(cmds: list[list[str]], what: str) -> None:
 
 
 def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str, str] | None = None,
-                  force: bool = False) -> Path:
+                  force: bool = False, link: list[str] | None = None) -> Path:
     """Return the path of the library, compiling it if it is not there."""
     defines = dict(defines or {})
     # For experiments: LYAPUNOV_AMD_EXTRA_DEFINES="NAME=VALUE,OTHER=1" adds macros to every HIP compile
@@ -145,7 +146,7 @@ def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str
     flags = (HIP_FLAGS if hip else CXX_FLAGS) + [f"-D{k}={v}" for k, v in sorted(defines.items())]
     include = ["-I", str(CSRC / "kernels"), "-I", str(CSRC / "runtime")]
     out_dir = library_dir()
-    target = out_dir / f"lib{name}-{_key(sources, flags)}.so"
+    target = out_dir / f"lib{name}-{_key(sources, flags + list(link or []))}.so"
     with _lock:
         if target.exists() and not force:
             return target
@@ -160,10 +161,10 @@ def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str
                 cmds.append([compiler, *flags, *include, "-c", str(CSRC / rel), "-o", str(obj)])
             _run_with_progress(cmds, name)
             tmp_so = work / "out.so"
-            link = [compiler, "-shared", "-fPIC", *objs, "-o", str(tmp_so)]
+            link_cmd = [compiler, "-shared", "-fPIC", *objs, "-o", str(tmp_so), *(link or [])]
             if hip:
-                link.insert(1, f"--offload-arch={GPU_ARCH}")
-            _run_with_progress([link], name + " (link)")
+                link_cmd.insert(1, f"--offload-arch={GPU_ARCH}")
+            _run_with_progress([link_cmd], name + " (link)")
             os.replace(tmp_so, target)
         finally:
             shutil.rmtree(work, ignore_errors=True)
@@ -188,13 +189,19 @@ def attention_library(head_dim: int, force: bool = False) -> Path:
                          defines={"LYP_HEAD_DIM": str(head_dim)}, force=force)
 
 
+def blas_library(force: bool = False) -> Path:
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    return build_library("lyp_blas", BLAS_SOURCES, hip=True, force=force,
+                         link=[f"-L{os.path.join(rocm, 'lib')}", "-lhipblaslt"])
+
+
 def runtime_library(force: bool = False) -> Path:
     return build_library("lyp_runtime", RUNTIME_SOURCES, hip=False, force=force)
 
 
 def build_all(force: bool = True) -> list[Path]:
     """Compile every library (what ``__graft_entry__.build`` calls)."""
-    out = [runtime_library(force), core_library(force)]
+    out = [runtime_library(force), core_library(force), blas_library(force)]
     for hd in PREBUILT_HEAD_DIMS:
         out.append(attention_library(hd, force))
     return out

@@ -456,7 +456,13 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 # the reference's projections go to cuBLAS (nn.Linear, models/llama.py:45-48,
 # 112-117, 177).  Products with few rows (decode steps), every float product
 # (true 32-bit) and everything when LYAPUNOV_AMD_GEMM=own use the kernels here.
-LIBRARY_GEMM = os.environ.get("LYAPUNOV_AMD_GEMM", "library") != "own"
+# LYAPUNOV_AMD_GEMM: "library" (the default: hipBLASLt called directly, with the plan of every shape
+# kept), "torch" (the same library behind torch.matmul: 18 us of host time a call instead of 4), "own".
+LIBRARY_GEMM_MODE = os.environ.get("LYAPUNOV_AMD_GEMM", "library")
+if LIBRARY_GEMM_MODE not in ("library", "torch", "own"):
+    raise KernelError(f"LYAPUNOV_AMD_GEMM is 'library', 'torch' or 'own', not {LIBRARY_GEMM_MODE!r}")
+LIBRARY_GEMM = LIBRARY_GEMM_MODE != "own"
+LIBRARY_WORKSPACE_BYTES = 76 << 20    # what the library may use beside the operands (stream-K partial tiles)
 LIBRARY_GEMM_MIN_ROWS = 65
 # Between 17 and 64 rows the weight-streaming kernel re-reads the activations
 # once per 16 weight rows, which costs more than the weights themselves when the
@@ -466,6 +472,55 @@ LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
 
 
 _MM_FLOAT_OUT = True   # torch.mm(..., out_dtype=float32) exists and works (found out at the first use)
+_blas_lib = None
+_blas_workspace: dict = {}
+
+
+def blas() -> ctypes.CDLL:
+    global _blas_lib
+    if _blas_lib is None:
+        require_gpu()
+        try:
+            lib = _load(build.blas_library())
+        except (RuntimeError, KernelError) as e:
+            raise KernelError(f"{e}\n(LYAPUNOV_AMD_GEMM=torch reaches the same library through torch)") from None
+        lib.lyp_last_error.restype = ctypes.c_char_p
+        lib.lyp_library_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            c_int, c_void_p, c_longlong, c_void_p]
+        lib.lyp_library_gemm_plans.restype = c_int
+        _blas_lib = lib
+    return _blas_lib
+
+
+def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out [M, N] (bfloat16 or float) = a [M, K] @ w [N, K].T for bfloat16
+    operands, by the vendor's library."""
+    M, K = a.shape
+    N = w.shape[0]
+    if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != K or tuple(out.shape) != (M, N)
+            or out.dtype not in (torch.bfloat16, torch.float32) or a.stride(1) != 1 or w.stride(1) != 1
+            or out.stride(1) != 1 or not (a.is_cuda and w.is_cuda and out.is_cuda)):
+        raise KernelError(f"library gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, "
+                          f"out {tuple(out.shape)} {out.dtype}")
+    if LIBRARY_GEMM_MODE == "torch":
+        global _MM_FLOAT_OUT
+        if out.dtype == torch.bfloat16:
+            return torch.matmul(a, w.t(), out=out)
+        if _MM_FLOAT_OUT:
+            try:   # the library's float accumulators written out as they are
+                return torch.mm(a, w.t(), out_dtype=torch.float32, out=out)
+            except (TypeError, RuntimeError):
+                _MM_FLOAT_OUT = False   # this torch cannot: the operands' type, then a cast
+        y = torch.matmul(a, w.t())
+        _check(core().lyp_cast(_p(y), _code(y.dtype), _p(out), _code(out.dtype), y.numel(), _stream()), core())
+        return out
+    lib = blas()
+    ws = _blas_workspace.get(a.device)
+    if ws is None:
+        ws = _blas_workspace[a.device] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=a.device)
+    _check(lib.lyp_library_gemm_nt(_p(a), _p(w), _p(out), _code(out.dtype), M, N, K, a.stride(0), w.stride(0),
+                                   out.stride(0), _p(ws), ws.numel(), _stream()), lib)
+    return out
 
 
 def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
@@ -483,7 +538,7 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
     if w.shape[1] != K or tuple(out.shape) != (M, N) or a.dtype != w.dtype:
         raise KernelError(f"gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
     if out.dtype == torch.bfloat16 and not accumulate and _library_product(M, N, K, a.dtype):
-        return torch.matmul(a, w.t(), out=out)
+        return library_gemm_nt(a, w, out)
     if accumulate:
         if out.dtype != torch.float32:
             raise KernelError("gemm: accumulation needs a float output")
@@ -529,14 +584,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
                                          w.stride(0), _stream()), lib)
             return parts
     if out_dtype == torch.float32 and _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
-        global _MM_FLOAT_OUT
-        if _MM_FLOAT_OUT:
-            try:   # the library's float accumulators written out as they are
-                return torch.mm(x, w.t(), out_dtype=torch.float32)
-            except (TypeError, RuntimeError):
-                _MM_FLOAT_OUT = False   # this torch cannot: the operands' type, then a cast
-        y = torch.empty((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
-        return cast(gemm_nt(x, w, y), torch.float32)
+        _dev(x, w)   # the library's float accumulators written out as they are
+        return library_gemm_nt(x, w, torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device))
     if out_dtype in (x.dtype, torch.float32):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
         return gemm_nt(x, w, out)
