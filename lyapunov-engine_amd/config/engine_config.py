@@ -4,7 +4,7 @@ Names and defaults follow the reference's EngineConfig
 (python/lyapunov_engine/engine/llm_engine.py:18-38): ``num_blocks`` (alias
 ``num_gpu_blocks``) 1024, ``block_size`` 16, ``max_num_seqs`` 64,
 ``max_num_batched_tokens`` 2048, ``dtype``, ``device``.  Added: the model length,
-the longest prompt portion per step, a seed, the graph and look-ahead switches, and an override
+the longest prompt portion per step, a seed, the graph, look-ahead and warm-up switches, and an override
 of the end-of-sequence ids (the reference fixes 128001 in its scheduler,
 csrc/include/engine/scheduler.hpp:16).
 """
@@ -44,6 +44,7 @@ class EngineConfig:
     enable_graphs: bool = True              # replay pure-decode steps from captured HIP graphs
     lookahead: bool = True                  # start the next decode step before this one's tokens reach the host
     eos_token_ids: Optional[tuple] = None   # default: the model's
+    warmup: bool = True                     # run one full step at start-up: libraries loaded, GEMM algorithms chosen by measurement
 
     def __post_init__(self):
         if self.num_gpu_blocks is not None:

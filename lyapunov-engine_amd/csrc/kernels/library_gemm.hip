@@ -5,9 +5,18 @@
 //
 // The library's own call costs a few microseconds on the host once the product's
 // description and the chosen algorithm are kept; building them anew for every
-// call (what a general tensor library does) costs four times that, which is what
+// call (what a general tensor library does) costs twice that, which is what
 // a prompt of a few hundred tokens spends most of its time on.  So: one plan per
 // (shape, strides, output type), made at the first call and reused.
+//
+// The library's heuristic orders its algorithms by a model of the machine.  While
+// tuning is switched on (lyp_library_gemm_tuning, meant for an engine's warm-up and
+// for the run before a graph is captured), a shape's first call runs the first
+// few candidates on the call's own operands, under the conditions of a model step,
+// and keeps the fastest.  For the products of a prompt the library's first choice
+// wins every time; for those of 33 to 64 rows (decode steps of large batches) it
+// does not.  A plan, once made, is never changed: the same shape gives the same
+// sums for as long as the process lives.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 
@@ -38,6 +47,9 @@ State& state() {
   return s;
 }
 
+int g_tuning_candidates = 0;   // > 1: a new plan is chosen by measurement among this many candidates
+constexpr int kMostCandidates = 32;
+
 #define LYP_BLAS(call, what)                                                       \
   do {                                                                             \
     const hipblasStatus_t st_ = (call);                                            \
@@ -47,8 +59,67 @@ State& state() {
     }                                                                              \
   } while (0)
 
+// Runs the product `times` times with candidate `c`; false if the library refuses it.
+bool run_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulHeuristicResult_t& c, const void* a,
+                   const void* w, void* out, void* workspace, hipStream_t stream, int times) {
+  const float alpha = 1.0f, beta = 0.0f;
+  for (int i = 0; i < times; ++i)
+    if (hipblasLtMatmul(handle, p.desc, &alpha, w, p.lw, a, p.la, &beta, out, p.lo, out, p.lo, &c.algo, workspace,
+                        c.workspaceSize, stream) != HIPBLAS_STATUS_SUCCESS)
+      return false;
+  return true;
+}
+
+// The fastest of the candidates on the operands of this call (which it runs several times: the
+// output is written again and again with the same values).  Waits for the stream.  A product in
+// a model step finds its weights in memory, not in a cache (a step reads more weights than the
+// caches hold), and its activations just written: before every timed run the caches are filled
+// with other data and the activations are read once.  Candidates ranked with everything still
+// in the cache from the run before were slower in the step than the library's first choice.
+int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulHeuristicResult_t* found, int n_found,
+                      const void* a, size_t a_bytes, const void* w, void* out, void* workspace, size_t workspace_bytes,
+                      hipStream_t stream) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return 0;
+  constexpr size_t kFlushBytes = size_t{512} << 20;   // twice the memory-side cache
+  void* other = nullptr;
+  if (hipMalloc(&other, kFlushBytes + a_bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int best = 0;
+  float best_ms = -1.f;
+  if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+    for (int c = 0; c < n_found; ++c) {
+      if (found[c].workspaceSize > workspace_bytes) continue;
+      if (!run_candidate(handle, p, found[c], a, w, out, workspace, stream, 1)) continue;
+      float fastest = -1.f;
+      for (int run = 0; run < 3; ++run) {
+        float ms = 0.f;
+        if (hipMemsetAsync(other, run, kFlushBytes, stream) != hipSuccess ||
+            hipMemcpyAsync(static_cast<char*>(other) + kFlushBytes, a, a_bytes, hipMemcpyDeviceToDevice, stream) != hipSuccess ||
+            hipEventRecord(e0, stream) != hipSuccess || !run_candidate(handle, p, found[c], a, w, out, workspace, stream, 1) ||
+            hipEventRecord(e1, stream) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+            hipEventElapsedTime(&ms, e0, e1) != hipSuccess) {
+          fastest = -1.f;
+          break;
+        }
+        if (fastest < 0.f || ms < fastest) fastest = ms;
+      }
+      if (fastest >= 0.f && (best_ms < 0.f || fastest < best_ms)) best_ms = fastest, best = c;
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipStreamSynchronize(stream);
+  (void)hipFree(other);
+  // whatever candidate ran last, the output now holds the product; the caller runs the chosen one once more
+  return best_ms < 0.f ? 0 : best;
+}
+
 int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int lda, int ldw, int ldo, int out_type,
-              size_t workspace_bytes) {
+              const void* a, const void* w, void* out, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   // Row-major out = a w^T is, in the library's column-major terms, out^T [N, M] = w^T-stored [K, N] transposed
   // times a-stored [K, M].
   const hipDataType in_t = HIP_R_16BF, out_t = out_type == kF32 ? HIP_R_32F : HIP_R_16BF;
@@ -64,18 +135,23 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int lda, i
   uint64_t ws = workspace_bytes;
   hipblasStatus_t st =
       hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-  hipblasLtMatmulHeuristicResult_t found[1];
+  hipblasLtMatmulHeuristicResult_t found[kMostCandidates];
   int n_found = 0;
+  const int wanted = g_tuning_candidates < 1 ? 1 : (g_tuning_candidates > kMostCandidates ? kMostCandidates : g_tuning_candidates);
   if (st == HIPBLAS_STATUS_SUCCESS)
-    st = hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.lw, p.la, p.lo, p.lo, pref, 1, found, &n_found);
+    st = hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.lw, p.la, p.lo, p.lo, pref, wanted, found, &n_found);
   hipblasLtMatmulPreferenceDestroy(pref);
   LYP_BLAS(st, "AlgoGetHeuristic");
   if (n_found < 1) {
     lyp::set_error("library gemm: the library has no algorithm for %d x %d x %d", M, N, K);
     return -1;
   }
-  p.algo = found[0].algo;
-  p.workspace = found[0].workspaceSize;
+  const int chosen =
+      n_found > 1 ? fastest_candidate(handle, p, found, n_found, a, static_cast<size_t>(M - 1) * lda * 2 + static_cast<size_t>(K) * 2,
+                                      w, out, workspace, workspace_bytes, stream)
+                  : 0;
+  p.algo = found[chosen].algo;
+  p.workspace = found[chosen].workspaceSize;
   return 0;
 }
 
@@ -110,7 +186,9 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
   auto it = s.plans.find(key);
   if (it == s.plans.end()) {
     Plan p;
-    if (make_plan(h->second, p, M, N, K, lda, ldw, ldo, out_dtype, static_cast<size_t>(workspace_bytes)) != 0) return -1;
+    if (make_plan(h->second, p, M, N, K, lda, ldw, ldo, out_dtype, a, w, out, workspace,
+                  static_cast<size_t>(workspace_bytes), stream) != 0)
+      return -1;
     it = s.plans.emplace(key, p).first;
   }
   const Plan& p = it->second;
@@ -122,6 +200,15 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
                            p.workspace, stream),
            "hipblasLtMatmul");
   return 0;
+}
+
+// candidates > 1: from now on the plan of a shape not seen before is chosen by running that many of
+// the library's candidates (at most 32) on the first call's operands, which waits for the stream;
+// 0 or 1: the library's first choice, without a measurement.  Returns the previous setting.
+int lyp_library_gemm_tuning(int candidates) {
+  const int before = g_tuning_candidates;
+  g_tuning_candidates = candidates;
+  return before;
 }
 
 // Number of plans kept (for tests).

@@ -84,9 +84,11 @@ class _Captured:
             tile_q0=empty, n_tiles=0, dec_seqs=None, n_dec=B, max_ctx_dec=ctx_cap, q_start_host=list(range(B + 1)),
             ctx_len_host=[0] * B, state_slots_host=[0] * B, workspace=self.workspace)
         caches = runner.layer_caches(self.ctx)
-        # One run outside the capture loads the libraries and sizes the scratch
-        # buffers; with every context at 0 it stores nothing in the cache.
-        runner.model.forward(self.ctx, caches)
+        # One run outside the capture loads the libraries, sizes the scratch
+        # buffers and lets the vendor library's algorithms for this many rows be
+        # chosen by measurement; with every context at 0 it stores nothing in the cache.
+        with ops.library_gemm_tuning():
+            runner.model.forward(self.ctx, caches)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, pool=pool):

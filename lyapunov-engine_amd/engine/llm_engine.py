@@ -108,6 +108,37 @@ class LLMEngine:
         self._look_ahead = bool(config.lookahead) and not self.core.pools.state
         self._ahead: Optional[_Ahead] = None
         self.steps_taken_ahead = 0    # steps whose results came from a step started ahead
+        if config.warmup:
+            self._warm_up()
+
+    WARMUP_ID = -1   # the cache manager's name for the warm-up step's request; the scheduler counts from 0
+
+    def _warm_up(self) -> None:
+        """One step of as many tokens as a step may bring (as far as the model's
+        length and the pages go), of a request that is gone afterwards.  It
+        loads the kernels a full step needs, and the products of that many rows
+        are given the fastest of the vendor library's algorithms by measurement
+        (``ops.library_gemm_tuning``) rather than the library's first guess."""
+        from ..kernels import ops
+
+        cache, cfg = self.core.cache, self.config
+        pages = min(cache.num_free_pages(g) for g in range(len(cache.groups)))
+        sizes = {cfg.max_num_batched_tokens}
+        if cfg.max_chunk:
+            sizes.add(min(cfg.max_chunk, cfg.max_num_batched_tokens))
+        for n in sorted(min(s, self.max_model_len, pages * self.core.block_size) for s in sizes):
+            if n < 1 or cache.has(self.WARMUP_ID) or cache.num_free_slots() < 1:
+                continue
+            cache.add(self.WARMUP_ID)
+            try:
+                cache.extend(self.WARMUP_ID, n)
+                with ops.library_gemm_tuning():
+                    self.core.runner.step_arrays(np.asarray([self.WARMUP_ID], dtype=np.int64), np.zeros(1, dtype=np.int32),
+                                                 np.asarray([n], dtype=np.int32), np.zeros(n, dtype=np.int32),
+                                                 np.asarray([n - 1], dtype=np.int32))
+                torch.cuda.synchronize(self.core.device)
+            finally:
+                cache.free(self.WARMUP_ID)
 
     # ---------------------------------------------------------------- requests
     def add_request(self, arg1, arg2=None, arg3=None):

@@ -469,6 +469,10 @@ LIBRARY_GEMM_MIN_ROWS = 65
 # matrix is large; measured, the library is ahead from this many weights on.
 LIBRARY_GEMM_MID_ROWS = 17
 LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
+# In an engine's warm-up step and in the run before a graph is captured, a library product's algorithm is
+# chosen by measurement among this many of the library's candidates (at the shape's first call).
+# LYAPUNOV_AMD_GEMM_TUNE=0 leaves every choice to the library.
+LIBRARY_TUNE_CANDIDATES = int(os.environ.get("LYAPUNOV_AMD_GEMM_TUNE", "16"))
 
 
 _MM_FLOAT_OUT = True   # torch.mm(..., out_dtype=float32) exists and works (found out at the first use)
@@ -488,8 +492,30 @@ def blas() -> ctypes.CDLL:
         lib.lyp_library_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_library_gemm_plans.restype = c_int
+        lib.lyp_library_gemm_tuning.argtypes = [c_int]
         _blas_lib = lib
     return _blas_lib
+
+
+class library_gemm_tuning:
+    """While this context is open, a library product of a shape not seen before
+    in this process is given the fastest of the library's first ``candidates``
+    algorithms, found by running them on the call's operands (which waits for
+    the stream); shapes seen before keep their plan.  Meant for a warm-up step."""
+
+    def __init__(self, candidates: int | None = None):
+        self.candidates = LIBRARY_TUNE_CANDIDATES if candidates is None else candidates
+        self.before = None
+
+    def __enter__(self):
+        if LIBRARY_GEMM_MODE == "library" and self.candidates > 1:
+            self.before = blas().lyp_library_gemm_tuning(self.candidates)
+        return self
+
+    def __exit__(self, *exc):
+        if self.before is not None:
+            blas().lyp_library_gemm_tuning(self.before)
+        return False
 
 
 def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
