@@ -204,8 +204,9 @@ __device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
 // PAIRED (8 rows of W, or two tiles of 8; at most 8 tokens): the tile's upper half repeats the 8 rows of W and the
 // tile's upper 8 columns the tokens, both 64 values of K further on, so that one matrix instruction
 // does two chunks of K (on the tile's diagonal blocks; the other two are not used) and no load
-// asks for a value twice.
-template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false>
+// asks for a value twice.  With TB = 2 (9 to 16 tokens, 8 rows of W) a wave keeps two such tiles over
+// one set of weights: tokens 0-7 and 8-15.
+template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false, int TB = 1>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
                                                            int ldw, int ldc, RopeTail tail, NormHead head,
@@ -217,8 +218,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   // With 16 rows of W a paired wave keeps two tiles, rows 0-7 and 8-15, over the same tokens: MB counts them.
   static_assert(!PAIRED || (EPI == kEpiResidual && ((ROWS == 8 && MB == 1) || (ROWS == 16 && MB == 2))),
                 "two chunks per tile: 8 rows (or twice 8), 8 tokens");
+  static_assert(TB == 1 || (TB == 2 && PAIRED && MB == 1), "blocks of 8 tokens: for the paired tile of 8 rows");
+  constexpr int NT = MB * TB;                // tiles (accumulators) a wave keeps
+  constexpr int NB = PAIRED ? TB : MB;       // blocks of tokens whose activations it loads
   constexpr int CHUNK = PAIRED ? 128 : 64;  // values of K per step of a wave
-  extern __shared__ float red[];       // [waves][MB][64][4], then MB * 16 floats for the epilogues' row values
+  extern __shared__ float red[];       // [waves][NT][64][4], then [waves][16] floats for the epilogues' row values
 
   const int lane = threadIdx.x % kWave;
   // the same in every lane, and said so: the loop over this wave's share of K then has scalar bounds and
@@ -236,12 +240,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   const int per_wave = (s_end - s_begin + nwaves - 1) / nwaves;
   const int c_begin = min(s_end, s_begin + wave * per_wave), c_end = min(s_end, c_begin + per_wave);
 
-  f32x4 acc[MB];
+  f32x4 acc[NT];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int b = 0; b < NT; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // Small loads that the epilogue needs are started here, ahead of the stream of weights.
-  float* row_val = red + static_cast<size_t>(nwaves) * MB * 256;  // [waves][16]
+  float* row_val = red + static_cast<size_t>(nwaves) * NT * 256;  // [waves][16]
   if constexpr (NORMED) {
     // Every token's sum of squares, from the producer's partial sums [parts][16]: thread t adds up
     // four tokens (t % 4) over every (threads / 4)-th part, the lanes of a wave meet by shuffles, the
@@ -269,9 +273,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   float h_first = 0.f, nw_first = 0.f;  // kEpiResidual: what the thread's first element adds to and is weighted by
   if constexpr (EPI == kEpiResidual) {
     const int e = threadIdx.x, l = (e % 256) / 4, in_tile = 4 * (l / 16) + e % 4;
-    const int row = PAIRED ? 8 * (e / 256) + in_tile : in_tile;
-    const int m = (PAIRED ? 0 : (e / 256) * 16) + l % 16, n = n0 + row;
-    if (e < MB * 256 && in_tile < (PAIRED ? 8 : ROWS) && m < M && n < N) {
+    const int row = PAIRED ? 8 * (e / 256 / TB) + in_tile : in_tile;
+    const int m = (PAIRED ? 8 * (e / 256 % TB) : (e / 256) * 16) + l % 16, n = n0 + row;
+    if (e < NT * 256 && in_tile < (PAIRED ? 8 : ROWS) && (!PAIRED || l % 16 < 8) && m < M && n < N) {
       h_first = static_cast<const float*>(Cv)[static_cast<size_t>(m) * ldc + n];
       if (res.next_w)
         nw_first = res.next_w_f32 ? static_cast<const float*>(res.next_w)[n]
@@ -285,10 +289,10 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems + second;
   const T* wp_upper = wp;  // PAIRED with 16 rows: the same lanes' rows 8-15
   if constexpr (PAIRED && MB == 2) wp_upper = W + static_cast<size_t>(min(n0 + 8 + r % 8, N - 1)) * ldw + j * MM::kElems + second;
-  const T* ap[MB];  // rows past the end read the last row and are not stored
+  const T* ap[NB];  // rows past the end read the last row and are not stored
 #pragma unroll
-  for (int b = 0; b < MB; ++b)
-    ap[b] = A + static_cast<size_t>(min(PAIRED ? r % 8 : b * 16 + r, M - 1)) * lda + j * MM::kElems + second;
+  for (int b = 0; b < NB; ++b)
+    ap[b] = A + static_cast<size_t>(min(PAIRED ? 8 * b + r % 8 : b * 16 + r, M - 1)) * lda + j * MM::kElems + second;
 
   // U chunks of 64 values of K at once: all of their loads are asked for before the first product
   // needs one.  (The matrix instruction counts as a convergent operation, and the compiler does not
@@ -321,7 +325,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     }
     // the activations come from the cache: four chunks of them at a time are enough
 #pragma unroll
-    for (int b = 0; b < MB; ++b) {
+    for (int b = 0; b < NB; ++b) {
 #pragma unroll
       for (int u0 = 0; u0 < U; u0 += 4) {
         constexpr int V = U < 4 ? U : 4;
@@ -343,17 +347,17 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   for (; c < c_end; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
 
   // acc[b][i]: output feature n0 + 4 j + i, token 16 b + r
-  float* mine = red + (static_cast<size_t>(wave) * MB * 64 + lane) * 4;
+  float* mine = red + (static_cast<size_t>(wave) * NT * 64 + lane) * 4;
 #pragma unroll
-  for (int b = 0; b < MB; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
+  for (int b = 0; b < NT; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
   __syncthreads();
   // The sum over the waves, in order; NORMED: times the row's 1 / rms.
   auto total = [&](int e) {
     float sum = 0.f;
-    for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * MB * 256 + e];
+    for (int w = 0; w < nwaves; ++w) sum += red[static_cast<size_t>(w) * NT * 256 + e];
     if constexpr (PAIRED) {  // row + 8, token + 8: the chunks' second halves
       float upper = 0.f;
-      for (int w = 0; w < nwaves; ++w) upper += red[static_cast<size_t>(w) * MB * 256 + e + 160];
+      for (int w = 0; w < nwaves; ++w) upper += red[static_cast<size_t>(w) * NT * 256 + e + 160];
       sum += upper;
     }
     if constexpr (NORMED) {
@@ -363,14 +367,15 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     }
     return sum;
   };
-  float* sq_el = row_val + nwaves * 16;  // kEpiResidual with by-products: [256] squares of the new h, by element
-  for (int e = threadIdx.x; e < MB * 256; e += blockDim.x) {
+  float* sq_el = row_val + nwaves * 16;  // kEpiResidual with by-products: [NT][256] squares of the new h, by element
+  for (int e = threadIdx.x; e < NT * 256; e += blockDim.x) {
     const int b = e / 256, l = (e % 256) / 4, i = e % 4;
     const int in_tile = 4 * (l / 16) + i;
-    // PAIRED: tile b holds rows 8 b .. 8 b + 7 of W for tokens 0-7; else rows 0-15 for tokens 16 b .. + 15
-    const int row = PAIRED ? 8 * b + in_tile : in_tile;
-    const int m = (PAIRED ? 0 : b * 16) + l % 16, n = n0 + row;
-    if (in_tile >= (PAIRED ? 8 : ROWS) || m >= M || n >= N) continue;
+    // PAIRED: tile b holds rows 8 (b / TB) .. + 7 of W for tokens 8 (b % TB) .. + 7 (its lower left block; the
+    // upper right one is added by total()); else rows 0-15 for tokens 16 b .. + 15
+    const int row = PAIRED ? 8 * (b / TB) + in_tile : in_tile;
+    const int m = (PAIRED ? 8 * (b % TB) : b * 16) + l % 16, n = n0 + row;
+    if (in_tile >= (PAIRED ? 8 : ROWS) || (PAIRED && l % 16 >= 8) || m >= M || n >= N) continue;
     if constexpr (EPI == kEpiRope) {
       const int head = n0 / tail.hd, blk = (n0 % tail.hd) / 16;
       const bool is_q = head < tail.nh, is_k = !is_q && head < tail.nh + tail.nkv;
@@ -443,7 +448,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
         float sq = 0.f;
         for (int row = 0; row < ROWS && n0 + row < N && m < M; ++row) {
           const int in_tile = PAIRED ? row % 8 : row;
-          sq += sq_el[(PAIRED ? 256 * (row / 8) : 0) + 4 * (t % 16 + 16 * (in_tile / 4)) + in_tile % 4];
+          sq += sq_el[(PAIRED ? 256 * ((row / 8) * TB + t / 8) + 4 * (t % 8 + 16 * (in_tile / 4))
+                              : 4 * (t % 16 + 16 * (in_tile / 4))) + in_tile % 4];
         }
         res.ssq_part[static_cast<size_t>(blockIdx.x) * 16 + m] = sq;
       }
@@ -480,17 +486,22 @@ template <typename T, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED =
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                           int slices, hipStream_t stream, const RopeTail& tail = RopeTail{},
                           const NormHead& head = NormHead{}, const ResidualTail& res = ResidualTail{}) {
-  const int MB = PAIRED ? ROWS / 8 : (M + 15) / 16;  // tiles a wave keeps
+  // tiles a wave keeps: paired, 8 rows of W each for 8 tokens each; else 16 rows of W for 16 tokens each
+  const int MB = PAIRED ? (ROWS / 8) * ((M + 7) / 8) : (M + 15) / 16;
   const int waves = skinny_waves(N, K, MB, slices, ROWS, PAIRED ? 128 : 64);
   const dim3 grid((N + ROWS - 1) / ROWS, slices), block(waves * kWave);
   const size_t lds = (static_cast<size_t>(waves) * MB * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
                      sizeof(float);
-#define LYP_SKINNY(MBV)                                                                                      \
-  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, \
-                                                                                      ldc, tail, head, res)
+#define LYP_SKINNY_TB(MBV, TBV)                                                                                   \
+  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED, TBV><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, \
+                                                                                           ldc, tail, head, res)
+#define LYP_SKINNY(MBV) LYP_SKINNY_TB(MBV, 1)
   if constexpr (PAIRED && ROWS == 16) {
-    LYP_SKINNY(2);
-  } else if constexpr (NORMED || PAIRED) {
+    LYP_SKINNY(2);  // at most 8 rows: the caller has checked
+  } else if constexpr (PAIRED) {
+    if (M <= 8) LYP_SKINNY(1);
+    else LYP_SKINNY_TB(1, 2);  // at most 16 rows: the caller has checked
+  } else if constexpr (NORMED) {
     LYP_SKINNY(1);  // at most 16 rows: the callers have checked
   } else {
     if (MB == 1) LYP_SKINNY(1);
@@ -499,6 +510,7 @@ static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, 
     else LYP_SKINNY(4);
   }
 #undef LYP_SKINNY
+#undef LYP_SKINNY_TB
 }
 
 template <typename T, int MODE>
@@ -660,7 +672,7 @@ extern "C" int lyp_gemm_residual(const void* A, const void* W, float* h, int dty
   LYP_REQUIRE(!next_w || (xs && ssq_part && ldx >= N && M <= 16), "gemm_residual: by-products for %d rows", M);
   if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
   const ResidualTail res{next_w, next_w_dtype == kF32, xs, ldx, ssq_part};
-  const bool paired = M <= 8 && K % 128 == 0;  // two chunks of K per matrix instruction
+  const bool paired = M <= 16 && K % 128 == 0;  // two chunks of K per matrix instruction
   const bool wide = residual_rows(M, N, K) == 16;
 #define LYP_RESIDUAL(T, ROWS, PAIRED)                                                                           \
   launch_skinny<T, kEpiResidual, false, ROWS, PAIRED>(static_cast<const T*>(A), static_cast<const T*>(W), h, M, N, \

@@ -170,7 +170,7 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torc
 #                  and ``linear_swiglu`` multiply those rows and divide by the
 #                  rms at the end.
 # Whoever cannot fold one in calls its ``run()`` and gets the plain tensor.
-PENDING_MAX_ROWS = 8
+PENDING_MAX_ROWS = 16
 
 
 class PendingLinear:

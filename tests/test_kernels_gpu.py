@@ -136,7 +136,9 @@ def test_linear_partial_sums(ops, dtype, M, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 2048, 8192), (8, 100, 192), (5, 515, 1024), (8, 4096, 1024),
-                                   (3, 4101, 384), (7, 3072, 256)])
+                                   (3, 4101, 384), (7, 3072, 256),
+                                   # 9 to 16 rows: two blocks of 8 tokens over one set of weights
+                                   (9, 2048, 8192), (16, 2048, 2048), (12, 515, 1024), (13, 4101, 384), (16, 100, 192)])
 def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N, K):
     """A projection of few rows handed on instead of run (pending=True) and
     then added to the float residual stream by the product kernel itself."""
@@ -159,7 +161,8 @@ def test_product_added_to_the_residual_stream_in_its_own_kernel(ops, dtype, M, N
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,K,J", [(1, 2048, 192), (8, 192, 192), (5, 1024, 256), (7, 256, 384), (8, 320, 128), (6, 4096, 256)])
+@pytest.mark.parametrize("M,K,J", [(1, 2048, 192), (8, 192, 192), (5, 1024, 256), (7, 256, 384), (8, 320, 128), (6, 4096, 256),
+                                   (9, 2048, 256), (16, 1024, 384), (11, 320, 192), (16, 4096, 128)])
 def test_norm_folded_into_the_products_around_it(ops, dtype, M, K, J):
     """The product that adds to the residual stream prepares the RMS norm that
     follows (rmsnorm_pending), and the gate/up and the q/k/v products finish
@@ -182,7 +185,11 @@ def test_norm_folded_into_the_products_around_it(ops, dtype, M, K, J):
     g = torch.Generator().manual_seed(43)
     wg, wu = (torch.randn(I, K, generator=g) * 0.1).to(dtype), (torch.randn(I, K, generator=g) * 0.1).to(dtype)
     w = torch.stack([wg.view(-1, 8, K), wu.view(-1, 8, K)], dim=1).reshape(2 * I, K).contiguous().to(DEV)
-    want = P.mlp(x64, wg.double(), wu.double(), torch.eye(I, dtype=torch.float64))
+    # What the consuming products are given: h * weight rounded to the activations' type (its agreement with
+    # the plain norm was checked above), so that their own arithmetic is what the comparison below sees.
+    x_in = x64 if dtype == torch.float32 else (
+        pending.xs.cpu().double() / torch.sqrt(h.cpu().double().pow(2).mean(-1, keepdim=True) + eps))
+    want = P.mlp(x_in, wg.double(), wu.double(), torch.eye(I, dtype=torch.float64))
     got = ops.linear_swiglu(pending, w, 8)
     torch.testing.assert_close(got.cpu().double(), want, **tol(dtype, 2e-5, 3e-2))
     # q/k/v with rotation and page write
@@ -197,7 +204,7 @@ def test_norm_folded_into_the_products_around_it(ops, dtype, M, K, J):
     q = ops.linear_rope_kv(pending, wq.to(DEV), positions.to(DEV), table, slots.to(DEV), kpool, vpool, num_heads=nh,
                            num_kv_heads=nkv, head_dim=hd, page_size=bs)
     assert q.shape == (M, nh * hd)
-    qkv = (x64 @ wq.double().T).view(M, nh + 2 * nkv, hd)
+    qkv = (x_in @ wq.double().T).view(M, nh + 2 * nkv, hd)
     cos, sin = P.rope_cos_sin(positions, P.rope_inv_freq(hd, 10000.0))
     rotated = P.apply_rope(qkv[:, : nh + nkv].transpose(0, 1), cos.double(), sin.double()).transpose(0, 1)
     t = tol(dtype, 2e-5, 3e-2)
