@@ -148,6 +148,8 @@ class LLMEngine:
             request_id, prompt, params = arg1, list(arg2), arg3 or SamplingParams()
         elif isinstance(arg1, (list, tuple)):
             request_id, prompt = self.req_counter, list(arg1)
+            while request_id in self._by_request:    # a caller's own id may be this number already
+                request_id += 1
             params = arg2 if isinstance(arg2, SamplingParams) else SamplingParams()
         else:
             raise TypeError("Invalid arguments provided to add_request")
