@@ -38,6 +38,15 @@ def _bucket(n: int, smallest: int) -> int:
     return b
 
 
+def _batch_bucket(n: int) -> int:
+    """Batch sizes a graph is captured for: 1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48,
+    64, ...  A step pays for its padded rows nearly as for real ones (33
+    requests in a graph of 64 took 19 % longer than 32 in one of 32), so the
+    steps between powers of two (the reference's buckets) get graphs too."""
+    b = _bucket(n, 1)
+    return b * 3 // 4 if b >= 4 and n <= b * 3 // 4 else b
+
+
 class _Captured:
     TURNS = 3
 
@@ -134,7 +143,7 @@ class DecodeGraphs:
 
     def __init__(self, runner: ModelRunner, max_batch: int):
         self.runner = runner
-        self.max_batch = _bucket(max_batch, 1)
+        self.max_batch = _batch_bucket(max_batch)
         self.captured: dict = {}
         self.pool = None
         self.safe = all(part.graph_safe for _, part in runner.model.named_parts())
@@ -153,7 +162,7 @@ class DecodeGraphs:
         each request's one new token (int32); or the ids of the tokens as a
         tensor on the device (``tokens_dev``)."""
         ctx_need = int(starts.max()) + 1
-        key = (_bucket(len(ids), 1), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
+        key = (_batch_bucket(len(ids)), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
         cap = self.captured.get(key)
         if cap is None:
             if self.pool is None:
