@@ -48,6 +48,7 @@ State& state() {
 }
 
 int g_tuning_candidates = 0;   // > 1: a new plan is chosen by measurement among this many candidates
+bool g_tuning_no_workspace = false;  // ... of which only those that need no workspace are taken
 constexpr int kMostCandidates = 32;
 
 #define LYP_BLAS(call, what)                                                       \
@@ -92,7 +93,7 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
   float best_ms = -1.f;
   if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
     for (int c = 0; c < n_found; ++c) {
-      if (found[c].workspaceSize > workspace_bytes) continue;
+      if (found[c].workspaceSize > workspace_bytes || (g_tuning_no_workspace && found[c].workspaceSize > 0)) continue;
       if (!run_candidate(handle, p, found[c], a, w, out, workspace, stream, 1)) continue;
       float fastest = -1.f;
       for (int run = 0; run < 3; ++run) {
@@ -115,7 +116,11 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
   (void)hipStreamSynchronize(stream);
   (void)hipFree(other);
   // whatever candidate ran last, the output now holds the product; the caller runs the chosen one once more
-  return best_ms < 0.f ? 0 : best;
+  if (best_ms >= 0.f) return best;
+  if (g_tuning_no_workspace)   // none could be timed: at least one that needs no workspace, if there is one
+    for (int c = 0; c < n_found; ++c)
+      if (found[c].workspaceSize == 0) return c;
+  return 0;
 }
 
 int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int lda, int ldw, int ldo, int out_type,
@@ -204,10 +209,15 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
 
 // candidates > 1: from now on the plan of a shape not seen before is chosen by running that many of
 // the library's candidates (at most 32) on the first call's operands, which waits for the stream;
-// 0 or 1: the library's first choice, without a measurement.  Returns the previous setting.
-int lyp_library_gemm_tuning(int candidates) {
+// 0 or 1: the library's first choice, without a measurement.  Returns the previous number of
+// candidates (to be handed back, with no_workspace 0, when the tuning ends).
+// With no_workspace only candidates that need no workspace are taken: for products that are about
+// to be recorded into a graph (an algorithm with a workspace may clear it with a memset node, and
+// memset nodes in replayed graphs are not to be trusted on this machine).
+int lyp_library_gemm_tuning(int candidates, int no_workspace) {
   const int before = g_tuning_candidates;
   g_tuning_candidates = candidates;
+  g_tuning_no_workspace = no_workspace != 0;
   return before;
 }
 

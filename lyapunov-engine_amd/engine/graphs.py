@@ -95,8 +95,9 @@ class _Captured:
         caches = runner.layer_caches(self.ctx)
         # One run outside the capture loads the libraries, sizes the scratch
         # buffers and lets the vendor library's algorithms for this many rows be
-        # chosen by measurement; with every context at 0 it stores nothing in the cache.
-        with ops.library_gemm_tuning():
+        # chosen by measurement, among those that need no workspace (no memset is to be
+        # recorded); with every context at 0 it stores nothing in the cache.
+        with ops.library_gemm_tuning(for_graph=True):
             runner.model.forward(self.ctx, caches)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()

@@ -492,7 +492,7 @@ def blas() -> ctypes.CDLL:
         lib.lyp_library_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_library_gemm_plans.restype = c_int
-        lib.lyp_library_gemm_tuning.argtypes = [c_int]
+        lib.lyp_library_gemm_tuning.argtypes = [c_int, c_int]
         _blas_lib = lib
     return _blas_lib
 
@@ -503,18 +503,22 @@ class library_gemm_tuning:
     algorithms, found by running them on the call's operands (which waits for
     the stream); shapes seen before keep their plan.  Meant for a warm-up step."""
 
-    def __init__(self, candidates: int | None = None):
+    def __init__(self, candidates: int | None = None, for_graph: bool = False):
+        """``for_graph``: the products are about to be recorded into a graph;
+        only algorithms that need no workspace are taken (one with a workspace
+        may clear it with a memset node, which replayed graphs must not hold)."""
         self.candidates = LIBRARY_TUNE_CANDIDATES if candidates is None else candidates
+        self.for_graph = for_graph
         self.before = None
 
     def __enter__(self):
         if LIBRARY_GEMM_MODE == "library" and self.candidates > 1:
-            self.before = blas().lyp_library_gemm_tuning(self.candidates)
+            self.before = blas().lyp_library_gemm_tuning(self.candidates, int(self.for_graph))
         return self
 
     def __exit__(self, *exc):
         if self.before is not None:
-            blas().lyp_library_gemm_tuning(self.before)
+            blas().lyp_library_gemm_tuning(self.before, 0)
         return False
 
 

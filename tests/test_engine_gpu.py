@@ -216,6 +216,47 @@ def test_graph_steps_equal_eager_steps(model_folders):
     assert len(graphs.captured) == 1
 
 
+def test_graph_of_many_rows_with_library_products_equals_eager(tmp_path):
+    """A layer as wide as the 1B shape's, so that the products of a decode step
+    of 40 requests go to the vendor's library (in the graph with algorithms
+    chosen by measurement for the graph's 48 rows, eagerly with the library's
+    first choice for 40): every replay of the graph, with eager steps between
+    the replays, gives the eager step's logits up to bfloat16 rounding."""
+    from lyapunov_engine_amd.engine.core import EngineCore, StepEntry
+    from lyapunov_engine_amd.engine.graphs import DecodeGraphs
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=512, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
+    folder = str(tmp_path / "wide")
+    os.makedirs(folder)
+    write_random_model(cfg, folder, 3, "bfloat16", init_std=0.02)
+    n = 40
+    assert ops._library_product(n, 2 * 8192, 2048, torch.bfloat16) and ops._library_product(n, 2048, 8192, torch.bfloat16)
+    core = EngineCore.from_folder(folder, dtype="bfloat16", num_blocks=n * 4 + 8, block_size=16, num_state_slots=64)
+    graphs = DecodeGraphs(core.runner, max_batch=64)
+    lens = [3 + (5 * i) % 17 for i in range(n)]
+    for i in range(n):
+        core.cache.add(i)
+        core.cache.extend(i, lens[i] + 8)
+        core.step([StepEntry(i, random_tokens(lens[i], 512, seed=i), 0, [])])
+        core.cache.commit(i, lens[i])
+    plans_before = ops.blas().lyp_library_gemm_plans()
+    for k in range(5):
+        entries = [StepEntry(i, [(11 * k + 3 * i) % 512], lens[i] + k, [0]) for i in range(n)]
+        eager = core.step(entries).clone()
+        torch.cuda.synchronize()
+        replayed = graphs.step(entries).clone()
+        scale = float(eager.abs().max())
+        assert float((replayed - eager).abs().max()) <= 0.03 * scale, f"replay {k}"
+        for e in entries:
+            core.cache.commit(e.seq_id, e.start + 1)
+    assert [key[0] for key in graphs.captured] == [48]
+    assert ops.blas().lyp_library_gemm_plans() > plans_before       # the library was used, for 40 and for 48 rows
+
+
 def test_seeded_sampling_does_not_depend_on_batch_mates(model_folders):
     import lyapunov_engine_amd as L
 
