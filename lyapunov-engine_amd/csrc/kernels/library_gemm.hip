@@ -48,7 +48,7 @@ State& state() {
 }
 
 int g_tuning_candidates = 0;   // > 1: a new plan is chosen by measurement among this many candidates
-bool g_tuning_no_workspace = false;  // ... of which only those that need no workspace are taken
+bool g_tuning_no_workspace = false;  // a new plan's algorithm is one that needs no workspace
 constexpr int kMostCandidates = 32;
 
 #define LYP_BLAS(call, what)                                                       \
@@ -93,7 +93,7 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
   float best_ms = -1.f;
   if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
     for (int c = 0; c < n_found; ++c) {
-      if (found[c].workspaceSize > workspace_bytes || (g_tuning_no_workspace && found[c].workspaceSize > 0)) continue;
+      if (found[c].workspaceSize > workspace_bytes) continue;
       if (!run_candidate(handle, p, found[c], a, w, out, workspace, stream, 1)) continue;
       float fastest = -1.f;
       for (int run = 0; run < 3; ++run) {
@@ -116,11 +116,7 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
   (void)hipStreamSynchronize(stream);
   (void)hipFree(other);
   // whatever candidate ran last, the output now holds the product; the caller runs the chosen one once more
-  if (best_ms >= 0.f) return best;
-  if (g_tuning_no_workspace)   // none could be timed: at least one that needs no workspace, if there is one
-    for (int c = 0; c < n_found; ++c)
-      if (found[c].workspaceSize == 0) return c;
-  return 0;
+  return best_ms < 0.f ? 0 : best;
 }
 
 int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int lda, int ldw, int ldo, int out_type,
@@ -137,6 +133,7 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, int M, int N, int K, int lda, i
   LYP_BLAS(hipblasLtMatrixLayoutCreate(&p.lo, out_t, N, M, ldo), "layout of the output");
   hipblasLtMatmulPreference_t pref = nullptr;
   LYP_BLAS(hipblasLtMatmulPreferenceCreate(&pref), "PreferenceCreate");
+  if (g_tuning_no_workspace) workspace_bytes = 0;  // the library then offers only algorithms that need none
   uint64_t ws = workspace_bytes;
   hipblasStatus_t st =
       hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));

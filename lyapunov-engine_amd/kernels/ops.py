@@ -512,7 +512,7 @@ class library_gemm_tuning:
         self.before = None
 
     def __enter__(self):
-        if LIBRARY_GEMM_MODE == "library" and self.candidates > 1:
+        if LIBRARY_GEMM_MODE == "library" and (self.candidates > 1 or self.for_graph):
             self.before = blas().lyp_library_gemm_tuning(self.candidates, int(self.for_graph))
         return self
 
