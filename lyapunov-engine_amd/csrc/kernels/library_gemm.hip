@@ -35,7 +35,8 @@ struct Plan {
   size_t workspace = 0;
 };
 
-using Key = std::tuple<int, int, int, int, int, int, int, int>;  // device, M, N, K, lda, ldw, ldo, out type
+// device, M, N, K, lda, ldw, ldo, out type, made for a graph (without a workspace)
+using Key = std::tuple<int, int, int, int, int, int, int, int, int>;
 
 struct State {
   std::map<int, hipblasLtHandle_t> handles;  // per device
@@ -184,7 +185,7 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
     LYP_BLAS(hipblasLtCreate(&handle), "hipblasLtCreate");
     h = s.handles.emplace(device, handle).first;
   }
-  const Key key{device, M, N, K, lda, ldw, ldo, out_dtype};
+  const Key key{device, M, N, K, lda, ldw, ldo, out_dtype, g_tuning_no_workspace ? 1 : 0};
   auto it = s.plans.find(key);
   if (it == s.plans.end()) {
     Plan p;
@@ -208,9 +209,10 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
 // the library's candidates (at most 32) on the first call's operands, which waits for the stream;
 // 0 or 1: the library's first choice, without a measurement.  Returns the previous number of
 // candidates (to be handed back, with no_workspace 0, when the tuning ends).
-// With no_workspace only candidates that need no workspace are taken: for products that are about
-// to be recorded into a graph (an algorithm with a workspace may clear it with a memset node, and
-// memset nodes in replayed graphs are not to be trusted on this machine).
+// With no_workspace the library is asked for algorithms that need no workspace: for products that
+// are about to be recorded into a graph (an algorithm with a workspace may clear it with a memset
+// node, and memset nodes in replayed graphs are not to be trusted on this machine).  Such plans are
+// kept apart from the others, so the setting has to stay on while the graph is recorded.
 int lyp_library_gemm_tuning(int candidates, int no_workspace) {
   const int before = g_tuning_candidates;
   g_tuning_candidates = candidates;

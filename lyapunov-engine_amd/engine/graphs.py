@@ -99,10 +99,10 @@ class _Captured:
         # recorded); with every context at 0 it stores nothing in the cache.
         with ops.library_gemm_tuning(for_graph=True):
             runner.model.forward(self.ctx, caches)
-        torch.cuda.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, pool=pool):
-            self.logits = runner.model.forward(self.ctx, caches)
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, pool=pool):
+                self.logits = runner.model.forward(self.ctx, caches)
 
     def fill(self, runner: ModelRunner, ids, starts, tokens) -> None:
         """Write the step's tables into the pinned host buffer.  ids (int64),
