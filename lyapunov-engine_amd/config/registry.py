@@ -90,5 +90,13 @@ def load_config(model_dir: str):
         raise FileNotFoundError(f"{model_dir} has no config.json")
     with open(path, "r", encoding="utf-8") as f:
         raw = json.load(f)
+    # The end-of-sequence ids may stand in generation_config.json instead (the reference fixes
+    # 128001 in its scheduler, csrc/include/engine/scheduler.hpp:16, and reads neither file for them).
+    extra = os.path.join(model_dir, "generation_config.json")
+    if raw.get("eos_token_id") is None and os.path.exists(extra):
+        with open(extra, "r", encoding="utf-8") as f:
+            eos = json.load(f).get("eos_token_id")
+        if eos is not None:
+            raw = dict(raw, eos_token_id=eos)
     arch = architecture_of(raw)
     return arch, arch.config_class.from_dict(raw)

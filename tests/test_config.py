@@ -95,6 +95,23 @@ def test_registry_picks_the_model_by_name():
         MIXERS.register("paged_attention", object)
 
 
+def test_end_of_sequence_ids_may_stand_in_generation_config(tmp_path):
+    import json
+
+    from lyapunov_engine_amd.config.registry import load_config
+
+    d = dict(TINY_A)
+    d.pop("eos_token_id", None)
+    (tmp_path / "config.json").write_text(json.dumps(d))
+    assert load_config(str(tmp_path))[1].eos_token_id == ()
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [5, 9], "temperature": 0.6}))
+    assert load_config(str(tmp_path))[1].eos_token_id == (5, 9)
+    (tmp_path / "config.json").write_text(json.dumps(dict(d, eos_token_id=7)))   # config.json wins when it names them
+    assert load_config(str(tmp_path))[1].eos_token_id == (7,)
+    with pytest.raises(FileNotFoundError, match="config.json"):
+        load_config(str(tmp_path / "nowhere"))
+
+
 def test_the_two_tiny_configurations_differ_in_everything():
     a, b = LlamaConfig.from_dict(TINY_A), LlamaConfig.from_dict(TINY_B)
     for f in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
