@@ -156,8 +156,9 @@ class LLMEngine:
         if request_id in self._by_request:
             raise ValueError(f"request id {request_id!r} is in use")
         vocab = self.core.model.spec.vocab_size
-        if any((not isinstance(t, int)) or t < 0 or t >= vocab for t in prompt):
-            raise ValueError(f"prompt holds a token outside the vocabulary of {vocab}")
+        ids = np.asarray(prompt)
+        if ids.ndim != 1 or (ids.size and (ids.dtype.kind not in "iu" or int(ids.min()) < 0 or int(ids.max()) >= vocab)):
+            raise ValueError(f"a prompt is a list of token ids below the vocabulary's {vocab}")
         seq_id = self.req_counter
         self.req_counter += 1
         self.scheduler.add(seq_id, prompt, params)

@@ -4,7 +4,7 @@ csrc/engine/scheduler.cpp:7-138, bound there with pybind11,
 csrc/bindings.cpp:552-621)."""
 from __future__ import annotations
 
-from ctypes import c_float, c_int32, c_int64, c_uint64
+from ctypes import POINTER, c_float, c_int32, c_int64, c_uint64
 from dataclasses import dataclass
 
 import numpy as np
@@ -71,8 +71,9 @@ class Scheduler:
         return rc
 
     def add(self, seq_id: int, prompt: list, params: SamplingParams) -> None:
-        arr = (c_int32 * max(1, len(prompt)))(*prompt)
-        self._rc(self._lib.lyp_sched_add(self._h, seq_id, arr, len(prompt), params.temperature, params.top_p,
+        arr = np.ascontiguousarray(prompt, dtype=np.int32)
+        self._rc(self._lib.lyp_sched_add(self._h, seq_id, arr.ctypes.data_as(POINTER(c_int32)), len(arr),
+                                         params.temperature, params.top_p,
                                          params.top_k, params.max_tokens, int(params.ignore_eos),
                                          c_uint64((params.seed or 0) & ((1 << 64) - 1))))
 

@@ -274,6 +274,31 @@ def test_seeded_sampling_does_not_depend_on_batch_mates(model_folders):
     assert len(set(alone)) > 4  # it does sample: greedy on this model repeats itself quickly
 
 
+def test_requests_that_make_no_sense_are_refused_when_added(model_folders):
+    import lyapunov_engine_amd as L
+
+    engine = L.LLM(model_folders["A"]["float32"], dtype="float32", num_blocks=32, block_size=4).engine
+    sp = L.SamplingParams(temperature=0.0, max_tokens=4)
+    for prompt, words in [([1, 2, 256], "token ids below"), ([1, -1], "token ids below"), ([1.5, 2.0], "token ids below"),
+                          ([[1, 2], [3, 4]], "token ids below"), ([], "empty prompt"), ([1] * 256, "max_model_len"),
+                          ([1] * 200, "pages")]:
+        with pytest.raises((ValueError, RuntimeError), match=words):
+            engine.add_request("bad", prompt, sp)
+        assert not engine.has_unfinished_requests()
+    engine.add_request("a", [1, 2, 3], sp)
+    with pytest.raises(ValueError, match="in use"):
+        engine.add_request("a", [4, 5], sp)
+    first = engine.add_request([4, 5], sp)              # an anonymous request gets a number of its own
+    assert first != "a" and engine.add_request(first + 1, [6], sp) == first + 1
+    assert engine.add_request([7, 8], sp) not in ("a", first, first + 1)
+    done = {}
+    while engine.has_unfinished_requests():
+        for out in engine.step():
+            if out.finished:
+                done[out.request_id] = out
+    assert len(done) == 4 and all(len(o.output_tokens) == 4 for o in done.values())
+
+
 def test_eos_stops_a_request(model_folders):
     import lyapunov_engine_amd as L
 
