@@ -457,7 +457,7 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 # 112-117, 177).  Products with few rows (decode steps), every float product
 # (true 32-bit) and everything when LYAPUNOV_AMD_GEMM=own use the kernels here.
 # LYAPUNOV_AMD_GEMM: "library" (the default: hipBLASLt called directly, with the plan of every shape
-# kept), "torch" (the same library behind torch.matmul: 18 us of host time a call instead of 4), "own".
+# kept), "torch" (the same library behind torch.matmul: 18 us of host time a call instead of 10), "own".
 LIBRARY_GEMM_MODE = os.environ.get("LYAPUNOV_AMD_GEMM", "library")
 if LIBRARY_GEMM_MODE not in ("library", "torch", "own"):
     raise KernelError(f"LYAPUNOV_AMD_GEMM is 'library', 'torch' or 'own', not {LIBRARY_GEMM_MODE!r}")
