@@ -478,6 +478,7 @@ LIBRARY_TUNE_CANDIDATES = int(os.environ.get("LYAPUNOV_AMD_GEMM_TUNE", "16"))
 _MM_FLOAT_OUT = True   # torch.mm(..., out_dtype=float32) exists and works (found out at the first use)
 _blas_lib = None
 _blas_workspace: dict = {}
+_blas_tuning = (0, 0)   # (candidates, without a workspace): the library's setting, kept here while it is not loaded
 
 
 def blas() -> ctypes.CDLL:
@@ -493,6 +494,7 @@ def blas() -> ctypes.CDLL:
                                             c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_library_gemm_plans.restype = c_int
         lib.lyp_library_gemm_tuning.argtypes = [c_int, c_int]
+        lib.lyp_library_gemm_tuning(*_blas_tuning)   # what a tuning context asked for before the library was there
         _blas_lib = lib
     return _blas_lib
 
@@ -513,13 +515,23 @@ class library_gemm_tuning:
 
     def __enter__(self):
         if LIBRARY_GEMM_MODE == "library" and (self.candidates > 1 or self.for_graph):
-            self.before = blas().lyp_library_gemm_tuning(self.candidates, int(self.for_graph))
+            self.before = _blas_tuning
+            _set_blas_tuning(self.candidates, int(self.for_graph))
         return self
 
     def __exit__(self, *exc):
         if self.before is not None:
-            blas().lyp_library_gemm_tuning(self.before, 0)
+            _set_blas_tuning(*self.before)
         return False
+
+
+def _set_blas_tuning(candidates: int, no_workspace: int) -> None:
+    """The library is loaded by the first product that needs it (a 32-bit
+    engine never does); until then the setting waits here."""
+    global _blas_tuning
+    _blas_tuning = (candidates, no_workspace)
+    if _blas_lib is not None:
+        _blas_lib.lyp_library_gemm_tuning(candidates, no_workspace)
 
 
 def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
