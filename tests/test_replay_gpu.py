@@ -282,3 +282,32 @@ def test_trace_run_program(model_folders, tmp_path):
     got = {n: np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, vocab) for n in t.rows}
     assert not (out / "1.f32").exists()
     compare(t, got, want, dtype, "trace_run")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_layer_of_the_benchmark_shape(tmp_path, dtype):
+    """One layer as wide as the Llama 3.2 1B shape (the sizes the benchmark runs
+    at: products over 2,048 and 8,192 values, 32 heads over 8, llama3 scaling),
+    through steps of 100 rows (the vendor library's products in bfloat16, the
+    tiled 32-bit kernel in float32), 58 rows, 11 rows (a portion beside decoded
+    tokens, the folded kernels of up to 16 rows) and 3 rows, against the plain
+    implementation."""
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=128))
+    d = str(tmp_path / "wide")
+    os.makedirs(d)
+    write_random_model(cfg, d, 11, dtype, init_std=0.03, norm_init_std=0.1)
+    reqs = {"a": random_tokens(150, 1000, seed=1), "b": random_tokens(60, 1000, seed=2), "c": random_tokens(20, 1000, seed=3)}
+    t = Trace(reqs)
+    t.step([("a", 100)])
+    t.step([("a", 18), ("b", 40)], want="last")
+    t.step([("a", 1), ("b", 1), ("c", 9)])
+    for _ in range(8):
+        t.step([("a", 1), ("b", 1), ("c", 1)])
+    t.step([("a", 23), ("b", 11), ("c", 3)], end=["a", "b", "c"])
+    compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "wide layer")
