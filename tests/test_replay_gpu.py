@@ -285,17 +285,19 @@ def test_trace_run_program(model_folders, tmp_path):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_layer_of_the_benchmark_shape(tmp_path, dtype):
-    """One layer as wide as the Llama 3.2 1B shape (the sizes the benchmark runs
-    at: products over 2,048 and 8,192 values, 32 heads over 8, llama3 scaling),
-    through steps of 100 rows (the vendor library's products in bfloat16, the
-    tiled 32-bit kernel in float32), 58 rows, 11 rows (a portion beside decoded
+@pytest.mark.parametrize("hidden,heads,head_dim", [(2048, 32, 64), (3072, 24, 128)])
+def test_a_layer_of_the_benchmark_shape(tmp_path, dtype, hidden, heads, head_dim):
+    """One layer as wide as the Llama 3.2 1B shape, and one as wide as the 3B
+    shape (the sizes the benchmark runs at: products over 2,048 / 3,072 and
+    8,192 values, 32 heads of 64 or 24 of 128 over 8, llama3 scaling), through
+    steps of 100 rows (the vendor library's products in bfloat16, the tiled
+    32-bit kernel in float32), 58 rows, 11 rows (a portion beside decoded
     tokens, the folded kernels of up to 16 rows) and 3 rows, against the plain
     implementation."""
     from lyapunov_engine_amd.weights import write_random_model
 
-    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
-               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=hidden, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=heads, num_key_value_heads=8, head_dim=head_dim,
                max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
                rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
                                  original_max_position_embeddings=128))
