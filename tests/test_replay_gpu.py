@@ -313,3 +313,29 @@ def test_a_layer_of_the_benchmark_shape(tmp_path, dtype, hidden, heads, head_dim
         t.step([("a", 1), ("b", 1), ("c", 1)])
     t.step([("a", 23), ("b", 11), ("c", 3)], end=["a", "b", "c"])
     compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "wide layer")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_wide_layer_over_a_long_context(tmp_path, dtype):
+    """The same layer at 2,400 tokens: the prompt in two uneven portions (the
+    second one's workgroups take the keys of the first in runs), a portion of 40
+    tokens at the end of it, and decoded tokens over all of it in partitions."""
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=1024))
+    d = str(tmp_path / "wide")
+    os.makedirs(d)
+    write_random_model(cfg, d, 12, dtype, init_std=0.03, norm_init_std=0.1)
+    reqs = {"a": random_tokens(2400, 1000, seed=4), "b": random_tokens(30, 1000, seed=5)}
+    t = Trace(reqs)
+    t.step([("a", 1900)], want="last")
+    t.step([("a", 450), ("b", 20)], want="last")
+    t.step([("a", 40), ("b", 1)])
+    for _ in range(9):
+        t.step([("a", 1), ("b", 1)])
+    t.step([("a", 1)], end=["a", "b"])
+    compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "wide layer, long context")
