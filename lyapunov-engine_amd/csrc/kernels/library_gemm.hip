@@ -190,8 +190,13 @@ int lyp_library_gemm_nt(const void* a, const void* w, void* out, int out_dtype, 
   if (it == s.plans.end()) {
     Plan p;
     if (make_plan(h->second, p, M, N, K, lda, ldw, ldo, out_dtype, a, w, out, workspace,
-                  static_cast<size_t>(workspace_bytes), stream) != 0)
+                  static_cast<size_t>(workspace_bytes), stream) != 0) {
+      if (p.lw) hipblasLtMatrixLayoutDestroy(p.lw);  // what a failed attempt had made so far
+      if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
+      if (p.lo) hipblasLtMatrixLayoutDestroy(p.lo);
+      if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
       return -1;
+    }
     it = s.plans.emplace(key, p).first;
   }
   const Plan& p = it->second;
