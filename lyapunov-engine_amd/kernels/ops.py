@@ -116,14 +116,16 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _current_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _stream() -> c_void_p:
+# Addresses go to the libraries as plain integers: every function declares its pointer arguments,
+# so ctypes converts them, and no c_void_p object is built per argument.
+def _stream() -> int:
     if _raw_stream is not None and _current_device is not None:
-        return c_void_p(_raw_stream(_current_device()))
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(_current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
-def _p(t) -> c_void_p:
-    return c_void_p(0 if t is None else t.data_ptr())
+def _p(t) -> int:
+    return 0 if t is None else t.data_ptr()
 
 
 def _check(rc: int, lib: ctypes.CDLL) -> None:
