@@ -65,6 +65,7 @@ class ModelSpec:
     head_name: str = "lm_head.weight"
     layer_prefix: str = "model.layers.{i}."
     eos_token_ids: tuple = ()
+    ignorable_tensors: tuple = ()    # shell-style patterns of tensor names a file may hold unused
     init_std: float = 0.02           # random-weights mode: normal(0, init_std) matrices
     norm_init_std: float = 0.0       # random-weights mode: norm weights 1 + normal(0, norm_init_std)
 

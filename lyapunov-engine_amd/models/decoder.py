@@ -11,6 +11,7 @@ embedding matrix itself, not a copy (models/weight_loader.py:106-109 copies).
 """
 from __future__ import annotations
 
+import fnmatch
 from dataclasses import dataclass
 from typing import Iterator, Optional
 
@@ -90,9 +91,14 @@ class DecoderModel(Part):
                 out[s.name] = (tuple(s.shape), ws.init)
         return out
 
-    def ignorable_tensors(self) -> set:
-        """Names a file may hold without being used: a tied model's separate head."""
-        return {self.spec.head_name} if self.spec.tie_word_embeddings else set()
+    def ignorable(self, name: str) -> bool:
+        """Whether a file may hold this tensor without the model using it: a
+        tied model's separate head, and what the architecture declares
+        (``ModelSpec.ignorable_tensors``: shell-style patterns, for buffers that
+        exporters write and that are computed here, not loaded)."""
+        if self.spec.tie_word_embeddings and name == self.spec.head_name:
+            return True
+        return any(fnmatch.fnmatchcase(name, pat) for pat in self.spec.ignorable_tensors)
 
     def _plan_cache(self) -> CacheLayout:
         by_cache: dict = {}

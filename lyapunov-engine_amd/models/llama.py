@@ -40,6 +40,8 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         tie_word_embeddings=cfg.tie_word_embeddings,
         max_position=cfg.max_position_embeddings,
         eos_token_ids=tuple(cfg.eos_token_id),
+        # older exports carry every layer's rotary frequencies as a buffer; they are computed here
+        ignorable_tensors=("*.rotary_emb.inv_freq",),
     )
 
 

@@ -43,7 +43,7 @@ class FolderSource(TensorSource):
     def __init__(self, model_dir: str):
         self.files = open_model_files(model_dir)
         self.where = {}
-        for f in self.files:  # later files overwrite earlier ones (weight_loader.py:270-273)
+        for f in self.files:  # later files overwrite earlier ones (models/weight_loader.py:53-56: update() in sorted file order)
             for name in f.names():
                 self.where[name] = f
 
@@ -68,7 +68,7 @@ class DictSource(TensorSource):
 def check_tensors(model: DecoderModel, present: dict) -> None:
     expected = model.expected_tensors()
     missing = sorted(n for n in expected if n not in present)
-    unexpected = sorted(n for n in present if n not in expected and n not in model.ignorable_tensors())
+    unexpected = sorted(n for n in present if n not in expected and not model.ignorable(n))
     wrong = sorted((n, tuple(present[n]), expected[n][0]) for n in expected
                    if n in present and tuple(present[n]) != tuple(expected[n][0]))
     if not (missing or unexpected or wrong):
@@ -94,9 +94,10 @@ def kept_dtype(stored: torch.dtype, engine_dtype: torch.dtype) -> torch.dtype:
 
 def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, device) -> DecoderModel:
     check_tensors(model, source.shapes())
-    for name in sorted(set(source.shapes()) & model.ignorable_tensors()):
-        print(f"[lyapunov-amd] note: {name} is in the files but the model ties its head to the embedding; ignored",
-              file=sys.stderr)
+    expected = model.expected_tensors()
+    for name in sorted(n for n in source.shapes() if n not in expected):
+        print(f"[lyapunov-amd] note: {name} is in the files and not used by this model (a separate head of a tied "
+              f"model, or a buffer the architecture declares ignorable); ignored", file=sys.stderr)
     device = torch.device(device)
     for owner, ws in model.weight_table():
         pieces = [source.get(s.name) for s in ws.sources]

@@ -190,6 +190,73 @@ def test_forward_norm_placement_and_residuals():
     torch.testing.assert_close(P.forward(w, CFG, toks), want)
 
 
+def test_rope_frequencies_elementwise():
+    """theta^(-2i/d) for i = 0 .. d/2 - 1, as models/llama.py:180-183 and the oracle of
+    tests/test_fused_rope.py:16-18 (arange(0, d, 2) / d): an exponent of i/d would pass
+    "first is 1, then falling" and fails here."""
+    for d, theta in ((16, 10000.0), (64, 500000.0), (128, 10000.0)):
+        inv = P.rope_inv_freq(d, theta)
+        assert inv.shape == (d // 2,)
+        want = torch.tensor([theta ** (-2.0 * i / d) for i in range(d // 2)], dtype=torch.float64)
+        torch.testing.assert_close(inv.double(), want, rtol=1e-6, atol=0)
+        assert float(inv[-1]) == pytest.approx(theta ** (-(d - 2) / d), rel=1e-6)   # the slowest pair: almost 1/theta
+    # the table's angle at position p is p * inv_freq: the pair (i, i + d/2) of a one-hot vector turns by it
+    inv = P.rope_inv_freq(8, 100.0)
+    e = torch.zeros(1, 1, 8, dtype=torch.float64)
+    e[..., 2] = 1.0
+    cos, sin = P.rope_cos_sin(torch.tensor([5]), inv)
+    out = P.apply_rope(e, cos, sin)[0, 0]
+    angle = 5 * 100.0 ** (-2.0 * 2 / 8)
+    assert abs(out[2] - math.cos(angle)) < 1e-6 and abs(out[6] - math.sin(angle)) < 1e-6
+
+
+def test_llama3_middle_band_is_a_straight_blend():
+    """Inside the band the new frequency is (1 - s) f / factor + s f with s running straight from 0
+    at wavelength L / low to 1 at L / high in L / wavelength: halfway it is the mean of the two ends,
+    a quarter in it is 3:1.  Continuity at the ends alone would also pass a curve of another shape."""
+    L, low, high, factor = 8192.0, 1.0, 4.0, 32.0
+    for s in (0.25, 0.5, 0.75):
+        ratio = low + s * (high - low)            # L / wavelength
+        f = torch.tensor([2 * math.pi * ratio / L], dtype=torch.float64)
+        out = P.llama3_scale_inv_freq(f, factor, low, high, L)
+        want = (1 - s) * f / factor + s * f
+        torch.testing.assert_close(out.double(), want, rtol=1e-6, atol=0)
+
+
+def test_each_norm_stands_before_its_own_branch():
+    """A norm weight of zero silences the branch behind it and nothing else (no biases anywhere):
+    with input_layernorm = 0 the layer is h + mlp(norm2(h)), with post_attention_layernorm = 0 it is
+    h + attention(norm1(h)).  Swapped norm weights, a norm after the branch, or a branch fed from
+    the wrong stream fail one of the two (models/llama.py:147-165)."""
+    cfg = dict(CFG, num_hidden_layers=1)
+    w = {k: v.double() for k, v in tiny_weights(cfg, seed=3).items()}
+    p = "model.layers.0."
+    S = 5
+    h = torch.randn(S, cfg["hidden_size"], dtype=torch.float64)
+    pos = torch.arange(S)
+    inv = P.model_inv_freq(cfg)
+    eps = cfg["rms_norm_eps"]
+
+    w1 = dict(w, **{p + "input_layernorm.weight": torch.zeros_like(w[p + "input_layernorm.weight"])})
+    want = h + P.mlp(P.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps), w[p + "mlp.gate_proj.weight"],
+                     w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    torch.testing.assert_close(P.decoder_layer(h, pos, w1, 0, cfg, inv), want)
+
+    w2 = dict(w, **{p + "post_attention_layernorm.weight": torch.zeros_like(w[p + "input_layernorm.weight"])})
+    x = P.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+    want = h + P.attention_layer(x, pos, w, p + "self_attn.", cfg, inv)
+    torch.testing.assert_close(P.decoder_layer(h, pos, w2, 0, cfg, inv), want)
+    # the second branch reads the stream *after* the first was added: with both norms alive the
+    # result differs from the sum of the two single-branch results
+    both = P.decoder_layer(h, pos, w, 0, cfg, inv)
+    alone = P.decoder_layer(h, pos, w1, 0, cfg, inv) + P.decoder_layer(h, pos, w2, 0, cfg, inv) - h
+    assert not torch.allclose(both, alone, atol=1e-6)
+    h1 = h + P.attention_layer(x, pos, w, p + "self_attn.", cfg, inv)
+    want = h1 + P.mlp(P.rms_norm(h1, w[p + "post_attention_layernorm.weight"], eps), w[p + "mlp.gate_proj.weight"],
+                      w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    torch.testing.assert_close(both, want)
+
+
 def test_sampling_follows_the_reference_rules():
     logits = torch.tensor([2.0, 1.0, 0.5, 0.0, -1.0, -3.0])
     assert P.greedy(logits) == 0

@@ -126,14 +126,14 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes():
     cfg, model = make(TINY_B)
     t = dict(random_tensors(model, 0, torch.float32))
     del t["model.layers.2.mlp.up_proj.weight"], t["lm_head.weight"]
-    t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    t["model.layers.0.self_attn.extra_bias"] = torch.zeros(16)
     t["model.layers.1.self_attn.q_proj.weight"] = torch.zeros(96, 95)
     t["model.norm.weight"] = torch.zeros(97)
     with pytest.raises(WeightError) as e:
         load_weights(model, DictSource(t), torch.float32, "cpu")
     msg = str(e.value)
     assert "missing (2)" in msg and "model.layers.2.mlp.up_proj.weight" in msg and "lm_head.weight" in msg
-    assert "unexpected (1)" in msg and "rotary_emb.inv_freq" in msg
+    assert "unexpected (1)" in msg and "self_attn.extra_bias" in msg
     assert "wrong shape (2)" in msg and "q_proj.weight is [96, 95], expected [96, 96]" in msg and "model.norm.weight" in msg
 
 
@@ -143,3 +143,16 @@ def test_a_tied_model_ignores_a_separate_head(capsys):
     t["lm_head.weight"] = torch.zeros(256, 64)
     load_weights(model, DictSource(t), torch.float32, "cpu")
     assert model.lm_head is model.embed and "lm_head.weight" in capsys.readouterr().err
+
+
+def test_buffers_the_architecture_declares_ignorable_do_not_stop_loading(capsys):
+    """Older exports store every layer's rotary frequencies; the model computes its own."""
+    cfg, model = make(TINY_B)
+    t = dict(random_tensors(model, 0, torch.float32))
+    for i in range(cfg.num_hidden_layers):
+        t[f"model.layers.{i}.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    load_weights(model, DictSource(t), torch.float32, "cpu")
+    assert "rotary_emb.inv_freq" in capsys.readouterr().err
+    t["model.layers.0.self_attn.rotary_emb.cos_cached"] = torch.zeros(4)     # not declared: still an error
+    with pytest.raises(WeightError, match="unexpected"):
+        load_weights(model, DictSource(t), torch.float32, "cpu")
