@@ -15,6 +15,9 @@
 // token order at a uniform number the caller supplies, so a request's tokens
 // depend on its own seed and not on what else is in the batch.
 #include "common.h"
+#include "sampler_api.h"
+
+#include <mutex>
 
 namespace lyp {
 
@@ -575,4 +578,52 @@ extern "C" int lyp_sample(const float* logits, int ld, int rows, int V, const fl
                                                       mirror);
   LYP_LAUNCH_CHECK("sample");
   return 0;
+}
+
+// ------------------------------------------------ the same, allocating nothing
+namespace lyp {
+constexpr int kStaticSampleRows = 1024;
+constexpr int kMaxDevices = 64;
+
+// The per-piece maxima of lyp_sample_static.  In host code this name is only a
+// handle for hipGetSymbolAddress; the address each GPU holds its copy at is
+// looked up once per device and kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[kStaticSampleRows * kArgmaxChunks * sizeof(ArgMax)];
+
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+// The current device's copy of `scratch`, or null with the error text set.
+static void* static_scratch() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error("sample_static: no current device (or one beyond %d)", kMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      set_error("sample_static: the scratch array's address on device %d: %s", device, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  return g_scratch_ptr[device];
+}
+}  // namespace lyp
+
+extern "C" int lyp_sample_static_max_rows(void) { return kStaticSampleRows; }
+
+extern "C" int lyp_sample_static(const float* logits, int ld, int rows, int V, const float* temperature,
+                                 const int32_t* top_k, const float* top_p, const float* uniform, int32_t* out,
+                                 int32_t* mirror, hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample_static: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
+  LYP_REQUIRE(rows <= kStaticSampleRows, "sample_static: %d rows, the built-in scratch array holds %d", rows,
+              kStaticSampleRows);
+  if (rows == 0) return 0;
+  void* ptr = static_scratch();
+  if (!ptr) return -1;
+  return lyp_sample(logits, ld, rows, V, temperature, top_k, top_p, uniform, ptr, out, mirror, stream);
 }
