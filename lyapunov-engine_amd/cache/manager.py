@@ -153,7 +153,8 @@ class CachePools:
 
     ``kv[g]`` is (keys, values) of group g with a leading dimension over the
     group's cache buffers; ``index[cache_id]`` says where a buffer lives;
-    ``state[cache_id]`` is the slot tensor of a stateful buffer.  Everything
+    ``state[cache_id]`` is the slot tensor of a stateful buffer (its last slot
+    belongs to no request: rows that are only padding use it).  Everything
     starts at zero: a page that was never written must not hold a NaN pattern.
     """
 
@@ -169,7 +170,8 @@ class CachePools:
             self.kv.append((k, v))
             for i, cache_id in enumerate(gl.buffers):
                 self.index[cache_id] = (g, i)
-        self.state = {cid: torch.zeros((num_state_slots,) + tuple(st.shape), dtype=st.dtype, device=device)
+        # one slot more than requests can hold: the padded rows of a recorded step are pointed at it
+        self.state = {cid: torch.zeros((num_state_slots + 1,) + tuple(st.shape), dtype=st.dtype, device=device)
                       for cid, st in layout.states.items()}
 
     def buffer(self, cache_id: int):

@@ -28,8 +28,15 @@ class EngineCore:
         self.runner = ModelRunner(model, self.cache, self.pools, self.dtype, self.device)
 
     @classmethod
-    def from_folder(cls, model_dir: str, *, dtype, device="cuda:0", source: Optional[TensorSource] = None, **kw):
-        model, cfg = load_model(model_dir, parse_dtype(dtype), device, source=source)
+    def from_folder(cls, model_dir: str, *, dtype, device="cuda:0", source: Optional[TensorSource] = None,
+                    max_model_len: Optional[int] = None, **kw):
+        """``max_model_len``: no request will be longer; with the pool's size
+        (``num_blocks * block_size``) it bounds the positions the model is set
+        up for (the rows of its position tables)."""
+        reach = kw["num_blocks"] * kw.get("block_size", 16)
+        if max_model_len:
+            reach = min(reach, int(max_model_len))
+        model, cfg = load_model(model_dir, parse_dtype(dtype), device, source=source, max_positions=reach)
         return cls(model, cfg, dtype=dtype, device=device, **kw)
 
     def step(self, entries: list):

@@ -27,8 +27,8 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from ..parts.base import GroupView, StepContext
-from .runner import ModelRunner, _align4
+from ..parts.base import FixedStep
+from .runner import ModelRunner, StepError
 
 
 def _bucket(n: int, smallest: int) -> int:
@@ -52,51 +52,28 @@ class _Captured:
 
     def __init__(self, runner: ModelRunner, batch: int, ctx_cap: int, pool):
         self.batch, self.ctx_cap = batch, ctx_cap
-        cache = runner.cache
-        B = batch
-        # layout of the fixed table buffer, in int32 words
-        self.sizes = [B, B, B + 1, B, B, B]   # token ids, positions, q_start, ctx_len, state slots, logit rows
-        self.widths = []
-        for gc in cache.groups:
-            width = max(1, -(-ctx_cap // gc.page_size))
-            self.widths.append(width)
-            self.sizes += [B, B * width]
-        self.offsets, total = [], 0
-        for s in self.sizes:
-            self.offsets.append(total)
-            total += _align4(s)
+        self.fixed = FixedStep(rows=batch, max_context=ctx_cap)
+        none64, none32 = np.zeros(0, np.int64), np.zeros(0, np.int32)
+        # The step function lays the tables out, as for any step; with no live request every row is
+        # padding (context 0, slot -1), so the runs below store nothing in the cache.
+        first = runner.step_tables(none64, none32, None, none32, None, fixed=self.fixed)
+        self.shape = first.shape_key()
+        self.token_words = first.offsets[0]
+        words = first.host.size
         # Several pinned copies of the table, used in turn: a step may be filled in while the copy
         # of the one before it to the device has not run yet.
-        self.hosts = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(self.TURNS)]
+        self.hosts = [torch.zeros(words, dtype=torch.int32).pin_memory() for _ in range(self.TURNS)]
         self.turn = 0
-        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
-        self.workspace: dict = {}
-        self._rows = np.arange(B)
-        for host in self.hosts:
-            h = host.numpy()
-            h[self.offsets[2]:self.offsets[2] + B + 1] = np.arange(B + 1)
-            h[self.offsets[5]:self.offsets[5] + B] = np.arange(B)
-        self.h = self.hosts[0].numpy()
-        self.fill(runner, np.zeros(0, np.int64), np.zeros(0, np.int32), np.zeros(0, np.int32))
+        self.hosts[0].numpy()[:] = first.host
+        self.dev = torch.zeros(words, dtype=torch.int32, device=runner.device)
         self.dev.copy_(self.hosts[0])
-
-        def view(i):
-            return self.dev[self.offsets[i]:self.offsets[i] + self.sizes[i]]
-
-        groups = [GroupView(page_size=gc.page_size, block_tables=view(7 + 2 * g).view(B, self.widths[g]),
-                            slot_mapping=view(6 + 2 * g), max_blocks=self.widths[g], window=gc.window)
-                  for g, gc in enumerate(cache.groups)]
-        empty = self.dev[:0]
-        self.ctx = StepContext(
-            device=runner.device, dtype=runner.dtype, T=B, B=B, token_ids=view(0), positions=view(1), q_start=view(2),
-            ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=B, groups=groups, tile_seq=empty,
-            tile_q0=empty, n_tiles=0, dec_seqs=None, n_dec=B, max_ctx_dec=ctx_cap, q_start_host=list(range(B + 1)),
-            ctx_len_host=[0] * B, state_slots_host=[0] * B, workspace=self.workspace)
+        self.workspace: dict = {}
+        self.ctx = runner.context(first, self.dev, workspace=self.workspace)
         caches = runner.layer_caches(self.ctx)
         # One run outside the capture loads the libraries, sizes the scratch
         # buffers and lets the vendor library's algorithms for this many rows be
         # chosen by measurement, among those that need no workspace (no memset is to be
-        # recorded); with every context at 0 it stores nothing in the cache.
+        # recorded).
         with ops.library_gemm_tuning(for_graph=True):
             runner.model.forward(self.ctx, caches)
             torch.cuda.synchronize()
@@ -104,37 +81,17 @@ class _Captured:
             with torch.cuda.graph(self.graph, pool=pool):
                 self.logits = runner.model.forward(self.ctx, caches)
 
-    def fill(self, runner: ModelRunner, ids, starts, tokens) -> None:
-        """Write the step's tables into the pinned host buffer.  ids (int64),
-        starts and tokens (int32) are numpy arrays, one entry per request; rows
-        past them are inert (context 0, slot -1)."""
-        B, cache, h, o = self.batch, runner.cache, self.h, self.offsets
-        n = len(ids)
-        h[o[0]:o[0] + n] = tokens
-        h[o[1]:o[1] + n] = starts
-        h[o[3]:o[3] + n] = starts
-        h[o[3]:o[3] + n] += 1
-        for i in (0, 1, 3, 4):
-            h[o[i] + n:o[i] + B] = 0
-        rows = self._rows[:n]
-        for g, gc in enumerate(cache.groups):
-            width, ps = self.widths[g], gc.page_size
-            sm = h[o[6 + 2 * g]:o[6 + 2 * g] + B]
-            bt = h[o[7 + 2 * g]:o[7 + 2 * g] + B * width].reshape(B, width)
-            if n:
-                cache.export(ids, g, bt, h[o[4]:o[4] + n] if g == 0 else None)
-                sm[:n] = bt[rows, starts // ps] * ps + starts % ps
-            sm[n:] = -1
-
     def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None) -> torch.Tensor:
         """``tokens_dev``: the token ids as an int32 tensor on the device, for a
         step whose tokens the host does not know yet (``tokens`` is ignored)."""
         self.turn = (self.turn + 1) % self.TURNS
-        self.h = self.hosts[self.turn].numpy()
-        self.fill(runner, ids, starts, tokens)
+        host = self.hosts[self.turn]
+        tables = runner.step_tables(ids, starts, None, tokens, None, fixed=self.fixed, host_for=lambda n: host.numpy())
+        if tables.shape_key() != self.shape:
+            raise StepError("a planner's arrays or launch shapes changed between two steps of one recorded shape: "
+                            "in a fixed step they may depend on the step's bounds alone")
         # one small kernel reads the pinned table (and the device's token ids) into place
-        ops.table_load(self.hosts[self.turn], self.dev, None if tokens_dev is None else tokens_dev[:len(ids)],
-                       self.offsets[0])
+        ops.table_load(host, self.dev, None if tokens_dev is None else tokens_dev[:len(ids)], self.token_words)
         self.graph.replay()
         return self.logits[:len(ids)]
 

@@ -30,6 +30,7 @@ step changes in place) does not look ahead.
 """
 from __future__ import annotations
 
+import sys
 from typing import Optional
 
 import numpy as np
@@ -87,8 +88,11 @@ class LLMEngine:
         else:
             self.core = EngineCore.from_folder(str(model), dtype=config.dtype, device=config.device,
                                                num_blocks=config.num_blocks, block_size=config.block_size,
-                                               num_state_slots=config.max_num_seqs)
+                                               num_state_slots=config.max_num_seqs,
+                                               max_model_len=config.max_model_len)
         spec = self.core.model.spec
+        # (the model's position tables may have fewer rows than spec.max_position: as many as the
+        # pool could ever hold; a request longer than that is refused for its pages, not its length)
         self.max_model_len = min(config.max_model_len or spec.max_position, spec.max_position)
         eos = config.eos_token_ids if config.eos_token_ids is not None else spec.eos_token_ids
         self.scheduler = Scheduler(self.core.cache, max_num_seqs=config.max_num_seqs,
@@ -215,7 +219,14 @@ class LLMEngine:
                 pending = self.sampler.launch(logits, [r.params for r in wanting], [r.stream for r in wanting],
                                               [len(r.outputs) for r in wanting])
         if decoding and self._look_ahead:
-            self._ahead = self._start_ahead(ids, start, reqs, pending)
+            # Optional work must not break the planned step: whatever goes wrong in starting the next
+            # one (a new graph that cannot be recorded, no memory for it), this step's tokens still
+            # reach the scheduler; looking ahead is then switched off.
+            try:
+                self._ahead = self._start_ahead(ids, start, reqs, pending)
+            except Exception as err:  # noqa: BLE001
+                self._ahead, self._look_ahead = None, False
+                print(f"[lyapunov-amd] looking ahead switched off: {type(err).__name__}: {err}", file=sys.stderr)
         sampled = pending.result() if pending is not None else []
         status = self.scheduler.post_step_status(sampled)
         outputs, k = [], 0

@@ -23,9 +23,7 @@ import torch
 from ..cache.manager import CacheError, CacheManager, CachePools
 from ..kernels import ops
 from ..models.decoder import DecoderModel
-from ..parts.base import GroupView, LayerCache, StepContext
-
-PREFILL_TILE = 64   # new tokens of one request per workgroup of the prefill attention kernel
+from ..parts.base import FixedStep, GroupView, LayerCache, StepBatch, StepContext, StepPlan
 
 
 @dataclass
@@ -44,13 +42,71 @@ def _align4(n: int) -> int:
     return (n + 3) & ~3
 
 
+@dataclass
+class StepTables:
+    """One step's integers, laid out for the device: the sections of the one
+    int32 buffer a step uploads (token ids, positions, request offsets and
+    lengths, state slots, logit rows, per cache group a slot mapping and a
+    block table, then whatever the parts' planners ask for), in host memory."""
+
+    host: np.ndarray                   # int32: the words, sections aligned to 16 bytes
+    names: list                        # section names; a planner's array is ("plan", key, name)
+    sizes: list
+    offsets: list
+    T: int
+    B: int
+    R: int
+    widths: list                       # block-table width per cache group
+    plan_meta: dict                    # planner key -> meta
+    q_start_host: list
+    ctx_len_host: list
+    state_slots_host: list
+    fixed: Optional[FixedStep] = None
+
+    def shape_key(self) -> tuple:
+        """What a recorded step depends on beside the words themselves."""
+        return (tuple(self.names), tuple(self.sizes), self.T, self.B, self.R, tuple(self.widths),
+                tuple(sorted((k, tuple(sorted(m.items()))) for k, m in self.plan_meta.items())))
+
+
+class _PinnedRing:
+    """Pinned host buffers used in turn for the eager step's upload: a kernel
+    reads the words straight from pinned memory, so the host neither stages the
+    copy nor waits for it; a buffer is written again only after the kernel that
+    read it last has run (an event per buffer)."""
+
+    TURNS = 4
+
+    def __init__(self):
+        self.buffers = [None] * self.TURNS
+        self.events = [None] * self.TURNS
+        self.turn = 0
+
+    def take(self, words: int) -> torch.Tensor:
+        self.turn = (self.turn + 1) % self.TURNS
+        if self.events[self.turn] is not None:
+            self.events[self.turn].synchronize()
+        buf = self.buffers[self.turn]
+        if buf is None or buf.numel() < words:
+            size = 1024
+            while size < words:
+                size *= 2
+            buf = self.buffers[self.turn] = torch.zeros(size, dtype=torch.int32).pin_memory()
+        return buf[:words]
+
+    def sent(self) -> None:
+        if self.events[self.turn] is None:
+            self.events[self.turn] = torch.cuda.Event()
+        self.events[self.turn].record()
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache: CacheManager, pools: CachePools, dtype: torch.dtype, device):
         self.model, self.cache, self.pools = model, cache, pools
         self.dtype, self.device = dtype, torch.device(device)
         self.layout = model.cache_layout()
         self.vocab_size = model.spec.vocab_size
-        self.max_position = model.spec.max_position
+        self.max_position = model.max_positions
         self.workspace: dict = {}
         ops.require_gpu()
         # what each call of the running order gets, apart from the step's tables
@@ -61,8 +117,15 @@ class ModelRunner:
             if g is not None:
                 _, k, v = pools.buffer(call.cache)
             self._calls.append((g, k, v, pools.state.get(call.cache), call.writes))
+        # the parts' planners, one per distinct key, in the order the parts come
+        self.planners: dict = {}
+        for _, part in model.named_parts():
+            planner = part.step_planner()
+            if planner is not None:
+                self.planners.setdefault(planner.key, planner)
+        self._ring = _PinnedRing()
 
-    # ------------------------------------------------------------ the context
+    # ------------------------------------------------------------- the tables
     def build_context(self, entries: list) -> StepContext:
         if not entries:
             raise StepError("a step needs at least one entry")
@@ -81,93 +144,155 @@ class ModelRunner:
             at += len(e.tokens)
         return self.build_context_arrays(ids, start, count, tokens, np.asarray(rows, dtype=np.int32))
 
-    def build_context_arrays(self, ids, start, count, tokens, rows) -> StepContext:
-        """The same from numpy arrays: request ids (int64); the position of each
-        request's first new token and the number of its new tokens (int32); all
-        new tokens in the order of the requests (int32); the rows (indices into
-        ``tokens``) whose logits are wanted (int32)."""
-        B = len(ids)
-        if B == 0:
-            raise StepError("a step needs at least one entry")
-        if len(np.unique(ids)) != B:
-            raise StepError(f"a request appears twice in one step: {ids.tolist()}")
-        if int(count.min()) < 1:
-            raise StepError(f"request {int(ids[int(count.argmin())])} brings no tokens")
-        q_start = np.zeros(B + 1, dtype=np.int32)
-        np.cumsum(count, out=q_start[1:])
-        T = int(q_start[-1])
-        ctx_len = start + count
-        if tokens.size != T:
-            raise StepError(f"{tokens.size} tokens for requests that bring {T}")
+    def step_tables(self, ids, start, count, tokens, rows, fixed: Optional[FixedStep] = None,
+                    host_for=None) -> StepTables:
+        """The step's integers from numpy arrays: request ids (int64); the
+        position of each request's first new token and the number of its new
+        tokens (int32); all new tokens in the order of the requests (int32);
+        the rows (indices into ``tokens``) whose logits are wanted (int32).
+
+        ``fixed``: the step is (a replay of) a recorded one: ``fixed.rows``
+        requests of one token each, of which the given ones are live and the
+        rest padding; the logits of every row are wanted; ``count`` and ``rows``
+        are ignored, and the requests' pages are taken as they are (no check
+        that a request holds exactly ``start`` tokens: a step started ahead of
+        the bookkeeping runs this way).  ``host_for(words)`` supplies the host
+        memory (an int32 numpy array of that length)."""
+        n = len(ids)
+        if fixed is None:
+            B = n
+            if B == 0:
+                raise StepError("a step needs at least one entry")
+            if len(np.unique(ids)) != B:
+                raise StepError(f"a request appears twice in one step: {ids.tolist()}")
+            if int(count.min()) < 1:
+                raise StepError(f"request {int(ids[int(count.argmin())])} brings no tokens")
+            q_start = np.zeros(B + 1, dtype=np.int32)
+            np.cumsum(count, out=q_start[1:])
+            T = int(q_start[-1])
+            ctx_len = start + count
+            if tokens.size != T:
+                raise StepError(f"{tokens.size} tokens for requests that bring {T}")
+            if int(tokens.min()) < 0 or int(tokens.max()) >= self.vocab_size:
+                bad = int(np.flatnonzero((tokens < 0) | (tokens >= self.vocab_size))[0])
+                b = int(np.searchsorted(q_start, bad, side="right")) - 1
+                raise StepError(f"request {int(ids[b])} has a token outside the vocabulary of {self.vocab_size}")
+            if rows.size and (int(rows.min()) < 0 or int(rows.max()) >= T):
+                raise StepError("logits are wanted at a place the step does not bring")
+            positions = np.arange(T, dtype=np.int32) + np.repeat(start - q_start[:-1], count)
+            ctx_bound = int(ctx_len.max())
+        else:
+            B = T = fixed.rows
+            if n > B:
+                raise StepError(f"{n} requests in a recorded step of {B} rows")
+            q_start = np.arange(B + 1, dtype=np.int32)
+            count = np.ones(B, dtype=np.int32)
+            ctx_len = np.zeros(B, dtype=np.int32)
+            ctx_len[:n] = start
+            ctx_len[:n] += 1
+            positions = np.zeros(B, dtype=np.int32)
+            positions[:n] = start
+            full = np.zeros(B, dtype=np.int32)
+            full[:n] = tokens
+            tokens, start = full, positions
+            rows = np.arange(B, dtype=np.int32)
+            ctx_bound = fixed.max_context
+            if n and int(ctx_len.max()) > ctx_bound:
+                raise StepError(f"a request of {int(ctx_len.max())} tokens in a step recorded for {ctx_bound}")
         if int(ctx_len.max()) > self.max_position:
             b = int(ctx_len.argmax())
-            raise StepError(f"request {int(ids[b])} would reach position {int(ctx_len[b]) - 1}, beyond the model's "
-                            f"{self.max_position}")
-        if int(tokens.min()) < 0 or int(tokens.max()) >= self.vocab_size:
-            bad = int(np.flatnonzero((tokens < 0) | (tokens >= self.vocab_size))[0])
-            b = int(np.searchsorted(q_start, bad, side="right")) - 1
-            raise StepError(f"request {int(ids[b])} has a token outside the vocabulary of {self.vocab_size}")
-        if rows.size and (int(rows.min()) < 0 or int(rows.max()) >= T):
-            raise StepError("logits are wanted at a place the step does not bring")
-        positions = np.arange(T, dtype=np.int32) + np.repeat(start - q_start[:-1], count)
-        slots = np.empty(B, dtype=np.int32)
+            raise StepError(f"request {int(ids[b])} would reach position {int(ctx_len[b]) - 1}, beyond the "
+                            f"{self.max_position} positions this engine was set up for")
+        batch = StepBatch(start=start, count=count, q_start=q_start, ctx_len=ctx_len, T=T, B=B, fixed=fixed)
+        plans = {key: planner.plan(batch) for key, planner in self.planners.items()}
 
-        # Attention work: tiles of PREFILL_TILE new tokens of requests that bring several, sorted by
-        # (keys up to the tile's last token, request, first token): the attention kernel starts (or
-        # pairs) tiles by the work they are; and the requests with one new token.
-        several = np.flatnonzero(count > 1)
-        dec = np.flatnonzero(count == 1).astype(np.int32)
-        if several.size:
-            per = (count[several] + PREFILL_TILE - 1) // PREFILL_TILE
-            tile_b = np.repeat(several, per).astype(np.int32)
-            first = np.cumsum(per) - per
-            tile_q0 = ((np.arange(int(per.sum())) - np.repeat(first, per)) * PREFILL_TILE).astype(np.int32)
-            keys = start[tile_b] + np.minimum(count[tile_b], tile_q0 + PREFILL_TILE)
-            order = np.lexsort((tile_q0, tile_b, keys))
-            tile_seq, tile_q0, keys = tile_b[order], tile_q0[order], keys[order]
-            tile_keys = (int(keys[0]), int(keys[-1]))
-        else:
-            tile_seq = tile_q0 = np.zeros(0, dtype=np.int32)
-            tile_keys = (0, 0)
-        max_ctx_dec = int(ctx_len[dec].max()) if dec.size else 0
-
-        sections = [tokens, positions, q_start, ctx_len, slots, rows, tile_seq, tile_q0, dec]
-        group_meta = []
+        names = ["token_ids", "positions", "q_start", "ctx_len", "state_slots", "logit_rows"]
+        sizes = [T, T, B + 1, B, B, int(rows.size)]
+        widths = []
         for g, gc in enumerate(self.cache.groups):
-            ps = gc.page_size
-            width = max(1, -(-int(ctx_len.max()) // ps))
-            bt = np.empty((B, width), dtype=np.int32)
-            slot_map = np.empty(T, dtype=np.int32)
+            width = max(1, -(-ctx_bound // gc.page_size))
+            widths.append(width)
+            names += [("slot_mapping", g), ("block_table", g)]
+            sizes += [T, B * width]
+        plan_arrays = []
+        for key, (arrays, _) in plans.items():
+            for name, arr in arrays.items():
+                if arr.dtype != np.int32 or arr.ndim != 1:
+                    raise StepError(f"planner {key}: array {name!r} must be one-dimensional int32")
+                names.append(("plan", key, name))
+                sizes.append(int(arr.size))
+                plan_arrays.append(arr)
+        offsets, total = [], 0
+        for size in sizes:
+            offsets.append(total)
+            total += _align4(size)
+        total = max(total, 4)
+        host = host_for(total) if host_for is not None else np.zeros(total, dtype=np.int32)
+        if host.size != total:
+            raise StepError(f"the step's tables take {total} words, the buffer for them has {host.size}")
+
+        def sec(i: int) -> np.ndarray:
+            return host[offsets[i]:offsets[i] + sizes[i]]
+
+        sec(0)[:] = tokens
+        sec(1)[:] = positions
+        sec(2)[:] = q_start
+        sec(3)[:] = ctx_len
+        slots = sec(4)
+        # padded rows keep their hands off every request's state: the spare slot past the last one
+        slots[n:] = self.cache.num_state_slots
+        sec(5)[:] = rows
+        for g, gc in enumerate(self.cache.groups):
+            slot_map, bt = sec(6 + 2 * g), sec(7 + 2 * g).reshape(B, widths[g])
             try:
-                self.cache.step_tables(ids, start, count, g, bt, slot_map, slots if g == 0 else None)
+                if fixed is None:
+                    self.cache.step_tables(ids, start, count, g, bt, slot_map, slots if g == 0 else None)
+                elif n:
+                    ps = gc.page_size
+                    self.cache.export(ids, g, bt[:n], slots[:n] if g == 0 else None)
+                    at = positions[:n]
+                    slot_map[:n] = bt[np.arange(n), at // ps] * ps + at % ps
             except CacheError as err:
                 raise StepError(str(err)) from None
-            sections += [slot_map, bt.reshape(-1)]
-            group_meta.append((ps, width, gc.window))
+            if fixed is not None:
+                slot_map[n:] = -1
+        for i, arr in enumerate(plan_arrays):
+            sec(len(sizes) - len(plan_arrays) + i)[:] = arr
+        return StepTables(host=host, names=names, sizes=sizes, offsets=offsets, T=T, B=B, R=int(rows.size),
+                          widths=widths, plan_meta={key: meta for key, (_, meta) in plans.items()},
+                          q_start_host=q_start.tolist(), ctx_len_host=ctx_len.tolist(),
+                          state_slots_host=slots.tolist(), fixed=fixed)
 
-        offsets, total = [], 0
-        for s in sections:
-            offsets.append(total)
-            total += _align4(s.size)
-        host = np.zeros(max(total, 4), dtype=np.int32)
-        for s, o in zip(sections, offsets):
-            host[o:o + s.size] = s
-        dev = torch.from_numpy(host).to(self.device)
+    def context(self, tables: StepTables, dev: torch.Tensor, workspace: Optional[dict] = None) -> StepContext:
+        """The step as the parts see it, over ``dev``: the tables' words on the device."""
+        B = tables.B
 
         def view(i: int) -> torch.Tensor:
-            return dev[offsets[i]:offsets[i] + sections[i].size]
+            return dev[tables.offsets[i]:tables.offsets[i] + tables.sizes[i]]
 
         groups = []
-        for g, (ps, width, window) in enumerate(group_meta):
-            groups.append(GroupView(page_size=ps, block_tables=view(10 + 2 * g).view(B, width),
-                                    slot_mapping=view(9 + 2 * g), max_blocks=width, window=window))
+        for g, gc in enumerate(self.cache.groups):
+            groups.append(GroupView(page_size=gc.page_size, block_tables=view(7 + 2 * g).view(B, tables.widths[g]),
+                                    slot_mapping=view(6 + 2 * g), max_blocks=tables.widths[g], window=gc.window))
+        plans = {key: StepPlan({}, meta) for key, meta in tables.plan_meta.items()}
+        for i, name in enumerate(tables.names):
+            if isinstance(name, tuple) and name[0] == "plan":
+                plans[name[1]].arrays[name[2]] = view(i)
         return StepContext(
-            device=self.device, dtype=self.dtype, T=T, B=B, token_ids=view(0), positions=view(1), q_start=view(2),
-            ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=int(rows.size), groups=groups,
-            tile_seq=view(6), tile_q0=view(7), n_tiles=int(tile_seq.size), tile_keys=tile_keys,
-            dec_seqs=view(8) if dec.size else None,
-            n_dec=int(dec.size), max_ctx_dec=max_ctx_dec, q_start_host=q_start.tolist(), ctx_len_host=ctx_len.tolist(),
-            state_slots_host=slots.tolist(), workspace=self.workspace)
+            device=self.device, dtype=self.dtype, T=tables.T, B=B, token_ids=view(0), positions=view(1),
+            q_start=view(2), ctx_len=view(3), state_slots=view(4), logit_rows=view(5), R=tables.R, groups=groups,
+            plans=plans, q_start_host=tables.q_start_host, ctx_len_host=tables.ctx_len_host,
+            state_slots_host=tables.state_slots_host, workspace=self.workspace if workspace is None else workspace,
+            fixed=tables.fixed)
+
+    def build_context_arrays(self, ids, start, count, tokens, rows) -> StepContext:
+        """The eager step's context: tables written into pinned memory and read
+        from there by one small kernel (see ``step_tables`` for the arguments)."""
+        tables = self.step_tables(ids, start, count, tokens, rows, host_for=lambda n: self._ring.take(n).numpy())
+        dev = torch.empty(tables.host.size, dtype=torch.int32, device=self.device)
+        ops.table_load(self._ring.buffers[self._ring.turn], dev)
+        self._ring.sent()
+        return self.context(tables, dev)
 
     def layer_caches(self, ctx: StepContext) -> list:
         return [LayerCache(group=ctx.groups[g] if g is not None else None, k=k, v=v, state=state, writes=writes)
@@ -182,6 +307,6 @@ class ModelRunner:
         return self.model.forward(ctx, self.layer_caches(ctx))
 
     def step_arrays(self, ids, start, count, tokens, rows) -> Optional[torch.Tensor]:
-        """``step`` from numpy arrays (see ``build_context_arrays``)."""
+        """``step`` from numpy arrays (see ``step_tables``)."""
         ctx = self.build_context_arrays(ids, start, count, tokens, rows)
         return self.model.forward(ctx, self.layer_caches(ctx))

@@ -748,13 +748,13 @@ def _pinned(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
 
 
 def table_load(src: torch.Tensor, dst: torch.Tensor, patch: torch.Tensor | None = None, patch_at: int = 0) -> None:
-    """dst (int32, device) = src (int32, pinned host memory, read by the kernel
-    itself: no copy engine, no second launch); ``patch`` (int32, device)
-    replaces the words from ``patch_at`` on."""
+    """dst (int32, device) = the first dst.numel() words of src (int32, pinned
+    host memory, read by the kernel itself: no copy engine, no second launch);
+    ``patch`` (int32, device) replaces the words from ``patch_at`` on."""
     _pinned(src, torch.int32, "table_load: the source")
     _dev(dst, patch)
-    if dst.dtype != torch.int32 or dst.numel() != src.numel() or not dst.is_contiguous():
-        raise KernelError("table_load: the destination must be a contiguous int32 tensor as long as the source")
+    if dst.dtype != torch.int32 or dst.numel() > src.numel() or not dst.is_contiguous():
+        raise KernelError("table_load: the destination must be a contiguous int32 tensor no longer than the source")
     n_patch = 0
     if patch is not None:
         n_patch = patch.numel()

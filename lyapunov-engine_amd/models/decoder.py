@@ -20,7 +20,8 @@ import torch
 from ..config.registry import BLOCKS, NORMS
 from ..config.specs import LayerCall, ModelSpec
 from ..kernels import ops
-from ..parts.base import KVCacheSpec, LayerCache, Part, StateSpec, StepContext, WeightSource, WeightSpec
+from ..parts.base import (KVCacheSpec, LayerCache, Part, PositionEncoding, StateSpec, StepContext, WeightSource,
+                          WeightSpec)
 
 
 @dataclass(frozen=True)
@@ -54,6 +55,7 @@ class DecoderModel(Part):
         self.lm_head: Optional[torch.Tensor] = None
         self.device: Optional[torch.device] = None
         self.dtype: Optional[torch.dtype] = None
+        self.max_positions = spec.max_position      # positions a step may reach; ``materialize`` may lower it
         self._layout = self._plan_cache()
 
     # -------------------------------------------------------------- structure
@@ -130,8 +132,16 @@ class DecoderModel(Part):
         return self._layout
 
     # ---------------------------------------------------------------- weights
-    def materialize(self, device, dtype):
+    def materialize(self, device, dtype, max_positions: Optional[int] = None):
+        """Build what is computed rather than loaded.  ``max_positions``: the
+        engine will never hold a request longer than this (its model length, its
+        pool), so position tables need no more rows."""
         self.device, self.dtype = torch.device(device), dtype
+        if max_positions is not None:
+            self.max_positions = max(1, min(self.spec.max_position, int(max_positions)))
+            for _, part in self.named_parts():
+                if isinstance(part, PositionEncoding):
+                    part.limit_positions(self.max_positions)
         for layer in self.layers:
             layer.materialize(self.device, dtype)
         self.final_norm.materialize(self.device, dtype)

@@ -17,12 +17,60 @@ from __future__ import annotations
 import math
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..config.specs import PartSpec
 from ..kernels import ops
-from .base import KVCacheSpec, LayerCache, Mixer, StepContext, WeightSource, WeightSpec
+from .base import KVCacheSpec, LayerCache, Mixer, StepBatch, StepContext, StepPlanner, WeightSource, WeightSpec
+
+PREFILL_TILE = 64   # new tokens of one request per workgroup of the prefill attention kernel
+
+
+class AttentionWork(StepPlanner):
+    """The attention kernels' work lists for a step.  Requests that bring
+    several tokens are cut into tiles of PREFILL_TILE tokens, sorted by (keys up
+    to the tile's last token, request, first token): the prefill kernel starts
+    (or pairs) tiles by the work they are.  Requests that bring one token go to
+    the split kernel.
+
+    arrays: ``tile_seq``, ``tile_q0`` (request and first token of every tile),
+    ``dec`` (the one-token requests; absent when there are none, and in a fixed
+    step, where every row is one).  meta: ``n_tiles``, ``tile_keys`` (keys seen
+    by the first and by the last tile), ``n_dec``, ``max_ctx_dec`` (the longest
+    context among the one-token requests; in a fixed step the step's bound)."""
+
+    key = ("paged_attention_work", PREFILL_TILE)
+
+    def plan(self, batch: StepBatch) -> tuple:
+        none = np.zeros(0, dtype=np.int32)
+        if batch.fixed is not None:
+            return ({"tile_seq": none, "tile_q0": none},
+                    dict(n_tiles=0, tile_keys=(0, 0), n_dec=batch.fixed.rows, max_ctx_dec=batch.fixed.max_context))
+        start, count, ctx_len = batch.start, batch.count, batch.ctx_len
+        several = np.flatnonzero(count > 1)
+        dec = np.flatnonzero(count == 1).astype(np.int32)
+        if several.size:
+            per = (count[several] + PREFILL_TILE - 1) // PREFILL_TILE
+            tile_b = np.repeat(several, per).astype(np.int32)
+            first = np.cumsum(per) - per
+            tile_q0 = ((np.arange(int(per.sum())) - np.repeat(first, per)) * PREFILL_TILE).astype(np.int32)
+            keys = start[tile_b] + np.minimum(count[tile_b], tile_q0 + PREFILL_TILE)
+            order = np.lexsort((tile_q0, tile_b, keys))
+            tile_seq, tile_q0, keys = tile_b[order], tile_q0[order], keys[order]
+            tile_keys = (int(keys[0]), int(keys[-1]))
+        else:
+            tile_seq = tile_q0 = none
+            tile_keys = (0, 0)
+        arrays = {"tile_seq": tile_seq, "tile_q0": tile_q0}
+        if dec.size:
+            arrays["dec"] = dec
+        return arrays, dict(n_tiles=int(tile_seq.size), tile_keys=tile_keys, n_dec=int(dec.size),
+                            max_ctx_dec=int(ctx_len[dec].max()) if dec.size else 0)
+
+
+_WORK = AttentionWork()
 
 
 @MIXERS.register("paged_attention")
@@ -60,6 +108,9 @@ class PagedAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    def step_planner(self):
+        return _WORK
+
     takes_pending_norm = True   # x may be an ops.PendingNorm: the q/k/v product norms on its way in
 
     def forward(self, ctx: StepContext, x, cache: LayerCache):
@@ -73,27 +124,29 @@ class PagedAttention(Mixer):
         out = torch.empty((ctx.T, self.num_heads * self.head_dim), dtype=ctx.dtype, device=qkv.device)
         common = dict(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                       window=self.window, scale=self.scale)
-        if ctx.n_tiles:
+        work = ctx.plans[AttentionWork.key]
+        n_tiles, n_dec, max_ctx_dec = work.meta["n_tiles"], work.meta["n_dec"], work.meta["max_ctx_dec"]
+        if n_tiles:
             # Tiles come in rising order of the keys they see; when the first sees less than half
             # of what the last does, a workgroup may take one from each end.
-            few, many = (min(k, self.window + 64) if self.window else k for k in ctx.tile_keys)
+            few, many = (min(k, self.window + 64) if self.window else k for k in work.meta["tile_keys"])
             # few new tokens over many keys: the keys in runs, for workgroups of their own
-            parts = ops.attn_prefill_plan(ctx.n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim,
+            parts = ops.attn_prefill_plan(n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim,
                                           ctx.dtype, g.page_size)
             part_o = part_ml = None
             if parts > 1:
-                n = ctx.n_tiles * 64 * self.num_heads * parts
+                n = n_tiles * PREFILL_TILE * self.num_heads * parts
                 part_o = ctx.scratch("attn_part_o", n * self.head_dim)
                 part_ml = ctx.scratch("attn_part_ml", n * 2)
-            ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.tile_seq,
-                             ctx.tile_q0, ctx.n_tiles, pair=2 * few <= many, parts=parts, part_o=part_o,
-                             part_ml=part_ml, **common)
-        if ctx.n_dec:
-            part = ops.attn_decode_plan(ctx.n_dec, ctx.max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
-            max_parts = max(1, (ctx.max_ctx_dec + part - 1) // part)
-            n = ctx.n_dec * self.num_heads * max_parts
+            ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len,
+                             work.arrays["tile_seq"], work.arrays["tile_q0"], n_tiles, pair=2 * few <= many,
+                             parts=parts, part_o=part_o, part_ml=part_ml, **common)
+        if n_dec:
+            part = ops.attn_decode_plan(n_dec, max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
+            max_parts = max(1, (max_ctx_dec + part - 1) // part)
+            n = n_dec * self.num_heads * max_parts
             part_o = ctx.scratch("attn_part_o", n * self.head_dim)
             part_ml = ctx.scratch("attn_part_ml", n * 2)
-            ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len, ctx.dec_seqs,
-                            ctx.n_dec, part_o, part_ml, max_parts, part, **common)
+            ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len,
+                            work.arrays.get("dec"), n_dec, part_o, part_ml, max_parts, part, **common)
         return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True, pending=True)

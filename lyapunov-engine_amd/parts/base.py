@@ -24,6 +24,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
+import numpy as np
 import torch
 
 
@@ -54,8 +55,10 @@ class Part:
     """Anything that may own weights and sub-parts."""
 
     # False for a part whose forward reads the host copies of the step's tables
-    # (``ctx.q_start_host`` and the like): such a forward cannot be captured in
-    # a graph and replayed with other tables, so its model steps eagerly.
+    # (``ctx.q_start_host`` and the like) or lets the device's values decide
+    # what is launched: such a forward cannot be recorded once and replayed with
+    # other tables, so its model steps eagerly.  A part that needs lists of its
+    # own on the device gets them through ``step_planner`` and stays graph-safe.
     graph_safe = True
 
     def weight_specs(self) -> list:
@@ -70,6 +73,11 @@ class Part:
         """Build device tables that are computed rather than loaded."""
         for c in self.children().values():
             c.materialize(device, dtype)
+
+    def step_planner(self) -> Optional["StepPlanner"]:
+        """What this part wants worked out once per step, on the host, from the
+        step's requests (see ``StepPlanner``); None: nothing."""
+        return None
 
 
 # ----------------------------------------------------------------------- cache
@@ -115,6 +123,57 @@ class LayerCache:
 
 
 @dataclass
+class FixedStep:
+    """A step whose shapes are frozen so that it can be recorded once and
+    replayed: ``rows`` requests of one new token each (rows past the live ones
+    are padding: context 0, cache slot -1, the spare state slot), contexts of
+    at most ``max_context`` tokens."""
+
+    rows: int
+    max_context: int
+
+
+@dataclass
+class StepBatch:
+    """The requests of a step as the host sees them (numpy), for planners."""
+
+    start: np.ndarray                     # int32 [B]: position of each request's first new token
+    count: np.ndarray                     # int32 [B]: how many new tokens it brings
+    q_start: np.ndarray                   # int32 [B + 1]: offsets into the flat batch
+    ctx_len: np.ndarray                   # int32 [B]: length after the step (0: a padded row of a fixed step)
+    T: int
+    B: int
+    fixed: Optional[FixedStep] = None
+
+
+class StepPlanner:
+    """Host work a part wants done once per step: from the step's requests to
+    the lists its kernels walk (tiles, queues, segment tables).  The step
+    function calls ``plan`` once per step and distinct ``key`` (parts whose
+    planners have equal keys share one plan), sends the arrays to the device in
+    the step's one upload, and hands the part a ``StepPlan`` under
+    ``ctx.plans[key]``.
+
+    For a fixed step (``batch.fixed``) the sizes of the arrays and every value
+    of ``meta`` may depend on ``batch.fixed`` alone, never on the live
+    requests: the kernels' launch shapes are recorded once; the arrays'
+    contents are written afresh before every replay."""
+
+    key: tuple = ()
+
+    def plan(self, batch: StepBatch) -> tuple:
+        """-> (arrays, meta): int32 numpy arrays by name, and host values
+        (launch shapes, counts) by name."""
+        raise NotImplementedError
+
+
+@dataclass
+class StepPlan:
+    arrays: dict                          # name -> int32 tensor on the device
+    meta: dict                            # name -> host value
+
+
+@dataclass
 class StepContext:
     """Everything about the batch of one step, on the device and on the host."""
 
@@ -130,20 +189,13 @@ class StepContext:
     logit_rows: torch.Tensor              # int32 [R] rows of the flat batch whose logits are wanted
     R: int
     groups: list                          # of GroupView
-    # attention work lists: requests with more than one new token are cut into
-    # tiles of 64 tokens, requests with exactly one go to the split kernel
-    tile_seq: torch.Tensor
-    tile_q0: torch.Tensor
-    n_tiles: int
-    dec_seqs: Optional[torch.Tensor]
-    n_dec: int
-    max_ctx_dec: int                      # longest context among the single-token requests
-    # host copies for parts written in Python
+    plans: dict = field(default_factory=dict)       # StepPlanner.key -> StepPlan
+    # host copies for parts written in Python (a part that reads them is not graph_safe)
     q_start_host: list = field(default_factory=list)
     ctx_len_host: list = field(default_factory=list)
     state_slots_host: list = field(default_factory=list)
     workspace: dict = field(default_factory=dict)   # scratch tensors shared by the layers of a step
-    tile_keys: tuple = (0, 0)             # keys up to the last token of the first and of the last tile
+    fixed: Optional[FixedStep] = None     # set while a fixed step is recorded or replayed
 
     def scratch(self, key: str, numel: int, dtype: torch.dtype = torch.float32) -> torch.Tensor:
         t = self.workspace.get(key)
@@ -176,6 +228,10 @@ class PositionEncoding(Part):
 
     table: Optional[torch.Tensor] = None
     rotary_dim: int = 0
+
+    def limit_positions(self, n: int) -> None:
+        """Called before ``materialize`` when the engine will never reach
+        position ``n``: tables need no more rows than that."""
 
 
 class Mixer(Part):
@@ -218,5 +274,6 @@ class Block(Part):
 
 __all__ = [
     "WeightSource", "WeightSpec", "Part", "KVCacheSpec", "StateSpec", "GroupView", "LayerCache", "StepContext",
+    "StepBatch", "StepPlan", "StepPlanner", "FixedStep",
     "Norm", "PositionEncoding", "Mixer", "FeedForward", "Block", "Any",
 ]

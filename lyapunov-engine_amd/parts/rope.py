@@ -17,6 +17,7 @@ s = (L/wavelength - low) / (high - low): (1 - s) * inv_freq/factor + s * inv_fre
 from __future__ import annotations
 
 import math
+import weakref
 from typing import Optional
 
 import torch
@@ -43,6 +44,12 @@ def rotary_inv_freq(dim: int, theta: float, scaling: Optional[dict] = None) -> t
     return torch.where(medium, blended, scaled)
 
 
+# Tables in use, by what fixes their contents: parts with equal parameters (the
+# layers of a model, as a rule) share one tensor.  A table goes when the last
+# part that uses it does.
+_TABLES: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
+
+
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
     def __init__(self, dim: int, theta: float, max_position: int, scaling: Optional[dict] = None):
@@ -51,16 +58,26 @@ class RotaryEncoding(PositionEncoding):
         self.rotary_dim = dim
         self.theta = float(theta)
         self.max_position = max_position
+        self.positions = max_position      # rows of the table: max_position, or fewer (``limit_positions``)
         self.scaling = scaling
         self.table: Optional[torch.Tensor] = None
 
+    def limit_positions(self, n: int) -> None:
+        self.positions = max(1, min(self.max_position, int(n)))
+
     def build_table(self) -> torch.Tensor:
         inv_freq = rotary_inv_freq(self.rotary_dim, self.theta, self.scaling)
-        angles = torch.outer(torch.arange(self.max_position, dtype=torch.float32), inv_freq)
+        angles = torch.outer(torch.arange(self.positions, dtype=torch.float32), inv_freq)
         return torch.cat((angles.cos(), angles.sin()), dim=-1).contiguous()
 
     def materialize(self, device, dtype):
-        self.table = self.build_table().to(device)
+        scaling = tuple(sorted(self.scaling.items())) if self.scaling else None
+        key = (self.rotary_dim, self.theta, scaling, self.positions, str(torch.device(device)))
+        table = _TABLES.get(key)
+        if table is None:
+            table = self.build_table().to(device)
+            _TABLES[key] = table
+        self.table = table
 
 
 @POSITION_ENCODINGS.register("none")

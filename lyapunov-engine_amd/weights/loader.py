@@ -92,7 +92,8 @@ def kept_dtype(stored: torch.dtype, engine_dtype: torch.dtype) -> torch.dtype:
     return torch.bfloat16
 
 
-def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, device) -> DecoderModel:
+def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, device,
+                 max_positions: Optional[int] = None) -> DecoderModel:
     check_tensors(model, source.shapes())
     expected = model.expected_tensors()
     for name in sorted(n for n in source.shapes() if n not in expected):
@@ -112,14 +113,16 @@ def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, 
                 raise WeightError(f"{ws.attr}: rows of {[tuple(p.shape) for p in pieces]} cannot alternate in runs of {n}")
             t = t.view(k, rows // n, n, *t.shape[1:]).transpose(0, 1).reshape(t.shape)
         setattr(owner, ws.attr, t.contiguous())
-    model.materialize(device, dtype)
+    model.materialize(device, dtype, max_positions)
     return model
 
 
-def load_model(model_dir: str, dtype: torch.dtype, device="cuda:0", source: Optional[TensorSource] = None):
+def load_model(model_dir: str, dtype: torch.dtype, device="cuda:0", source: Optional[TensorSource] = None,
+               max_positions: Optional[int] = None):
     """config.json -> architecture -> model, with its tensors from the folder's
-    safetensors files.  Returns (model, typed configuration)."""
+    safetensors files.  Returns (model, typed configuration).  ``max_positions``:
+    see ``DecoderModel.materialize``."""
     arch, cfg = load_config(model_dir)
     model = build_model(arch.to_spec(cfg))
-    load_weights(model, source or FolderSource(model_dir), dtype, device)
+    load_weights(model, source or FolderSource(model_dir), dtype, device, max_positions)
     return model, cfg

@@ -157,3 +157,34 @@ def test_engine_config_names_follow_the_reference():
         EngineConfig(dtype="float16")
     with pytest.raises(ValueError):
         EngineConfig(block_size=0)
+
+
+def test_layers_with_equal_position_parameters_share_one_table():
+    """A model of the 1B shape's depth with 131,072 positions holds one table of cosines and sines
+    (131,072 x 64 floats = 32 MiB), not one per layer; an engine that will never reach beyond 4,096
+    positions builds 4,096 rows."""
+    import torch
+
+    from lyapunov_engine_amd.models import build_model
+    from lyapunov_engine_amd.models.llama import llama_spec
+
+    raw = dict(architectures=["LlamaForCausalLM"], vocab_size=64, hidden_size=128, intermediate_size=64,
+               num_hidden_layers=16, num_attention_heads=2, num_key_value_heads=1, head_dim=64,
+               max_position_embeddings=131072, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    model = build_model(llama_spec(LlamaConfig.from_dict(raw)))
+    model.materialize("cpu", torch.float32)
+    tables = [layer.mixer.position.table for layer in model.layers]
+    assert len({t.data_ptr() for t in tables}) == 1 and all(t is tables[0] for t in tables)
+    assert tables[0].shape == (131072, 64) and tables[0].numel() * 4 == 32 << 20
+    assert model.max_positions == 131072
+
+    small = build_model(llama_spec(LlamaConfig.from_dict(raw)))
+    small.materialize("cpu", torch.float32, max_positions=4096)
+    assert small.layers[0].mixer.position.table.shape == (4096, 64) and small.max_positions == 4096
+    torch.testing.assert_close(small.layers[0].mixer.position.table, tables[0][:4096], rtol=0, atol=0)
+    # other parameters, another table
+    other = build_model(llama_spec(LlamaConfig.from_dict(dict(raw, rope_theta=10000.0, max_position_embeddings=4096))))
+    other.materialize("cpu", torch.float32)
+    assert other.layers[0].mixer.position.table.data_ptr() != small.layers[0].mixer.position.table.data_ptr()

@@ -184,7 +184,7 @@ def test_a_step_that_does_not_fit_the_cache_is_refused(model_folders):
         with pytest.raises(StepError, match=words):
             core.step(entries)
     core.cache.extend(0, 300)
-    with pytest.raises(StepError, match="beyond the model's 256"):
+    with pytest.raises(StepError, match="beyond the 256 positions"):
         core.step([StepEntry(0, [1] * 257, 0, [])])
     logits = core.step([StepEntry(0, [1, 2, 3], 0, [2])])       # and what fits still runs
     assert tuple(logits.shape) == (1, 256) and bool(torch.isfinite(logits).all())
@@ -325,3 +325,38 @@ def test_command_line_generate(model_folders):
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert "--- Output Generation ---" in proc.stdout
     assert proc.stdout.strip().splitlines()[-1].split() == [str(t) for t in want]
+
+
+def test_a_step_ahead_that_cannot_start_does_not_break_the_planned_step(model_folders, capsys):
+    """Starting the next step early is optional work: if it raises (a new graph that cannot be
+    recorded, no memory for it), the planned step's tokens still reach the scheduler, looking ahead
+    is switched off with a note, and generation gives the tokens it gives without looking ahead."""
+    from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.llm_engine import LLMEngine
+    from lyapunov_engine_amd.sampling.params import SamplingParams
+
+    folder = model_folders["B"]["float32"]
+    prompts = [random_tokens(n, 515, seed=70 + n) for n in (12, 5)]
+    params = SamplingParams(temperature=0.0, max_tokens=15, ignore_eos=True)
+
+    def run(lookahead, break_it):
+        engine = LLMEngine(folder, EngineConfig(dtype="float32", num_blocks=24, block_size=16, max_num_seqs=4,
+                                                lookahead=lookahead))
+        if break_it:
+            real = engine.graphs.step_arrays
+
+            def failing(ids, starts, tokens, tokens_dev=None):
+                if tokens_dev is not None:
+                    raise RuntimeError("no memory for a new graph")
+                return real(ids, starts, tokens)
+
+            engine.graphs.step_arrays = failing
+        outs = engine.generate(prompts, params)
+        engine.core.cache.check()
+        assert engine.core.cache.num_requests() == 0 and engine.core.cache.num_free_pages() == 24
+        return [o.output_tokens for o in outs], engine
+
+    want, _ = run(False, False)
+    got, engine = run(True, True)
+    assert got == want and engine._look_ahead is False and engine.steps_taken_ahead == 0
+    assert "looking ahead switched off" in capsys.readouterr().err

@@ -454,3 +454,159 @@ def test_routed_feed_forward_and_another_position_encoding(tmp_path, dtype):
         ARCHITECTURES.unregister("ToyRoutedForCausalLM")
         FEED_FORWARDS.unregister("toy_routed_experts")
         POSITION_ENCODINGS.unregister("toy_linear_angles")
+
+
+# ----------------------- a third toy: a mixer with state, lists of its own, and graphs
+TOY3 = dict(architectures=["ToyScanForCausalLM"], vocab_size=100, hidden_size=64, intermediate_size=96, state_size=32,
+            num_heads=2, num_kv_heads=1, head_dim=32, max_position=200, eps=1e-5, theta=10000.0, decay=0.7)
+
+
+def register_toy3():
+    """A recurrence that never looks at the host's copy of the batch: what it needs to know about
+    the step's requests it asks for through a planner of its own, as device lists, and so its
+    decode steps can be recorded once and replayed."""
+    from lyapunov_engine_amd.config import MIXERS, LayerSpec, ModelSpec, PartSpec, default_schedule, register_architecture
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.parts import Mixer, StateSpec, StepPlanner, WeightSource, WeightSpec
+
+    class Segments(StepPlanner):
+        """Per request: 1 if it starts from nothing.  meta: the most tokens any request brings
+        (the number of rounds the scan takes; 1 in a fixed step)."""
+        key = ("toy_segments",)
+
+        def plan(self, batch):
+            fresh = (batch.ctx_len - batch.count == 0).astype(np.int32)
+            longest = 1 if batch.fixed is not None else int(batch.count.max())
+            return {"fresh": fresh}, {"longest": longest}
+
+    class ScanOnDevice(Mixer):
+        """s_t = decay * s_{t-1} + W_in x_t ;  y_t = W_out s_t, one round per token position within
+        the requests, all requests at once."""
+
+        def __init__(self, hidden_size, state_size, decay):
+            self.hidden_size, self.state_size, self.decay = hidden_size, state_size, decay
+            self.in_proj = self.out_proj = None
+
+        def weight_specs(self):
+            return [WeightSpec("in_proj", (WeightSource("in_proj.weight", (self.state_size, self.hidden_size)),)),
+                    WeightSpec("out_proj", (WeightSource("out_proj.weight", (self.hidden_size, self.state_size)),))]
+
+        def state_spec(self):
+            return StateSpec((self.state_size,), torch.float32)
+
+        def step_planner(self):
+            return Segments()
+
+        def forward(self, ctx, x, cache):
+            plan = ctx.plans[Segments.key]
+            u = ops.linear(x, self.in_proj, out_dtype=torch.float32)                  # [T, S]
+            slots = ctx.state_slots.long()
+            first = ctx.q_start[:-1].long()
+            count = (ctx.q_start[1:] - ctx.q_start[:-1]).long()
+            keep = (1 - plan.arrays["fresh"]).float()[:, None]
+            s = cache.state.index_select(0, slots) * keep                               # [B, S]
+            out = torch.zeros((ctx.T + 1, self.state_size), dtype=torch.float32, device=x.device)
+            for j in range(plan.meta["longest"]):
+                live = (count > j)
+                at = torch.where(live, first + j, torch.full_like(first, ctx.T))       # done requests write row T
+                s = torch.where(live[:, None], self.decay * s + u.index_select(0, at.clamp(max=ctx.T - 1)), s)
+                out.index_copy_(0, at, s)
+            cache.state.index_copy_(0, slots, s)      # padded rows all write the spare slot
+            return ops.linear(ops.cast(out[:ctx.T].contiguous(), ctx.dtype), self.out_proj, out_dtype=ctx.dtype)
+
+    MIXERS.register("toy_scan_on_device", ScanOnDevice, replace=True)
+
+    def to_spec(cfg: ToyConfig) -> ModelSpec:
+        c = dict(cfg.raw)
+        H = c["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": c["eps"]})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
+        rope = PartSpec("rope", {"dim": c["head_dim"], "theta": c["theta"], "max_position": c["max_position"]})
+        attn = PartSpec("paged_attention", dict(hidden_size=H, num_heads=c["num_heads"], num_kv_heads=c["num_kv_heads"],
+                                                head_dim=c["head_dim"], position=rope))
+        scan = PartSpec("toy_scan_on_device", {"hidden_size": H, "state_size": c["state_size"], "decay": c["decay"]})
+        layers = (LayerSpec("prenorm", attn, ffn, norm, norm), LayerSpec("prenorm", scan, ffn, norm, norm))
+        return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=default_schedule(2),
+                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"])
+
+    register_architecture("ToyScanForCausalLM", ToyConfig, to_spec, replace=True)
+
+
+def toy3_plain(folder, tokens):
+    from safetensors.torch import load_file
+
+    c = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    S, nh, nkv, hd = len(tokens), c["num_heads"], c["num_kv_heads"], c["head_dim"]
+    pos = torch.arange(S)
+    cos, sin = P.rope_cos_sin(pos, P.rope_inv_freq(hd, c["theta"]))
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    for layer in range(2):
+        p = f"model.layers.{layer}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
+        if layer == 0:
+            q = P.apply_rope((x @ w[p + "self_attn.q_proj.weight"].T).view(S, nh, hd).transpose(0, 1), cos, sin)
+            k = P.apply_rope((x @ w[p + "self_attn.k_proj.weight"].T).view(S, nkv, hd).transpose(0, 1), cos, sin)
+            v = (x @ w[p + "self_attn.v_proj.weight"].T).view(S, nkv, hd).transpose(0, 1)
+            a = P.attention(q, k, v, pos, pos).transpose(0, 1).reshape(S, nh * hd) @ w[p + "self_attn.o_proj.weight"].T
+        else:
+            u = x @ w[p + "self_attn.in_proj.weight"].T
+            s, out = torch.zeros(c["state_size"], dtype=torch.float64), []
+            for t in range(S):
+                s = c["decay"] * s + u[t]
+                out.append(s)
+            a = torch.stack(out) @ w[p + "self_attn.out_proj.weight"].T
+        h = h + a
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
+        h = h + P.mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_stateful_mixer_with_lists_of_its_own_decodes_through_graphs(tmp_path, dtype):
+    """Registered from here, with a planner of its own: the step function uploads its list with the
+    step's tables, the recorded decode step replays with it, padded rows touch no request's state.
+    Replay against the plain model; generation with graphs against generation without (three
+    requests that start and end at different steps, so the batch and its padding change while the
+    graphs are replayed), and in 32-bit against the plain model's greedy tokens."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.config import ARCHITECTURES, MIXERS
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import compare
+
+    register_toy3()
+    try:
+        folder = str(tmp_path / "toy3")
+        write_random_model(dict(TOY3), folder, seed=4, dtype=dtype, init_std=0.15, norm_init_std=0.1)
+        reqs = {"x": random_tokens(45, 100, seed=7), "y": random_tokens(18, 100, seed=8)}
+        want = {k: toy3_plain(folder, v) for k, v in reqs.items()}
+        cut = Trace(reqs)
+        cut.step([("x", 9), ("y", 3)])
+        cut.step([("x", 2), ("y", 15)], end=["y"])
+        for _ in range(10):
+            cut.step([("x", 1)])
+        cut.step([("x", 24)], end=["x"])
+        compare(cut, replay(folder, dtype, cut), want, dtype, "scan cut")
+
+        prompts = [reqs["x"][:12], reqs["y"][:5], reqs["x"][20:27]]
+        lengths = [30, 12, 21]
+
+        def run(graphs):
+            llm = L.LLM(folder, dtype=dtype, num_blocks=64, block_size=4, max_num_seqs=4, enable_graphs=graphs)
+            params = [L.SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in lengths]
+            outs = llm.generate(prompts, params)
+            return [o.output_tokens for o in outs], llm.engine
+
+        with_graphs, engine = run(True)
+        assert engine.graphs.safe and engine.graphs.captured, "the toy's decode steps were meant to be recorded"
+        assert {key[0] for key in engine.graphs.captured} >= {1, 2, 3}       # batches of 3, 2 and 1 as requests end
+        eager, _ = run(False)
+        assert with_graphs == eager
+        if dtype == "float32":
+            toks = list(prompts[0])
+            for t in with_graphs[0]:
+                assert t == int(toy3_plain(folder, toks)[-1].argmax())
+                toks.append(t)
+    finally:
+        ARCHITECTURES.unregister("ToyScanForCausalLM")
+        MIXERS.unregister("toy_scan_on_device")
