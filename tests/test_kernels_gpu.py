@@ -613,6 +613,171 @@ def test_attention_at_the_edge_of_the_window(ops, dtype, kind, window):
         assert (want[i] - v_in).abs().max() < 0.5 * (want[i] - v_out).abs().max()
 
 
+# ------------------------------------------------ attention at long contexts
+def paged_setup_long(seqs, nh, nkv, hd, bs, dtype, seed=0, q_scale=4.0):
+    """``paged_setup`` for contexts of thousands of tokens: built on the device, whole pages at a
+    time.  Queries are scaled so that the softmax is peaked (a handful of keys among thousands carry
+    a row's weight): a run or a partition of keys that is dropped, read twice or merged wrongly
+    then moves the result far beyond the tolerance, which a flat softmax would not."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    cpu_g = torch.Generator().manual_seed(seed)
+    need = sum(-(-c // bs) for c, _ in seqs)
+    n_pages = need + 5
+    perm = torch.randperm(n_pages, generator=cpu_g)
+    rand = lambda *shape: torch.randn(*shape, generator=g, device=DEV)
+    kpool = (rand(n_pages, nkv, bs, hd) * 3).to(dtype)     # stale data everywhere
+    vpool = (rand(n_pages, nkv, hd, bs) * 3).to(dtype)
+    width = max(-(-c // bs) for c, _ in seqs)
+    bt = torch.full((len(seqs), width), -1, dtype=torch.int32)
+    qs, ks, vs, q_start, at = [], [], [], [0], 0
+    for b, (ctx, ql) in enumerate(seqs):
+        npg = -(-ctx // bs)
+        pages = perm[at:at + npg]
+        at += npg
+        bt[b, :npg] = pages.to(torch.int32)
+        k = (rand(nkv, npg * bs, hd)).to(dtype)            # the tail past ctx is stale data too
+        v = (rand(nkv, npg * bs, hd)).to(dtype)
+        q = (rand(nh, ql, hd) * q_scale).to(dtype)
+        kpool[pages.to(DEV)] = k.view(nkv, npg, bs, hd).permute(1, 0, 2, 3)
+        vpool[pages.to(DEV)] = v.view(nkv, npg, bs, hd).permute(1, 0, 3, 2)
+        qs.append(q.cpu()), ks.append(k[:, :ctx].cpu()), vs.append(v[:, :ctx].cpu())
+        q_start.append(q_start[-1] + ql)
+    q_flat = torch.cat([q.transpose(0, 1).reshape(q.shape[1], nh * hd) for q in qs], dim=0)
+    return dict(q=q_flat, qs=qs, ks=ks, vs=vs, kpool=kpool, vpool=vpool, bt=bt,
+                q_start=torch.tensor(q_start, dtype=torch.int32),
+                ctx_len=torch.tensor([c for c, _ in seqs], dtype=torch.int32))
+
+
+def plain_attention_by_group(s, seqs):
+    """The plain attention, one key/value head at a time (a whole request's scores would not fit)."""
+    outs = []
+    for (ctx, ql), q, k, v in zip(seqs, s["qs"], s["ks"], s["vs"]):
+        nh, nkv = q.shape[0], k.shape[0]
+        grp = nh // nkv
+        heads = [P.attention(q[j * grp:(j + 1) * grp].double(), k[j:j + 1].double(), v[j:j + 1].double(),
+                             torch.arange(ctx - ql, ctx), torch.arange(ctx)) for j in range(nkv)]
+        outs.append(torch.cat(heads, dim=0).transpose(0, 1).reshape(ql, -1))
+    return torch.cat(outs, dim=0)
+
+
+def run_decode(ops, s, n, nh, nkv, hd, max_ctx, dtype):
+    """The split kernel as the attention part launches it: partition size from the plan for this
+    many requests and this bound on the context."""
+    part = ops.attn_decode_plan(n, max_ctx, nh, nkv, hd)
+    max_parts = -(-max_ctx // part)
+    part_o = torch.full((n * nh * max_parts * hd,), float("nan"), device=DEV)
+    part_ml = torch.full((n * nh * max_parts * 2,), float("nan"), device=DEV)
+    out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.attn_decode(s["q"].to(DEV), out, s["kpool"], s["vpool"], s["bt"].to(DEV), s["q_start"].to(DEV),
+                    s["ctx_len"].to(DEV), None, n, part_o, part_ml, max_parts, part, num_heads=nh, num_kv_heads=nkv,
+                    head_dim=hd)
+    return out, part, max_parts
+
+
+def run_prefill(ops, s, seqs, nh, nkv, hd, bs, dtype):
+    """The prefill kernel as the attention part launches it: tiles sorted by the keys they see, the
+    keys of few new tokens cut into the runs the plan says."""
+    tiles = sorted((ctx - ql + min(ql, q0 + 64), b, q0) for b, (ctx, ql) in enumerate(seqs) for q0 in range(0, ql, 64))
+    tile_seq = torch.tensor([t[1] for t in tiles], dtype=torch.int32, device=DEV)
+    tile_q0 = torch.tensor([t[2] for t in tiles], dtype=torch.int32, device=DEV)
+    few, many = tiles[0][0], tiles[-1][0]
+    parts = ops.attn_prefill_plan(len(tiles), many, nh, nkv, hd, dtype, bs)
+    work = {}
+    if parts > 1:
+        n = len(tiles) * 64 * nh * parts
+        work = dict(parts=parts, part_o=torch.full((n * hd,), float("nan"), device=DEV),
+                    part_ml=torch.full((n * 2,), float("nan"), device=DEV))
+    out = torch.full((s["q"].shape[0], nh * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.attn_prefill(s["q"].to(DEV), out, s["kpool"], s["vpool"], s["bt"].to(DEV), s["q_start"].to(DEV),
+                     s["ctx_len"].to(DEV), tile_seq, tile_q0, len(tiles), num_heads=nh, num_kv_heads=nkv, head_dim=hd,
+                     pair=2 * few <= many, **work)
+    return out, parts
+
+
+LONG_DECODE_CASES = [
+    # heads, key/value heads, head size, page size, bound on the context, contexts
+    (32, 8, 64, 16, 8192, [8192]),                                             # the benchmark's shape, batch 1
+    (32, 8, 64, 16, 8192, [8192, 8191, 8177, 8166, 8130, 8100, 8065, 8129]),   # and batch 8, contexts as they grow
+    (24, 8, 128, 16, 8192, [8192]),
+    (24, 8, 128, 16, 8192, [8192, 8000, 8111, 7777, 8190, 8050, 8001, 8160]),
+    (32, 8, 64, 16, 32768, [32768]),
+    (32, 8, 64, 16, 32768, [32768, 32700, 30000, 32767, 31000, 32000, 29000, 32100]),
+    (24, 8, 128, 16, 32768, [32768]),
+    (32, 8, 64, 16, 16384, [8193, 9000]),                                      # a recorded step's bound above every context
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", LONG_DECODE_CASES, ids=[f"{c[0]}/{c[1]}x{c[2]}-{c[4]}-b{len(c[5])}" for c in LONG_DECODE_CASES])
+def test_attention_decode_at_the_benchmarks_contexts(ops, dtype, case):
+    """Contexts of 8,192 and 32,768 keys, batch 1 and 8, the 1B shape's heads (32 over 8, 64 wide)
+    and the 3B shape's (24 over 8, 128 wide), with the partition size that the plan gives for exactly
+    these launches: many partitions per request, block tables 512 to 2,048 entries wide."""
+    nh, nkv, hd, bs, bound, ctxs = case
+    seqs = [(c, 1) for c in ctxs]
+    s = paged_setup_long(seqs, nh, nkv, hd, bs, dtype, seed=hd + len(ctxs))
+    out, part, max_parts = run_decode(ops, s, len(seqs), nh, nkv, hd, bound, dtype)
+    assert max_parts >= 4, "the case is meant to be cut into several partitions"
+    want = plain_attention_by_group(s, seqs)
+    assert float(want.abs().max()) > 0.5          # peaked: single keys show in the result
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 3e-5, 2e-2))
+
+
+LONG_PREFILL_CASES = [
+    (32, 8, 64, 16, [(8192, 512)]),
+    (32, 8, 64, 16, [(8192, 64)]),
+    (24, 8, 128, 16, [(8192, 512)]),
+    (24, 8, 128, 16, [(8192, 64)]),
+    (32, 8, 64, 16, [(8192, 300), (4100, 100), (9000, 2)]),
+    (32, 8, 64, 16, [(8300, 40)]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", LONG_PREFILL_CASES, ids=[f"{c[0]}/{c[1]}x{c[2]}-{c[4]}" for c in LONG_PREFILL_CASES])
+def test_attention_prefill_of_a_portion_over_8192_keys(ops, dtype, case):
+    """512 and 64 new tokens at the end of 8,192 keys, with the runs of keys the plan gives."""
+    nh, nkv, hd, bs, seqs = case
+    s = paged_setup_long(seqs, nh, nkv, hd, bs, dtype, seed=hd + seqs[0][1])
+    out, parts = run_prefill(ops, s, seqs, nh, nkv, hd, bs, dtype)
+    if dtype == torch.bfloat16 and len(seqs) == 1:
+        assert parts > 1, "few tokens over many keys were meant to be cut into runs"
+    want = plain_attention_by_group(s, seqs)
+    assert float(want.abs().max()) > 0.5
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 3e-5, 2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["prefill", "decode"])
+@pytest.mark.parametrize("nh,nkv,hd", [(32, 8, 64), (24, 8, 128)])
+def test_attention_finds_a_key_anywhere_in_8192(ops, dtype, kind, nh, nkv, hd):
+    """Eight requests of about 8,192 keys; in each, one key matches the queries strongly, and each
+    has it elsewhere: the first key, the last, both sides of a partition's edge and of a page's, the
+    middle.  Every output must be that key's value, which a partition, a run or a table entry that
+    is skipped or read for the wrong request cannot give."""
+    bs = 16
+    ql = 1 if kind == "decode" else 3
+    ctxs = [8192, 8191, 8177, 8166, 8130, 8100, 8065, 8129]
+    seqs = [(c, ql) for c in ctxs]
+    s = paged_setup_long(seqs, nh, nkv, hd, bs, dtype, seed=9, q_scale=1.0)
+    part = ops.attn_decode_plan(len(seqs), 8192, nh, nkv, hd)
+    far = [0, ctxs[1] - ql, part - 1, part, 4095, 4096, 3 * part + 17, ctxs[7] // 2]
+    for b, f in enumerate(far):
+        s["qs"][b][:] = 4.0          # score with the planted key: 16 hd / sqrt(hd); with the others ~ N(0, 16)
+        page = int(s["bt"][b, f // bs])
+        s["kpool"][page, :, f % bs, :] = 4.0
+    s["q"] = torch.cat([q.transpose(0, 1).reshape(q.shape[1], nh * hd) for q in s["qs"]], dim=0)
+    if kind == "decode":
+        out, _, _ = run_decode(ops, s, len(seqs), nh, nkv, hd, 8192, dtype)
+    else:
+        out, _ = run_prefill(ops, s, seqs, nh, nkv, hd, bs, dtype)
+    for b, f in enumerate(far):
+        v_far = s["vs"][b][:, f].float()                                   # [nkv, hd]
+        want = v_far.repeat_interleave(nh // nkv, dim=0).reshape(1, nh * hd).expand(ql, -1)
+        got = out[b * ql:(b + 1) * ql].cpu().float()
+        torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2, msg=lambda m: f"request {b}, key {f}: {m}")
+
+
 # --------------------------------------------------------------------- sampler
 def test_sampler_greedy_and_draws(ops):
     V = 1003

@@ -274,3 +274,26 @@ def test_sampling_follows_the_reference_rules():
     assert cold[0] > 0.999                                         # T -> 0 tends to the argmax
     probs = torch.tensor([0.1, 0.2, 0.3, 0.4])
     assert [P.inverse_cdf(probs, u) for u in (0.0, 0.05, 0.1, 0.29, 0.3, 0.95, 0.9999)] == [0, 0, 1, 1, 2, 3, 3]
+
+
+def test_the_long_request_helper_is_the_plain_forward(tmp_path):
+    """``trace_util.plain_logits_at`` (queries a few at a time, the last layer at the wanted places
+    only) gives what ``P.forward`` gives."""
+    import json
+    import os
+
+    from safetensors.torch import save_file
+    from trace_util import plain_logits_at
+
+    cfg = dict(CFG, num_hidden_layers=3, rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
+                                                           high_freq_factor=4.0, original_max_position_embeddings=16))
+    w = tiny_weights(cfg, seed=5)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(tmp_path, "model.safetensors"))
+    json.dump(cfg, open(os.path.join(tmp_path, "config.json"), "w"))
+    toks = torch.randint(0, cfg["vocab_size"], (41,), generator=torch.Generator().manual_seed(1)).tolist()
+    w2, cfg2 = P.read_model(str(tmp_path))
+    full = P.forward(w2, cfg2, toks)
+    got = plain_logits_at(str(tmp_path), toks, [40, 0, 17, 39], chunk=7)
+    assert sorted(got) == [0, 17, 39, 40]
+    for r, row in got.items():
+        torch.testing.assert_close(row, full[r], rtol=1e-9, atol=1e-9)

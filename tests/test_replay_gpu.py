@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 
 from conftest import ROOT, TINY
-from trace_util import Trace, compare, plain_logits, random_tokens, random_trace, replay
+from trace_util import Trace, compare, plain_logits, plain_logits_at, random_tokens, random_trace, replay
 
 pytestmark = pytest.mark.gpu
 
@@ -339,3 +339,33 @@ def test_a_wide_layer_over_a_long_context(tmp_path, dtype):
         t.step([("a", 1), ("b", 1)])
     t.step([("a", 1)], end=["a", "b"])
     compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "wide layer, long context")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_wide_layer_at_the_benchmarks_context(tmp_path, dtype):
+    """The 1B shape's layer to 8,300 tokens, where the benchmark runs: the prompt in portions of
+    2,048 (each one's keys beyond the first in runs for workgroups of their own), a last portion of
+    92 beside the prompt of a second, short request, then sixteen decoded tokens of both (the long
+    one's keys in many partitions, block tables over 512 entries wide), against the plain model."""
+    from lyapunov_engine_amd.weights import write_random_model
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=8448, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=2048))
+    d = str(tmp_path / "wide")
+    os.makedirs(d)
+    write_random_model(cfg, d, 13, dtype, init_std=0.03, norm_init_std=0.1)
+    reqs = {"a": random_tokens(8300, 1000, seed=6), "b": random_tokens(40, 1000, seed=7)}
+    t = Trace(reqs)
+    for _ in range(4):
+        t.step([("a", 2048)], want="last")
+    t.step([("a", 92), ("b", 24)], want="last")
+    for _ in range(16):
+        t.step([("a", 1), ("b", 1)])
+    t.steps[-1]["end"] = ["a", "b"]
+    t.live.clear()
+    rows_a = sorted(pos for rows in t.rows.values() for rid, pos in rows if rid == "a")
+    want = {"a": plain_logits_at(d, reqs["a"], rows_a), "b": plain_logits(d, {"b": reqs["b"]})["b"]}
+    compare(t, replay(d, dtype, t), want, dtype, "wide layer at 8,300 tokens")

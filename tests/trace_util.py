@@ -84,6 +84,43 @@ def plain_logits(folder: str, requests: dict) -> dict:
     return {rid: P.forward(w, cfg, toks) for rid, toks in requests.items()}
 
 
+def plain_logits_at(folder: str, tokens: list, rows: list, chunk: int = 256) -> dict:
+    """position -> float64 logits, for the wanted positions of one long request.  The plain
+    model part by part, as ``P.forward`` puts it together, but with the queries taken a few at a time
+    (a whole request's scores would not fit in memory at thousands of tokens) and, in the last layer,
+    only at the wanted positions.  ``tests/test_plain.py`` checks it against ``P.forward``."""
+    w, cfg = P.read_model(folder)
+    w = {k: v.double() for k, v in w.items()}
+    S = len(tokens)
+    pos = torch.arange(S)
+    inv = P.model_inv_freq(cfg)
+    cos, sin = P.rope_cos_sin(pos, inv)
+    nh, nkv, hd, eps = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["rms_norm_eps"]
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    layers = cfg["num_hidden_layers"]
+    keep = torch.tensor(sorted(rows))
+    for i in range(layers):
+        p = f"model.layers.{i}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+        k = P.apply_rope((x @ w[p + "self_attn.k_proj.weight"].T).view(S, nkv, hd).transpose(0, 1), cos, sin)
+        v = (x @ w[p + "self_attn.v_proj.weight"].T).view(S, nkv, hd).transpose(0, 1)
+        need = keep if i == layers - 1 else pos
+        outs = []
+        for lo in range(0, len(need), chunk):
+            r = need[lo:lo + chunk]
+            q = (x[r] @ w[p + "self_attn.q_proj.weight"].T).view(len(r), nh, hd).transpose(0, 1)
+            q = P.apply_rope(q, cos[r], sin[r])
+            o = P.attention(q, k, v, r, pos)
+            outs.append(o.transpose(0, 1).reshape(len(r), nh * hd) @ w[p + "self_attn.o_proj.weight"].T)
+        h = h[need] + torch.cat(outs)
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+        h = h + P.mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    h = P.rms_norm(h, w["model.norm.weight"], eps)
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]
+    logits = h @ head.T
+    return {int(r): logits[j] for j, r in enumerate(keep.tolist())}
+
+
 def replay(folder: str, dtype: str, trace: Trace, max_tokens=None) -> dict:
     """Run the trace through the engine in this process: step -> [rows, vocab]."""
     from lyapunov_engine_amd.engine.replay import TraceReplayer
