@@ -34,7 +34,8 @@ SHAPES = {
 }
 
 
-def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget, shape=MODEL):
+def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget, shape=MODEL, rounded=False):
+    """``rounded``: the random weights are rounded to bfloat16 whatever the engine's precision."""
     import torch
 
     from lyapunov_engine_amd.config import EngineConfig, LlamaConfig
@@ -47,7 +48,8 @@ def build_engine(layers, dtype, num_blocks, max_num_seqs, block_size, budget, sh
     cfg = LlamaConfig.from_dict(dict(shape, num_hidden_layers=layers))
     model = build_model(llama_spec(cfg))
     tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
-    tensors = dict(random_tensors(model, 4, tdtype, device="cuda:0"))   # seed 4, N(0, 0.02)
+    tensors = dict(random_tensors(model, 4, torch.bfloat16 if rounded else tdtype, device="cuda:0"))   # seed 4, N(0, 0.02)
+    tensors = {k: v.to(tdtype) for k, v in tensors.items()}
     load_weights(model, DictSource(tensors), tdtype, "cuda:0")
     del tensors
     core = EngineCore(model, cfg, dtype=tdtype, device="cuda:0", num_blocks=num_blocks, block_size=block_size,
@@ -175,28 +177,50 @@ def measure_mixed(engine, cfg, requests=64, seed=0):
     return time.perf_counter() - t0, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps
 
 
-def check_logits(shape=MODEL, layers=2, tokens=96):
-    """The 32-bit engine against the bfloat16 engine on the same shape (fewer
-    layers) and the same random weights before rounding: the largest difference
-    of the last position's logits, relative to the largest logit."""
+CHECK_LIMIT = 0.02   # largest bf16-against-fp32 logit difference over the largest logit that passes
+
+
+def check_logits(shape=MODEL, layers=2, context=8192, portion=2048):
+    """The bfloat16 engine against the 32-bit engine at the benchmark's context, on the same shape
+    (fewer layers) and the same weights (random, rounded to bfloat16 for both, so that only the
+    arithmetic differs): a prompt of context - 1 tokens in portions, through the eager step, then
+    one decoded token through the recorded graph of that context.  Returns, for the last prompt
+    position and for the decoded position, the largest difference of the logits relative to the
+    largest logit, and whether both engines agree on the best token."""
+    import numpy as np
     import torch
 
+    from lyapunov_engine_amd.engine.graphs import DecodeGraphs
     from lyapunov_engine_amd.engine.runner import StepEntry
 
-    prompt = random_prompt(tokens, shape["vocab_size"], 6)
+    prompt = random_prompt(context, shape["vocab_size"], 6)
     logits = {}
     for dtype in ("fp32", "bf16"):
-        engine, _ = build_engine(layers, dtype, num_blocks=64, max_num_seqs=4, block_size=16, budget=2048, shape=shape)
+        engine, _ = build_engine(layers, dtype, num_blocks=context // 16 + 8, max_num_seqs=1, block_size=16,
+                                 budget=portion, shape=shape, rounded=True)
         core = engine.core
         core.cache.add(0)
-        core.cache.extend(0, tokens)
-        logits[dtype] = core.step([StepEntry(0, prompt, 0, [tokens - 1])]).float().cpu()
-        core.cache.commit(0, tokens)
+        rows = []
+        for lo in range(0, context - 1, portion):
+            hi = min(context - 1, lo + portion)
+            core.cache.extend(0, hi)
+            out = core.step([StepEntry(0, prompt[lo:hi], lo, [hi - lo - 1] if hi == context - 1 else [])])
+            core.cache.commit(0, hi)
+        rows.append(out.float().cpu()[0])
+        core.cache.extend(0, context)
+        graphs = DecodeGraphs(core.runner, max_batch=1)
+        out = graphs.step_arrays(np.zeros(1, np.int64), np.asarray([context - 1], np.int32),
+                                 np.asarray(prompt[-1:], np.int32))
+        rows.append(out.float().cpu()[0])
+        assert list(graphs.captured) == [(1, context)]
+        core.cache.commit(0, context)
         core.cache.free(0)
-        del engine, core
+        logits[dtype] = rows
+        del engine, core, graphs
         torch.cuda.empty_cache()
-    ref = logits["fp32"]
-    return float((logits["bf16"] - ref).abs().max() / ref.abs().max()), int(ref.argmax() == logits["bf16"].argmax())
+    rel = [float((b - a).abs().max() / a.abs().max()) for a, b in zip(logits["fp32"], logits["bf16"])]
+    same = [bool(a.argmax() == b.argmax()) for a, b in zip(logits["fp32"], logits["bf16"])]
+    return rel, same
 
 
 def main():
@@ -264,9 +288,12 @@ def main():
     if not args.skip_check:
         del engine
         torch.cuda.empty_cache()
-        rel, same = check_logits(shape)
-        check = {"what": "bf16 against fp32 logits, same weights, 2 layers, 96-token prompt, last position",
-                 "max_diff_over_max_logit": round(rel, 5), "same_argmax": bool(same)}
+        rel, same = check_logits(shape, context=args.context)
+        check = {"what": f"bf16 against fp32 logits, same bf16-rounded weights, 2 layers, prompt of {args.context - 1} "
+                         f"tokens in portions of 2048 (eager), then one decoded token at context {args.context} "
+                         f"through the recorded graph; largest difference over largest logit",
+                 "prompt_last": round(rel[0], 5), "decoded_through_graph": round(rel[1], 5), "limit": CHECK_LIMIT,
+                 "same_argmax": all(same), "ok": max(rel) <= CHECK_LIMIT}
 
     peak = MFMA_PEAK[args.dtype]
     line = {
@@ -292,6 +319,10 @@ def main():
         "logits_check": check,
     }
     print(json.dumps(line))
+    if check is not None and not check["ok"]:
+        print(f"bench.py: bfloat16 logits at context {args.context} are off by {max(rel):.4f} of the largest logit "
+              f"(limit {CHECK_LIMIT})", file=sys.stderr)
+        return 1
     return 0
 
 
