@@ -12,7 +12,8 @@ import numpy as np
 import pytest
 
 from conftest import ROOT, TINY
-from trace_util import Trace, compare, plain_logits, plain_logits_at, random_tokens, random_trace, replay
+from trace_util import (Trace, compare, compare_with_alone, plain_logits, plain_logits_at, random_tokens, random_trace,
+                        replay)
 
 pytestmark = pytest.mark.gpu
 
@@ -73,7 +74,9 @@ def test_most_in_one_step_then_token_by_token(model_folders, name, dtype):
         t.step([(rid, len(toks) - 32)], want="last")
         for _ in range(32):
             t.step([(rid, 1)])
-        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"decode {rid}")
+        got = replay(folder(model_folders, name, dtype), dtype, t)
+        compare(t, got, want, dtype, f"decode {rid}")
+        compare_with_alone(t, got, folder(model_folders, name, dtype), dtype, f"decode {rid}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -94,7 +97,9 @@ def test_portions_of_changing_size(model_folders, name, dtype):
             t.step([(rid, n)])
             left -= n
             i += 1
-        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"portions {rid}")
+        got = replay(folder(model_folders, name, dtype), dtype, t)
+        compare(t, got, want, dtype, f"portions {rid}")
+        compare_with_alone(t, got, folder(model_folders, name, dtype), dtype, f"portions {rid}")
 
 
 def mixed_trace(reqs):
@@ -123,20 +128,26 @@ def test_mixed_batches_with_pages_used_again(model_folders, name, dtype):
     t = mixed_trace(reqs)
     total = sum(64 * -(-len(v) // 64) for v in reqs.values())
     assert t.max_tokens < total, "the pool is meant to be too small for all requests at once"
-    compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, "mixed")
+    got = replay(folder(model_folders, name, dtype), dtype, t)
+    compare(t, got, want, dtype, "mixed")
+    compare_with_alone(t, got, folder(model_folders, name, dtype), dtype, "mixed")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_random_schedules(model_folders, name, dtype):
-    """Twelve random sets of requests under random schedules each (a sweep of 3,000 seeds of this
-    generator found no logits that depend on the schedule)."""
+    """Twelve random sets of requests under random schedules each, against the plain model and
+    against the same requests alone and whole.  (Sweeps of thousands of seeds of this generator are
+    where the tolerances of trace_util come from; in 32-bit they found no logits that depend on the
+    schedule beyond 2e-6.)"""
     cfg = TINY[name][0]
     for seed in range(12):
         rng = random.Random(1000 * seed + ord(name))
         reqs, t = random_trace(rng, cfg["vocab_size"], min(200, cfg["max_position_embeddings"] - 1))
         want = plain_for(model_folders, name, dtype, reqs)
-        compare(t, replay(folder(model_folders, name, dtype), dtype, t), want, dtype, f"random schedule {seed}")
+        got = replay(folder(model_folders, name, dtype), dtype, t)
+        compare(t, got, want, dtype, f"random schedule {seed}")
+        compare_with_alone(t, got, folder(model_folders, name, dtype), dtype, f"random schedule {seed}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -369,3 +380,29 @@ def test_a_wide_layer_at_the_benchmarks_context(tmp_path, dtype):
     rows_a = sorted(pos for rows in t.rows.values() for rid, pos in rows if rid == "a")
     want = {"a": plain_logits_at(d, reqs["a"], rows_a), "b": plain_logits(d, {"b": reqs["b"]})["b"]}
     compare(t, replay(d, dtype, t), want, dtype, "wide layer at 8,300 tokens")
+
+
+def test_the_largest_bfloat16_error_a_sweep_found(model_folders):
+    """Seed 1098 of configuration A in a sweep of 3,000 random schedules: at position 32 of its
+    first request the bfloat16 logits are 7.3 % of the largest logit off the plain model's, the
+    largest such error seen.  It is rounding: the request run alone and whole is off by the same
+    amount there, the mixed schedule agrees with that run to 3 %, and the 32-bit engine is exact.
+    The case is kept so that the per-row bound stays where measurement put it."""
+    name = "A"
+    vocab = TINY[name][0]["vocab_size"]
+    made = [(69, 713405), (3, 36094), (2, 167777), (3, 176177), (108, 911988), (1, 834276), (3, 610150)]
+    reqs = {f"r{i}": random_tokens(n, vocab, seed) for i, (n, seed) in enumerate(made)}
+    steps = [([("r0", 23)], [], "last"), ([("r0", 15), ("r1", 2), ("r2", 2), ("r3", 1)], [], "all"),
+             ([("r3", 2)], ["r2"], "all"), ([("r0", 1), ("r1", 1)], ["r1"], "all"), ([("r0", 24)], [], "all"),
+             ([("r0", 2), ("r4", 1), ("r5", 1)], ["r3", "r5"], "all"), ([("r0", 1)], [], "all"),
+             ([("r0", 3), ("r6", 2)], [], "all"), ([("r4", 6), ("r6", 1)], ["r0", "r6"], "last")]
+    for dtype in DTYPES:
+        t = Trace(reqs)
+        for portions, end, want in steps:
+            t.step(portions, end=end, want=want)
+        f = folder(model_folders, name, dtype)
+        got = replay(f, dtype, t)
+        rel = compare(t, got, plain_for(model_folders, name, dtype, reqs), dtype, "seed 1098")
+        compare_with_alone(t, got, f, dtype, "seed 1098")
+        if dtype == "bfloat16":
+            assert 0.05 < max(rel) < 0.08, f"the case is kept for its error of 7.3 %; it now shows {max(rel):.3f}"

@@ -136,24 +136,71 @@ def replay(folder: str, dtype: str, trace: Trace, max_tokens=None) -> dict:
     return out
 
 
-# atol is relative to the largest logit of the row.  Measured on these models:
-# about 2e-6 in 32-bit, about 3e-2 in bfloat16.
-TOL = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=6e-2, atol=6e-2)}
+# Tolerances, relative to the largest logit of the row (at least 1).
+#
+# 32-bit: about 2e-6 is measured; 5e-5 is allowed.
+#
+# bfloat16 (8 bits of mantissa, rounded after every kernel) against the plain model in float64 on
+# the same rounded weights, measured over random schedules of the three tiny configurations (600
+# seeds each, 220,000 rows; an earlier sweep of 3,000 seeds): per row median 1.0e-2, 99th
+# percentile 2.4e-2, 99.9th 3.2e-2, largest 5.6e-2 and 7.3e-2 (seed 1098 of configuration A, the
+# fixed case in test_replay_gpu.py; the same error with the request run alone, so rounding, not
+# scheduling).  Per trace the median over its rows was 1.23e-2 at worst.  So: no row beyond 8e-2,
+# and, for a trace of eight rows or more, a median of at most 1.5e-2: a defect that only shifts
+# results a little, which the per-row bound cannot see, moves the median.
+#
+# bfloat16 against the same request run alone and whole in bfloat16: the cuts choose the kernels
+# (rows of a step, prefill or split attention, partition sizes), and kernels round differently,
+# so this is not exact either: per row median 0.4-0.6e-2, 99.9th percentile 1.7e-2, largest 2.6e-2.
+# Allowed: 3e-2 per row, 1e-2 for a trace's median.
+TOL = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=0.0, atol=8e-2, median=1.5e-2)}
+TOL_ALONE = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=0.0, atol=3e-2, median=1e-2)}
 
 
-def compare(trace: Trace, got: dict, want: dict, dtype: str, label=""):
-    """Every row of every step against the plain logits at its (request,
+def compare(trace: Trace, got: dict, want: dict, dtype: str, label="", tol=None):
+    """Every row of every step against the reference logits at its (request,
     position); on failure name the first wrong place, which is where to look."""
     assert set(got) == set(trace.rows), f"{label}: steps with logits {sorted(got)} != expected {sorted(trace.rows)}"
-    tol = TOL[dtype]
+    tol = tol or TOL[dtype]
+    rel = []
     for n in sorted(trace.rows):
         rows = trace.rows[n]
         assert got[n].shape[0] == len(rows), f"{label}: step {n} has {got[n].shape[0]} rows, wanted {len(rows)}"
         for i, (rid, pos) in enumerate(rows):
-            ref = want[rid][pos].numpy()
+            ref = np.asarray(want[rid][pos], dtype=np.float64)
             scale = max(1.0, float(np.abs(ref).max()))
             err = np.abs(got[n][i].astype(np.float64) - ref)
             bad = err > tol["atol"] * scale + tol["rtol"] * np.abs(ref)
             assert not bad.any(), (f"{label}: first wrong logits at step {n}, request {rid!r}, position {pos}: "
                                    f"max error {err.max():.3e} (scale {scale:.3f}); entries of the step: "
                                    f"{[(e['id'], len(e['tokens'])) for e in trace.steps[n]['entries']]}")
+            rel.append(float(err.max()) / scale)
+    if "median" in tol and len(rel) >= 8:
+        med = float(np.median(rel))
+        assert med <= tol["median"], (f"{label}: the median error over the trace's {len(rel)} rows is {med:.3e} of the "
+                                      f"largest logit; {tol['median']:.1e} is what rounding accounts for")
+    return rel
+
+
+_ALONE: dict = {}
+
+
+def alone_logits(folder: str, dtype: str, requests: dict) -> dict:
+    """id -> [len, vocab] logits of every request run through the engine alone
+    and whole, one step each, in this precision (kept between tests)."""
+    out = {}
+    for rid, toks in requests.items():
+        key = (folder, dtype, tuple(toks))
+        if key not in _ALONE:
+            t = Trace({rid: toks})
+            t.step([(rid, len(toks))], end=[rid])
+            _ALONE[key] = replay(folder, dtype, t)[0]
+        out[rid] = _ALONE[key]
+    return out
+
+
+def compare_with_alone(trace: Trace, got: dict, folder: str, dtype: str, label=""):
+    """The trace's logits against the same requests run alone and whole in the
+    same precision: what the cuts and the batch mates may change is rounding."""
+    return compare(trace, got, alone_logits(folder, dtype, trace.requests), dtype, label + " (against alone and whole)",
+                   tol=TOL_ALONE[dtype])
