@@ -339,7 +339,37 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, siz
   if (idx < n) out[idx] = from_f32<TO>(to_f32(in[idx]));
 }
 
-static int norm_threads(int H) { return H <= 512 ? 128 : (H >= 4096 ? 512 : 256); }
+// Threads per row of the two-pass norm kernels (rows whose length or alignment keeps them from
+// the one-pass kernel).  Measured on gfx950 with 2,048 rows: a wave of 64 for every 512 values,
+// between one wave and sixteen; `g_norm_threads` (set by lyp_norm_threads_override, 0: this rule)
+// is there for that measurement.
+static int g_norm_threads = 0;
+static int norm_threads(int H) {
+  if (g_norm_threads > 0) return g_norm_threads;
+  const int waves = (H + 511) / 512;
+  return 64 * (waves < 1 ? 1 : (waves > 16 ? 16 : waves));
+}
+
+// Reads `n` 16-byte words once and keeps one word per workgroup: what memory gives a kernel that
+// does nothing but stream (the yardstick the weight-streaming products are held against).
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restrict__ src, size_t n,
+                                                          uint32_t* __restrict__ sink) {
+  uint32_t acc = 0;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  // four loads in flight per thread
+  for (; i + 3 * stride < n; i += 4 * stride) {
+    const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+  }
+  for (; i < n; i += stride) {
+    const uint4 a = src[i];
+    acc ^= a.x ^ a.y ^ a.z ^ a.w;
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, kWave);
+  if (threadIdx.x % kWave == 0) sink[blockIdx.x * (256 / kWave) + threadIdx.x / kWave] = acc;
+}
 
 // A step's table of small integers from pinned host memory (which the device reads through the
 // same address) to its place on the device, in one launch; `n_patch` words from `patch_at` on come
@@ -358,6 +388,24 @@ __global__ __launch_bounds__(256) void table_load_kernel(const int32_t* __restri
 using namespace lyp;
 
 extern "C" {
+
+// Threads per row for the two-pass norm kernels instead of the built-in rule (0: the rule again).
+// A multiple of 64 up to 1024; for measurements.
+int lyp_norm_threads_override(int threads) {
+  LYP_REQUIRE(threads >= 0 && threads <= 1024 && threads % 64 == 0, "norm threads: %d", threads);
+  g_norm_threads = threads;
+  return 0;
+}
+
+// Streams `bytes` (a multiple of 16) of device memory through `blocks` workgroups of 256 threads;
+// sink: blocks * 4 words.
+int lyp_stream_read(const void* src, long long bytes, int blocks, uint32_t* sink, hipStream_t stream) {
+  LYP_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && blocks > 0 && blocks <= 65535 &&
+              reinterpret_cast<uintptr_t>(src) % 16 == 0, "stream_read: %lld bytes in %d workgroups", bytes, blocks);
+  stream_read_kernel<<<blocks, 256, 0, stream>>>(static_cast<const uint4*>(src), static_cast<size_t>(bytes / 16), sink);
+  LYP_LAUNCH_CHECK("stream_read");
+  return 0;
+}
 
 // dst[0..n) on the device = src[0..n) in pinned host memory, except dst[patch_at .. patch_at + n_patch)
 // = patch[0..n_patch) (on the device; may be null).

@@ -118,11 +118,14 @@ class LLMEngine:
     WARMUP_ID = -1   # the cache manager's name for the warm-up step's request; the scheduler counts from 0
 
     def _warm_up(self) -> None:
-        """One step of as many tokens as a step may bring (as far as the model's
-        length and the pages go), of a request that is gone afterwards.  It
-        loads the kernels a full step needs, and the products of that many rows
-        are given the fastest of the vendor library's algorithms by measurement
-        (``ops.library_gemm_tuning``) rather than the library's first guess."""
+        """Steps of as many tokens as a step may bring (as far as the model's
+        length and the pages go), and of every power of two from 128 up to
+        that, by a request that is gone afterwards.  They load the kernels a
+        full step needs, and the products of that many rows are given the
+        fastest of the vendor library's algorithms by measurement
+        (``ops.library_gemm_tuning``) rather than the library's first guess; a
+        prompt portion of any other length later takes the choice measured for
+        the nearest of these sizes."""
         from ..kernels import ops
 
         cache, cfg = self.core.cache, self.config
@@ -130,12 +133,20 @@ class LLMEngine:
         sizes = {cfg.max_num_batched_tokens}
         if cfg.max_chunk:
             sizes.add(min(cfg.max_chunk, cfg.max_num_batched_tokens))
-        for n in sorted(min(s, self.max_model_len, pages * self.core.block_size) for s in sizes):
+        if ops.LIBRARY_GEMM and ops.LIBRARY_TUNE_CANDIDATES > 1 and self.core.dtype == torch.bfloat16:
+            n = 128
+            while n < cfg.max_num_batched_tokens:
+                sizes.add(n)
+                n *= 2
+        for n in sorted({min(s, self.max_model_len, pages * self.core.block_size) for s in sizes}):
             if n < 1 or cache.has(self.WARMUP_ID) or cache.num_free_slots() < 1:
                 continue
             cache.add(self.WARMUP_ID)
             try:
                 cache.extend(self.WARMUP_ID, n)
+                if len(sizes) > 2:
+                    print(f"[lyapunov-amd] warm-up: a step of {n} tokens (matrix-product algorithms chosen by measurement)",
+                          file=sys.stderr, flush=True)
                 with ops.library_gemm_tuning():
                     self.core.runner.step_arrays(np.asarray([self.WARMUP_ID], dtype=np.int64), np.zeros(1, dtype=np.int32),
                                                  np.asarray([n], dtype=np.int32), np.zeros(n, dtype=np.int32),

@@ -75,6 +75,8 @@ def core() -> ctypes.CDLL:
                                    c_void_p, c_void_p, c_void_p]
         lib.lyp_sample_workspace.argtypes = [c_int]
         lib.lyp_sample_workspace.restype = c_longlong
+        lib.lyp_norm_threads_override.argtypes = [c_int]
+        lib.lyp_stream_read.argtypes = [c_void_p, c_longlong, c_int, c_void_p, c_void_p]
         _core = lib
     return _core
 
@@ -292,6 +294,23 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
     return out
 
 
+def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
+    """Read all of ``src`` once with ``blocks`` workgroups (a yardstick for the
+    kernels that stream weights); ``sink``: int32, blocks * 4 values."""
+    _dev(src, sink)
+    nbytes = src.numel() * src.element_size()
+    if sink.dtype != torch.int32 or sink.numel() < blocks * 4:
+        raise KernelError("stream_read: the sink must hold four int32 values per workgroup")
+    lib = core()
+    _check(lib.lyp_stream_read(_p(src), nbytes, blocks, _p(sink), _stream()), lib)
+
+
+def norm_threads_override(threads: int) -> None:
+    """Threads per row of the two-pass norm kernels (0: the built-in rule); for measurements."""
+    lib = core()
+    _check(lib.lyp_norm_threads_override(threads), lib)
+
+
 def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
     _dev(x, weight, out)
     n, H = x.shape
@@ -454,15 +473,14 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------------ GEMM
-# Large bfloat16 products go to the vendor's matrix library (through torch), as
-# the reference's projections go to cuBLAS (nn.Linear, models/llama.py:45-48,
-# 112-117, 177).  Products with few rows (decode steps), every float product
-# (true 32-bit) and everything when LYAPUNOV_AMD_GEMM=own use the kernels here.
-# LYAPUNOV_AMD_GEMM: "library" (the default: hipBLASLt called directly, with the plan of every shape
-# kept), "torch" (the same library behind torch.matmul: 18 us of host time a call instead of 10), "own".
+# Large bfloat16 products go to the vendor's matrix library (hipBLASLt, called
+# directly with the plan of every shape kept), as the reference's projections go
+# to cuBLAS (nn.Linear, models/llama.py:45-48, 112-117, 177).  Products with few
+# rows (decode steps), every float product (true 32-bit) and everything when
+# LYAPUNOV_AMD_GEMM=own use the kernels of this package.
 LIBRARY_GEMM_MODE = os.environ.get("LYAPUNOV_AMD_GEMM", "library")
-if LIBRARY_GEMM_MODE not in ("library", "torch", "own"):
-    raise KernelError(f"LYAPUNOV_AMD_GEMM is 'library', 'torch' or 'own', not {LIBRARY_GEMM_MODE!r}")
+if LIBRARY_GEMM_MODE not in ("library", "own"):
+    raise KernelError(f"LYAPUNOV_AMD_GEMM is 'library' or 'own', not {LIBRARY_GEMM_MODE!r}")
 LIBRARY_GEMM = LIBRARY_GEMM_MODE != "own"
 LIBRARY_WORKSPACE_BYTES = 76 << 20    # what the library may use beside the operands (stream-K partial tiles)
 LIBRARY_GEMM_MIN_ROWS = 65
@@ -473,11 +491,12 @@ LIBRARY_GEMM_MID_ROWS = 17
 LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
 # In an engine's warm-up step and in the run before a graph is captured, a library product's algorithm is
 # chosen by measurement among this many of the library's candidates (at the shape's first call).
-# LYAPUNOV_AMD_GEMM_TUNE=0 leaves every choice to the library.
+# Which candidate wins a timing may differ from process to process, and with it the last bits of
+# bfloat16 results; LYAPUNOV_AMD_GEMM_TUNE=0 leaves every choice to the library's own heuristic, which
+# gives the same bits in every run.
 LIBRARY_TUNE_CANDIDATES = int(os.environ.get("LYAPUNOV_AMD_GEMM_TUNE", "16"))
 
 
-_MM_FLOAT_OUT = True   # torch.mm(..., out_dtype=float32) exists and works (found out at the first use)
 _blas_lib = None
 _blas_workspace: dict = {}
 _blas_tuning = (0, 0)   # (candidates, without a workspace): the library's setting, kept here while it is not loaded
@@ -490,7 +509,7 @@ def blas() -> ctypes.CDLL:
         try:
             lib = _load(build.blas_library())
         except (RuntimeError, KernelError) as e:
-            raise KernelError(f"{e}\n(LYAPUNOV_AMD_GEMM=torch reaches the same library through torch)") from None
+            raise KernelError(f"{e}\n(LYAPUNOV_AMD_GEMM=own runs every product in this package's kernels)") from None
         lib.lyp_last_error.restype = ctypes.c_char_p
         lib.lyp_library_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_int, c_void_p, c_longlong, c_void_p]
@@ -546,18 +565,6 @@ def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torc
             or out.stride(1) != 1 or not (a.is_cuda and w.is_cuda and out.is_cuda)):
         raise KernelError(f"library gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, "
                           f"out {tuple(out.shape)} {out.dtype}")
-    if LIBRARY_GEMM_MODE == "torch":
-        global _MM_FLOAT_OUT
-        if out.dtype == torch.bfloat16:
-            return torch.matmul(a, w.t(), out=out)
-        if _MM_FLOAT_OUT:
-            try:   # the library's float accumulators written out as they are
-                return torch.mm(a, w.t(), out_dtype=torch.float32, out=out)
-            except (TypeError, RuntimeError):
-                _MM_FLOAT_OUT = False   # this torch cannot: the operands' type, then a cast
-        y = torch.matmul(a, w.t())
-        _check(core().lyp_cast(_p(y), _code(y.dtype), _p(out), _code(out.dtype), y.numel(), _stream()), core())
-        return out
     lib = blas()
     ws = _blas_workspace.get(a.device)
     if ws is None:
@@ -575,12 +582,16 @@ def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
 
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
     """out = a @ w.T (or out += ...).  a [M, K], w [N, K] of one dtype; out
-    [M, N] of that dtype or float."""
-    _dev(a, w, out)
+    [M, N] of that dtype or float.  Rows may lie further apart than they are
+    long (column ranges of wider tensors); a row's values must be neighbours."""
     M, K = a.shape
     N = w.shape[0]
     if w.shape[1] != K or tuple(out.shape) != (M, N) or a.dtype != w.dtype:
         raise KernelError(f"gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, out {tuple(out.shape)}")
+    for name, t in (("a", a), ("w", w), ("out", out)):
+        if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.stride(0) < t.shape[1]:
+            raise KernelError(f"gemm: {name} {tuple(t.shape)} with strides {t.stride()} on {t.device}: the values of "
+                              f"a row must be neighbours in GPU memory")
     if out.dtype == torch.bfloat16 and not accumulate and _library_product(M, N, K, a.dtype):
         return library_gemm_nt(a, w, out)
     if accumulate:
@@ -594,7 +605,8 @@ def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: boo
     else:
         raise KernelError(f"gemm: output dtype {out.dtype} for operands of {a.dtype}")
     lib = core()
-    _check(lib.lyp_gemm_nt(_p(a), _p(w), _p(out), _code(a.dtype), mode, M, N, K, K, K, N, _stream()), lib)
+    _check(lib.lyp_gemm_nt(_p(a), _p(w), _p(out), _code(a.dtype), mode, M, N, K, a.stride(0), w.stride(0),
+                           out.stride(0), _stream()), lib)
     return out
 
 

@@ -5,6 +5,8 @@
     python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 8 --out-features 16384 --in-features 2048
     python -m lyapunov_engine_amd.utils.kernel_bench residual --rows 8 --out-features 2048 --in-features 8192
     python -m lyapunov_engine_amd.utils.kernel_bench sample --rows 8 --vocab 128256 --top-k 50 --top-p 0.9
+    python -m lyapunov_engine_amd.utils.kernel_bench stream --megabytes 64
+    python -m lyapunov_engine_amd.utils.kernel_bench rmsnorm --rows 2048 --in-features 4100 --threads 256
 
 Prints the time per call and what it means in TFLOP/s or TB/s.  Small enough to
 run under ``rocprofv3 --pmc ...`` when a kernel's counters are wanted; the
@@ -139,9 +141,56 @@ def sample(a) -> None:
           f"{t * 1e6:.1f} us")
 
 
+def stream(a) -> None:
+    """A kernel that only reads: ``megabytes`` of device memory once per launch, cold (another
+    buffer four times the size of the memory-side cache is read in between) and warm (the same
+    buffer again and again), over a range of grid sizes.  What the weight-streaming products and
+    the split attention can be held against."""
+    dev = a.device
+    sizes = [a.megabytes] if a.megabytes else [4, 13, 34, 67, 134, 525, 2048]
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    for mb in sizes:
+        src = torch.empty(mb << 20, dtype=torch.uint8, device=dev).random_()
+        for blocks in ([a.blocks] if a.blocks else [256, 512, 1024, 2048, 4096]):
+            sink = torch.empty(blocks * 4, dtype=torch.int32, device=dev)
+            warm = _time(lambda: ops.stream_read(src, sink, blocks), a.repeat)
+            cold = []
+            for _ in range(5):
+                ops.stream_read(flush, torch.empty(4096 * 4, dtype=torch.int32, device=dev), 4096)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                ops.stream_read(src, sink, blocks)
+                e1.record()
+                torch.cuda.synchronize()
+                cold.append(e0.elapsed_time(e1) * 1e-3)
+            c = sorted(cold)[len(cold) // 2]
+            print(f"stream {mb} MiB in {blocks} workgroups: cold {c * 1e6:.1f} us {src.numel() / c / 1e12:.2f} TB/s, "
+                  f"again and again {warm * 1e6:.1f} us {src.numel() / warm / 1e12:.2f} TB/s")
+
+
+def rmsnorm(a) -> None:
+    """The norm kernels on ``rows`` rows of ``in-features`` values; ``--threads`` sets the
+    workgroup size of the two-pass kernels (rows of odd lengths) instead of the built-in rule."""
+    dt, dev = _dtype(a.dtype), a.device
+    h = torch.randn(a.rows, a.in_features, device=dev)
+    w = torch.ones(a.in_features, device=dev, dtype=dt)
+    delta = torch.randn(a.rows, a.in_features, device=dev).to(dt)
+    out = torch.empty(a.rows, a.in_features, device=dev, dtype=dt)
+    for threads in ([a.threads] if a.threads else [0, 64, 128, 256, 512, 1024]):
+        ops.norm_threads_override(threads)
+        t = _time(lambda: ops.rmsnorm(h, w, 1e-5, out, delta=delta), a.repeat)
+        nbytes = a.rows * a.in_features * (8 + 2 * out.element_size())
+        print(f"rmsnorm rows={a.rows} width={a.in_features} {a.dtype} threads={threads or 'rule'}: {t * 1e6:.1f} us  "
+              f"{nbytes / t / 1e12:.2f} TB/s")
+    ops.norm_threads_override(0)
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
-    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample"])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample", "stream", "rmsnorm"])
+    ap.add_argument("--megabytes", type=int, default=0, help="stream: size of the buffer (0: a range of sizes)")
+    ap.add_argument("--blocks", type=int, default=0, help="stream: workgroups (0: a range)")
+    ap.add_argument("--threads", type=int, default=0, help="rmsnorm: threads per row of the two-pass kernels (0: sweep)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--repeat", type=int, default=20)
@@ -165,7 +214,7 @@ def main(argv=None) -> None:
     ops.require_gpu()
     torch.manual_seed(0)
     {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual,
-     "sample": sample}[a.kernel](a)
+     "sample": sample, "stream": stream, "rmsnorm": rmsnorm}[a.kernel](a)
 
 
 if __name__ == "__main__":

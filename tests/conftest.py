@@ -3,6 +3,11 @@ import sys
 
 import pytest
 
+# The vendor library's algorithm for a new shape is otherwise chosen by timing (in an engine's
+# warm-up step and before a graph is recorded), which can differ from run to run and with it the
+# last bits of bfloat16 results; tests want the same bits every time.
+os.environ.setdefault("LYAPUNOV_AMD_GEMM_TUNE", "0")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -258,34 +258,44 @@ def test_float_logits_of_many_rows_are_not_rounded_to_bfloat16(ops):
 def test_library_products_keep_one_plan_per_shape(ops):
     """The vendor's library called directly: operands that are column ranges of
     wider tensors (rows further apart than they are long), both output types,
-    the same numbers as through torch, and a plan made once per shape."""
+    against the product in float64, and a plan made once per shape."""
     M, N, K = 200, 328, 136
     a_full, w_full = rnd(M, K + 24, dtype=torch.bfloat16, seed=61), rnd(N, K + 8, dtype=torch.bfloat16, scale=0.05, seed=62)
     a, w = a_full.to(DEV)[:, 8:8 + K], w_full.to(DEV)[:, :K]
     want = a.cpu().double() @ w.cpu().double().T
     bound = a.cpu().double().abs() @ w.cpu().double().abs().T
-    outs = {}
-    for mode in ("library", "torch"):
-        ops.LIBRARY_GEMM_MODE = mode
-        try:
-            for out_dtype, rel in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
-                out_full = torch.zeros(M, N + 16, dtype=out_dtype, device=DEV)
-                out = out_full[:, 16:]
-                for _ in range(3):
-                    ops.library_gemm_nt(a, w, out)
-                assert ((out.cpu().double() - want).abs() <= rel * bound + 1e-30).all()
-                assert float(out_full[:, :16].abs().max()) == 0.0       # nothing written beside the output
-                outs[mode, out_dtype] = out.cpu()
-        finally:
-            ops.LIBRARY_GEMM_MODE = "library"
+    for out_dtype, rel in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+        out_full = torch.zeros(M, N + 16, dtype=out_dtype, device=DEV)
+        out = out_full[:, 16:]
+        for _ in range(3):
+            ops.library_gemm_nt(a, w, out)
+        assert ((out.cpu().double() - want).abs() <= rel * bound + 1e-30).all()
+        assert float(out_full[:, :16].abs().max()) == 0.0       # nothing written beside the output
     before = ops.blas().lyp_library_gemm_plans()
     ops.library_gemm_nt(a, w, torch.empty(M, N, dtype=torch.float32, device=DEV))   # other stride of the output: a new plan
     ops.library_gemm_nt(a, w, torch.empty(M, N, dtype=torch.float32, device=DEV))
     assert ops.blas().lyp_library_gemm_plans() == before + 1
-    for out_dtype in (torch.float32, torch.bfloat16):
-        torch.testing.assert_close(outs["library", out_dtype], outs["torch", out_dtype], rtol=2e-2, atol=1e-3)
     with pytest.raises(ops.KernelError, match="library gemm"):
         ops.library_gemm_nt(a.float(), w, torch.empty(M, N, dtype=torch.float32, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_tiled_product_takes_operands_that_are_column_ranges(ops, dtype, monkeypatch):
+    """This package's tiled kernel with rows further apart than they are long (a column range of a
+    fused output handed on as an activation), and a refusal when a row's values are not
+    neighbours."""
+    monkeypatch.setattr(ops, "LIBRARY_GEMM", False)
+    M, N, K = 70, 96, 80
+    a_full, w_full = rnd(M, K + 24, dtype=dtype, seed=71).to(DEV), rnd(N, K + 8, dtype=dtype, scale=0.1, seed=72).to(DEV)
+    a, w = a_full[:, 8:8 + K], w_full[:, :K]
+    out_full = torch.zeros(M, N + 16, dtype=dtype, device=DEV)
+    out = out_full[:, 16:]
+    ops.gemm_nt(a, w, out)
+    want = a.cpu().double() @ w.cpu().double().T
+    torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
+    assert float(out_full[:, :16].abs().max()) == 0.0
+    with pytest.raises(ops.KernelError, match="neighbours"):      # every second column: not a row of neighbours
+        ops.gemm_nt(a_full[:, ::2][:, :K // 2], w_full[:, :K // 2].contiguous(), torch.empty(M, N, dtype=dtype, device=DEV))
 
 
 def test_gemm_float_is_true_32_bit(ops):

@@ -406,3 +406,36 @@ def test_the_largest_bfloat16_error_a_sweep_found(model_folders):
         compare_with_alone(t, got, f, dtype, "seed 1098")
         if dtype == "bfloat16":
             assert 0.05 < max(rel) < 0.08, f"the case is kept for its error of 7.3 %; it now shows {max(rel):.3f}"
+
+
+def test_bfloat16_without_the_vendor_library(model_folders, tmp_path, monkeypatch):
+    """LYAPUNOV_AMD_GEMM=own: every bfloat16 product in this package's kernels (the tiled one where
+    the library would stand).  Configuration C through a mixed trace, and the 1B shape's layer
+    through steps of 100, 58, 11 and 3 rows, against the plain model."""
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.weights import write_random_model
+
+    monkeypatch.setattr(ops, "LIBRARY_GEMM", False)
+    called = []
+    monkeypatch.setattr(ops, "library_gemm_nt", lambda *a, **k: called.append(1))
+    dtype = "bfloat16"
+    reqs = requests_for("C", {"e": 100, "f": 90, "g": 12, "h": 50})
+    t = mixed_trace(reqs)
+    compare(t, replay(folder(model_folders, "C", dtype), dtype, t), plain_for(model_folders, "C", dtype, reqs), dtype,
+            "own products, mixed")
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True)
+    d = str(tmp_path / "wide")
+    write_random_model(cfg, d, 11, dtype, init_std=0.03, norm_init_std=0.1)
+    reqs = {"a": random_tokens(150, 1000, seed=1), "b": random_tokens(60, 1000, seed=2), "c": random_tokens(20, 1000, seed=3)}
+    t = Trace(reqs)
+    t.step([("a", 100)])
+    t.step([("a", 18), ("b", 40)], want="last")
+    t.step([("a", 1), ("b", 1), ("c", 9)])
+    for _ in range(4):
+        t.step([("a", 1), ("b", 1), ("c", 1)])
+    t.step([("a", 27), ("b", 15), ("c", 7)], end=["a", "b", "c"])
+    compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "own products, wide layer")
+    assert not called
