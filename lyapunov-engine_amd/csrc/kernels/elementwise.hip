@@ -340,14 +340,16 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, siz
 }
 
 // Threads per row of the two-pass norm kernels (rows whose length or alignment keeps them from
-// the one-pass kernel).  Measured on gfx950 with 2,048 rows: a wave of 64 for every 512 values,
-// between one wave and sixteen; `g_norm_threads` (set by lyp_norm_threads_override, 0: this rule)
-// is there for that measurement.
+// the one-pass kernel).  Measured on gfx950 with 2,048 rows (kernel_bench rmsnorm): up to 1,024
+// values one or two waves are as good as any size; at 2,050 values 256 threads take 11.4 us where
+// 128 take 15.0, 320 16.1 and 512 13.9; from 4,100 values on every size from 64 to 1,024 gives
+// the same time.  `g_norm_threads` (set by lyp_norm_threads_override, 0: this rule) is there
+// for that measurement.
 static int g_norm_threads = 0;
 static int norm_threads(int H) {
   if (g_norm_threads > 0) return g_norm_threads;
-  const int waves = (H + 511) / 512;
-  return 64 * (waves < 1 ? 1 : (waves > 16 ? 16 : waves));
+  if (H <= 1024) return H <= 512 ? 64 : 128;
+  return H < 4096 ? 256 : 512;
 }
 
 // Reads `n` 16-byte words once and keeps one word per workgroup: what memory gives a kernel that

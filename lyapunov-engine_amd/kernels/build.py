@@ -133,7 +133,7 @@ def _run_with_progress(cmds: list[list[str]], what: str) -> None:
 
 
 def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str, str] | None = None,
-                  force: bool = False, link: list[str] | None = None) -> Path:
+                  force: bool = False, link: list[str] | None = None, extra_flags: list[str] | None = None) -> Path:
     """Return the path of the library, compiling it if it is not there."""
     defines = dict(defines or {})
     # For experiments: LYAPUNOV_AMD_EXTRA_DEFINES="NAME=VALUE,OTHER=1" adds macros to every HIP compile
@@ -143,7 +143,7 @@ def build_library(name: str, sources: list[str], *, hip: bool, defines: dict[str
             k, _, v = item.partition("=")
             defines[k.strip()] = v.strip() or "1"
     compiler = hipcc_path() if hip else cxx_path()
-    flags = (HIP_FLAGS if hip else CXX_FLAGS) + [f"-D{k}={v}" for k, v in sorted(defines.items())]
+    flags = (HIP_FLAGS if hip else CXX_FLAGS) + list(extra_flags or []) + [f"-D{k}={v}" for k, v in sorted(defines.items())]
     include = ["-I", str(CSRC / "kernels"), "-I", str(CSRC / "runtime")]
     out_dir = library_dir()
     target = out_dir / f"lib{name}-{_key(sources, flags + list(link or []))}.so"
@@ -195,8 +195,47 @@ def blas_library(force: bool = False) -> Path:
                          link=[f"-L{os.path.join(rocm, 'lib')}", "-lhipblaslt"])
 
 
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-g", "-O1"]
+
+
+def sanitizing() -> bool:
+    """LYAPUNOV_AMD_SANITIZE=1: host code (the cache manager and the scheduler) is compiled with the
+    address and undefined-behaviour sanitizers.  The self-test program then runs under them as it
+    is; the library so built can only be loaded by a process that has the sanitizer's runtime
+    loaded first."""
+    return os.environ.get("LYAPUNOV_AMD_SANITIZE", "0") not in ("", "0")
+
+
 def runtime_library(force: bool = False) -> Path:
+    if sanitizing():
+        return build_library("lyp_runtime_sanitized", RUNTIME_SOURCES, hip=False, force=force,
+                             link=["-fsanitize=address,undefined"], extra_flags=SANITIZE_FLAGS)
     return build_library("lyp_runtime", RUNTIME_SOURCES, hip=False, force=force)
+
+
+def runtime_selftest(force: bool = False) -> Path:
+    """The program of csrc/runtime/selftest.cpp (random requests through the scheduler and the
+    cache manager, invariants checked after every step), with the sanitizers when
+    LYAPUNOV_AMD_SANITIZE=1.  Returns the executable's path."""
+    sources = [s for s in RUNTIME_SOURCES if not s.endswith("c_api.cpp")] + ["runtime/selftest.cpp"]
+    flags = CXX_FLAGS + (SANITIZE_FLAGS if sanitizing() else [])
+    out_dir = library_dir()
+    target = out_dir / f"runtime_selftest{'_sanitized' if sanitizing() else ''}-{_key(sources, flags)}"
+    with _lock:
+        if target.exists() and not force:
+            return target
+        _say(f"compiling the runtime's self-test -> {target}")
+        tmp = target.with_suffix(f".tmp{os.getpid()}")
+        cmd = [cxx_path(), *flags, "-I", str(CSRC / "runtime"), *[str(CSRC / rel) for rel in sources], "-o", str(tmp)]
+        _run_with_progress([cmd], "runtime self-test")
+        os.replace(tmp, target)
+        for old in out_dir.glob(f"{target.name.rsplit('-', 1)[0]}-*"):
+            if old != target:
+                try:
+                    old.unlink()
+                except OSError:
+                    pass
+    return target
 
 
 def build_all(force: bool = True) -> list[Path]:

@@ -360,3 +360,30 @@ def test_a_step_ahead_that_cannot_start_does_not_break_the_planned_step(model_fo
     got, engine = run(True, True)
     assert got == want and engine._look_ahead is False and engine.steps_taken_ahead == 0
     assert "looking ahead switched off" in capsys.readouterr().err
+
+
+def test_sampled_tokens_are_the_plain_rules_at_the_engines_uniform_numbers(model_folders):
+    """Temperature, top-k and top-p through the whole engine, in 32-bit: every token is the one the
+    reference's rules give (python/lyapunov_engine/engine/sampling.py:40-69: scale, keep the k
+    largest, cut the tail beyond p, draw) on the plain model's logits, at the uniform number the
+    engine derives from (engine seed, request seed, index of the token)."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.sampling.sampler import uniform
+
+    folder = model_folders["B"]["float32"]
+    w, cfg = P.read_model(folder)
+    for seed, temperature, top_k, top_p in ((1234, 0.8, 50, 0.95), (77, 1.3, -1, 0.7), (5, 0.6, 8, 1.0)):
+        prompt = random_tokens(9, 515, seed=seed)
+        sp = L.SamplingParams(temperature=temperature, top_k=top_k, top_p=top_p, max_tokens=20, ignore_eos=True, seed=seed)
+        got = L.LLM(folder, dtype="float32", num_blocks=64, seed=3).generate([prompt], sp)[0].output_tokens
+        toks = list(prompt)
+        for i, t in enumerate(got):
+            probs = P.sample_filter(P.forward(w, cfg, toks)[-1], temperature, top_k, top_p)
+            u = uniform(3, seed, i)
+            if t != P.inverse_cdf(probs, u):
+                # only where the uniform number falls on the border between two tokens' shares
+                cdf = torch.cumsum(probs, 0)
+                assert probs[t] > 0 and float(cdf[t] - probs[t]) - 2e-5 <= u <= float(cdf[t]) + 2e-5, \
+                    f"seed {seed}, token {i}: engine {t}, plain {P.inverse_cdf(probs, u)} at u = {u}"
+            toks.append(t)
+        assert len(set(got)) > 4
