@@ -50,9 +50,8 @@ def _batch_bucket(n: int) -> int:
 class _Captured:
     TURNS = 3
 
-    def __init__(self, runner: ModelRunner, batch: int, ctx_cap: int, pool):
-        self.batch, self.ctx_cap = batch, ctx_cap
-        self.fixed = FixedStep(rows=batch, max_context=ctx_cap)
+    def __init__(self, runner: ModelRunner, fixed: FixedStep, pool):
+        self.fixed = fixed
         none64, none32 = np.zeros(0, np.int64), np.zeros(0, np.int32)
         # The step function lays the tables out, as for any step; with no live request every row is
         # padding (context 0, slot -1), so the runs below store nothing in the cache.
@@ -81,12 +80,13 @@ class _Captured:
             with torch.cuda.graph(self.graph, pool=pool):
                 self.logits = runner.model.forward(self.ctx, caches)
 
-    def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None) -> torch.Tensor:
+    def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None, counts=None) -> torch.Tensor:
         """``tokens_dev``: the token ids as an int32 tensor on the device, for a
-        step whose tokens the host does not know yet (``tokens`` is ignored)."""
+        step whose tokens the host does not know yet (``tokens`` is ignored).
+        ``counts``: new tokens per request, for a recorded step with prompt tokens."""
         self.turn = (self.turn + 1) % self.TURNS
         host = self.hosts[self.turn]
-        tables = runner.step_tables(ids, starts, None, tokens, None, fixed=self.fixed, host_for=lambda n: host.numpy())
+        tables = runner.step_tables(ids, starts, counts, tokens, None, fixed=self.fixed, host_for=lambda n: host.numpy())
         if tables.shape_key() != self.shape:
             raise StepError("a planner's arrays or launch shapes changed between two steps of one recorded shape: "
                             "in a fixed step they may depend on the step's bounds alone")
@@ -96,8 +96,15 @@ class _Captured:
         return self.logits[:len(ids)]
 
 
-class DecodeGraphs:
+class StepGraphs:
+    """Recorded steps of a model, by shape: decode steps (every request one
+    token) per (batch bucket, context bucket), and short prompt steps (one
+    request, up to ``PROMPT_TOKENS[-1]`` tokens, nothing else in the step) per
+    (token bucket, context bucket): a prompt of a few tokens is as much bound
+    by its launches as a decode step is."""
+
     MIN_CTX = 256
+    PROMPT_TOKENS = (16, 32, 64, 128)   # token rows a recorded prompt step may have
 
     def __init__(self, runner: ModelRunner, max_batch: int):
         self.runner = runner
@@ -109,6 +116,18 @@ class DecodeGraphs:
     def usable(self, entries: list) -> bool:
         return self.safe and all(len(e.tokens) == 1 and e.want == [0] for e in entries) and len(entries) <= self.max_batch
 
+    def _captured(self, fixed: FixedStep) -> _Captured:
+        key = (fixed.rows, fixed.max_context) if not fixed.tokens else (fixed.rows, fixed.max_context, fixed.tokens)
+        cap = self.captured.get(key)
+        if cap is None:
+            if self.pool is None:
+                self.pool = torch.cuda.graph_pool_handle()
+            cap = self.captured[key] = _Captured(self.runner, fixed, self.pool)
+        return cap
+
+    def _context_bucket(self, ctx_need: int) -> int:
+        return min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position)
+
     def step(self, entries: list) -> torch.Tensor:
         """Logits [len(entries), vocab]; valid until the next graph step."""
         return self.step_arrays(np.asarray([e.seq_id for e in entries], dtype=np.int64),
@@ -119,11 +138,19 @@ class DecodeGraphs:
         """The same from numpy arrays: request ids (int64), position and id of
         each request's one new token (int32); or the ids of the tokens as a
         tensor on the device (``tokens_dev``)."""
-        ctx_need = int(starts.max()) + 1
-        key = (_batch_bucket(len(ids)), min(_bucket(ctx_need, self.MIN_CTX), self.runner.max_position))
-        cap = self.captured.get(key)
-        if cap is None:
-            if self.pool is None:
-                self.pool = torch.cuda.graph_pool_handle()
-            cap = self.captured[key] = _Captured(self.runner, key[0], key[1], self.pool)
-        return cap.run(self.runner, ids, starts, tokens, tokens_dev)
+        fixed = FixedStep(rows=_batch_bucket(len(ids)), max_context=self._context_bucket(int(starts.max()) + 1))
+        return self._captured(fixed).run(self.runner, ids, starts, tokens, tokens_dev)
+
+    def prompt_usable(self, count) -> bool:
+        """Whether a step of these new-token counts (one per request) is one that is recorded as a
+        prompt step: one request, more than one token, no more than the largest bucket."""
+        return self.safe and len(count) == 1 and 1 < int(count[0]) <= self.PROMPT_TOKENS[-1]
+
+    def prompt_step_arrays(self, ids, starts, counts, tokens) -> torch.Tensor:
+        """A short prompt (or its last portion) alone in a step: logits [1, vocab] of its last token."""
+        rows = next(t for t in self.PROMPT_TOKENS if t >= int(counts.sum()))
+        fixed = FixedStep(rows=len(ids), max_context=self._context_bucket(int((starts + counts).max())), tokens=rows)
+        return self._captured(fixed).run(self.runner, ids, starts, tokens, counts=counts)
+
+
+DecodeGraphs = StepGraphs

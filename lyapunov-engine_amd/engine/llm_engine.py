@@ -221,6 +221,8 @@ class LLMEngine:
         else:
             if decoding:
                 logits = self.graphs.step_arrays(ids, start, tokens)
+            elif self.graphs is not None and bool(wants.all()) and self.graphs.prompt_usable(count):
+                logits = self.graphs.prompt_step_arrays(ids, start, count, tokens)   # a short prompt alone in its step
             else:
                 rows = (np.cumsum(count, dtype=np.int32) - 1)[wants != 0]   # the last token of each request that wants
                 logits = self.core.runner.step_arrays(ids, start, count, tokens, rows)

@@ -151,12 +151,12 @@ class ModelRunner:
         tokens (int32); all new tokens in the order of the requests (int32);
         the rows (indices into ``tokens``) whose logits are wanted (int32).
 
-        ``fixed``: the step is (a replay of) a recorded one: ``fixed.rows``
-        requests of one token each, of which the given ones are live and the
-        rest padding; the logits of every row are wanted; ``count`` and ``rows``
-        are ignored, and the requests' pages are taken as they are (no check
-        that a request holds exactly ``start`` tokens: a step started ahead of
-        the bookkeeping runs this way).  ``host_for(words)`` supplies the host
+        ``fixed``: the step is (a replay of) a recorded one (see ``FixedStep``):
+        the given requests are live and the rest of its rows padding; the logits
+        of every request's last token are wanted (``rows`` is ignored, and
+        ``count`` too in a step of one token per request), and the requests'
+        pages are taken as they are (no check that a request holds exactly
+        ``start`` tokens: a step started ahead of the bookkeeping runs this way).  ``host_for(words)`` supplies the host
         memory (an int32 numpy array of that length)."""
         n = len(ids)
         if fixed is None:
@@ -182,20 +182,32 @@ class ModelRunner:
             positions = np.arange(T, dtype=np.int32) + np.repeat(start - q_start[:-1], count)
             ctx_bound = int(ctx_len.max())
         else:
-            B = T = fixed.rows
+            B, T = fixed.rows, fixed.token_rows
             if n > B:
                 raise StepError(f"{n} requests in a recorded step of {B} rows")
-            q_start = np.arange(B + 1, dtype=np.int32)
-            count = np.ones(B, dtype=np.int32)
+            live = np.ones(n, dtype=np.int32) if count is None or not fixed.tokens else np.asarray(count, dtype=np.int32)
+            if n and int(live.min()) < 1:
+                raise StepError("a request brings no tokens")
+            used = int(live.sum())
+            if used > T or tokens.size != used:
+                raise StepError(f"{tokens.size} tokens for requests that bring {used}, in a recorded step of {T} token rows")
+            count = np.zeros(B, dtype=np.int32)
+            count[:n] = live
+            if not fixed.tokens:
+                count[n:] = 1          # a padded row of a decode step is a token row of its own
+            q_start = np.zeros(B + 1, dtype=np.int32)
+            np.cumsum(count, out=q_start[1:])
+            first = np.zeros(B, dtype=np.int32)
+            first[:n] = start
             ctx_len = np.zeros(B, dtype=np.int32)
-            ctx_len[:n] = start
-            ctx_len[:n] += 1
-            positions = np.zeros(B, dtype=np.int32)
-            positions[:n] = start
-            full = np.zeros(B, dtype=np.int32)
-            full[:n] = tokens
-            tokens, start = full, positions
-            rows = np.arange(B, dtype=np.int32)
+            ctx_len[:n] = first[:n] + live
+            positions = np.zeros(T, dtype=np.int32)
+            positions[:used] = np.arange(used, dtype=np.int32) + np.repeat(first[:n] - q_start[:n], live)
+            full = np.zeros(T, dtype=np.int32)
+            full[:used] = tokens
+            tokens, start = full, first
+            # the logits of every request's last token (row 0 for a padded request of a prompt step)
+            rows = np.maximum(q_start[1:] - 1, 0).astype(np.int32)
             ctx_bound = fixed.max_context
             if n and int(ctx_len.max()) > ctx_bound:
                 raise StepError(f"a request of {int(ctx_len.max())} tokens in a step recorded for {ctx_bound}")
@@ -250,12 +262,13 @@ class ModelRunner:
                 elif n:
                     ps = gc.page_size
                     self.cache.export(ids, g, bt[:n], slots[:n] if g == 0 else None)
-                    at = positions[:n]
-                    slot_map[:n] = bt[np.arange(n), at // ps] * ps + at % ps
+                    used = int(q_start[n])
+                    at = positions[:used]
+                    slot_map[:used] = bt[np.repeat(np.arange(n), count[:n]), at // ps] * ps + at % ps
             except CacheError as err:
                 raise StepError(str(err)) from None
             if fixed is not None:
-                slot_map[n:] = -1
+                slot_map[int(q_start[n]):] = -1
         for i, arr in enumerate(plan_arrays):
             sec(len(sizes) - len(plan_arrays) + i)[:] = arr
         return StepTables(host=host, names=names, sizes=sizes, offsets=offsets, T=T, B=B, R=int(rows.size),

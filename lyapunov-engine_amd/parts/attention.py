@@ -45,9 +45,25 @@ class AttentionWork(StepPlanner):
 
     def plan(self, batch: StepBatch) -> tuple:
         none = np.zeros(0, dtype=np.int32)
-        if batch.fixed is not None:
+        fixed = batch.fixed
+        if fixed is not None and not fixed.tokens:
             return ({"tile_seq": none, "tile_q0": none},
-                    dict(n_tiles=0, tile_keys=(0, 0), n_dec=batch.fixed.rows, max_ctx_dec=batch.fixed.max_context))
+                    dict(n_tiles=0, tile_keys=(0, 0), n_dec=fixed.rows, max_ctx_dec=fixed.max_context))
+        if fixed is not None:
+            # A recorded step with prompt tokens: every request goes in tiles (one with a single
+            # token too), in as many list entries as the step can ever need; entries past the live
+            # tiles start beyond any request's tokens, which the kernels take as "nothing to do".
+            n_tiles = -(-fixed.token_rows // PREFILL_TILE) + fixed.rows
+            tile_seq = np.zeros(n_tiles, dtype=np.int32)
+            tile_q0 = np.full(n_tiles, 1 << 30, dtype=np.int32)
+            at = n_tiles
+            for b in range(batch.B - 1, -1, -1):       # live tiles at the list's heavy end
+                for q0 in range(-(-int(batch.count[b]) // PREFILL_TILE) - 1, -1, -1):
+                    if batch.ctx_len[b] > 0:
+                        at -= 1
+                        tile_seq[at], tile_q0[at] = b, q0 * PREFILL_TILE
+            return ({"tile_seq": tile_seq, "tile_q0": tile_q0},
+                    dict(n_tiles=n_tiles, tile_keys=(PREFILL_TILE, fixed.max_context), n_dec=0, max_ctx_dec=0))
         start, count, ctx_len = batch.start, batch.count, batch.ctx_len
         several = np.flatnonzero(count > 1)
         dec = np.flatnonzero(count == 1).astype(np.int32)

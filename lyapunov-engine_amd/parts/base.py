@@ -125,12 +125,21 @@ class LayerCache:
 @dataclass
 class FixedStep:
     """A step whose shapes are frozen so that it can be recorded once and
-    replayed: ``rows`` requests of one new token each (rows past the live ones
-    are padding: context 0, cache slot -1, the spare state slot), contexts of
-    at most ``max_context`` tokens."""
+    replayed.  ``tokens == 0``: ``rows`` requests of one new token each (rows
+    past the live ones are padding: context 0, cache slot -1, the spare state
+    slot).  ``tokens > 0``: up to ``rows`` requests that bring up to ``tokens``
+    new tokens between them, a request's tokens side by side as in any step;
+    the token rows past the live ones are padding (position 0, cache slot -1,
+    owned by no request), and so are requests past the live ones (no tokens,
+    context 0).  Contexts are at most ``max_context`` tokens either way."""
 
     rows: int
     max_context: int
+    tokens: int = 0
+
+    @property
+    def token_rows(self) -> int:
+        return self.tokens or self.rows
 
 
 @dataclass

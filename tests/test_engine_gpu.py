@@ -387,3 +387,74 @@ def test_sampled_tokens_are_the_plain_rules_at_the_engines_uniform_numbers(model
                     f"seed {seed}, token {i}: engine {t}, plain {P.inverse_cdf(probs, u)} at u = {u}"
             toks.append(t)
         assert len(set(got)) > 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_prompts_run_as_recorded_steps(model_folders, dtype):
+    """A prompt of up to 128 tokens alone in its step is replayed from a graph recorded for the next
+    bucket of token rows (the rows past its tokens are padding): the tokens it leads to are those of
+    the engine without graphs, for lengths at and around the buckets' edges, for a prompt whose last
+    portion starts in the middle of its pages, and with the graphs used again for other prompts."""
+    import lyapunov_engine_amd as L
+
+    folder = model_folders["B"][dtype]
+    lengths = [2, 5, 16, 17, 40, 64, 100, 128, 129, 200]
+    prompts = [random_tokens(n, 515, seed=300 + n) for n in lengths]
+    sp = L.SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True)
+
+    def run(graphs):
+        llm = L.LLM(folder, dtype=dtype, num_blocks=64, block_size=16, max_num_batched_tokens=128, enable_graphs=graphs)
+        outs = [llm.generate([p], sp)[0].output_tokens for p in prompts]       # one at a time: alone in its step
+        outs += [llm.generate([p], sp)[0].output_tokens for p in prompts[:4]]   # the recorded steps again
+        return outs, llm.engine
+
+    with_graphs, engine = run(True)
+    prompt_keys = sorted(key for key in engine.graphs.captured if len(key) == 3)
+    assert {key[2] for key in prompt_keys} == {16, 32, 64, 128}, prompt_keys
+    eager, _ = run(False)
+    assert with_graphs == eager
+    assert with_graphs[:4] == with_graphs[len(prompts):]
+    for p, got in zip(prompts[:8], with_graphs):
+        check_against_plain(folder, p, got, dtype)
+    engine.core.cache.check()
+    assert engine.core.cache.num_requests() == 0
+
+
+def test_a_recorded_prompt_step_of_two_requests_equals_the_eager_step(model_folders):
+    """The table builder's recorded layout with prompt tokens, beyond what the engine uses it for:
+    two requests in one recorded step (a portion of 9 tokens from position 20 and a whole prompt of
+    30), replayed with other requests and lengths, against the same steps run eagerly."""
+    import numpy as np
+
+    from lyapunov_engine_amd.engine.core import EngineCore, StepEntry
+    from lyapunov_engine_amd.engine.graphs import _Captured
+    from lyapunov_engine_amd.parts.base import FixedStep
+
+    core = EngineCore.from_folder(model_folders["C"]["float32"], dtype="float32", num_blocks=64, block_size=16)
+    cache, runner = core.cache, core.runner
+    cap = _Captured(runner, FixedStep(rows=2, max_context=256, tokens=64), torch.cuda.graph_pool_handle())
+    toks = {i: random_tokens(90, 320, seed=40 + i) for i in range(4)}
+    for i in toks:
+        cache.add(i)
+
+    def both(entries):
+        for e in entries:
+            cache.extend(e.seq_id, e.start + len(e.tokens))
+        eager = core.step(entries).clone()
+        ids = np.asarray([e.seq_id for e in entries], dtype=np.int64)
+        starts = np.asarray([e.start for e in entries], dtype=np.int32)
+        counts = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
+        flat = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+        replayed = cap.run(runner, ids, starts, flat, counts=counts).clone()
+        for e in entries:
+            cache.commit(e.seq_id, e.start + len(e.tokens))
+        torch.testing.assert_close(replayed, eager, rtol=1e-5, atol=1e-5)
+        return eager
+
+    cache.extend(0, 20)
+    core.step([StepEntry(0, toks[0][:20], 0, [])])
+    cache.commit(0, 20)
+    both([StepEntry(0, toks[0][20:29], 20, [8]), StepEntry(1, toks[1][:30], 0, [29])])
+    both([StepEntry(2, toks[2][:64], 0, [63])])                              # one request, every token row live
+    both([StepEntry(1, toks[1][30:31], 30, [0]), StepEntry(0, toks[0][29:70], 29, [40])])   # a single token beside a portion
+    both([StepEntry(3, toks[3][:2], 0, [1]), StepEntry(2, toks[2][64:66], 64, [1])])

@@ -471,12 +471,12 @@ def register_toy3():
 
     class Segments(StepPlanner):
         """Per request: 1 if it starts from nothing.  meta: the most tokens any request brings
-        (the number of rounds the scan takes; 1 in a fixed step)."""
+        (the number of rounds the scan takes; in a recorded step the most it could bring)."""
         key = ("toy_segments",)
 
         def plan(self, batch):
             fresh = (batch.ctx_len - batch.count == 0).astype(np.int32)
-            longest = 1 if batch.fixed is not None else int(batch.count.max())
+            longest = int(batch.count.max()) if batch.fixed is None else (batch.fixed.tokens or 1)
             return {"fresh": fresh}, {"longest": longest}
 
     class ScanOnDevice(Mixer):
@@ -607,6 +607,11 @@ def test_a_stateful_mixer_with_lists_of_its_own_decodes_through_graphs(tmp_path,
             for t in with_graphs[0]:
                 assert t == int(toy3_plain(folder, toks)[-1].argmax())
                 toks.append(t)
+        # a short prompt alone in its step is a recorded step too (16 token rows, of which 12 are live)
+        llm = L.LLM(folder, dtype=dtype, num_blocks=64, block_size=4, max_num_seqs=4)
+        one = llm.generate([prompts[0]], L.SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))[0].output_tokens
+        assert any(len(key) == 3 for key in llm.engine.graphs.captured)
+        assert one == with_graphs[0][:8]
     finally:
         ARCHITECTURES.unregister("ToyScanForCausalLM")
         MIXERS.unregister("toy_scan_on_device")
