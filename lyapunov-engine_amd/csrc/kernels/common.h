@@ -172,6 +172,17 @@ struct Mma32<bf16_t> {
   }
 };
 
+// ------------------------------------------------------------------- maxima
+// A value and where it stands; of two equal values the one that stands first wins.
+struct ArgMax {
+  float v;
+  int i;
+};
+__device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
 // ------------------------------------------------------------- host-side glue
 // Every exported function returns 0 or a negative code and leaves a message
 // for lyp_last_error().

@@ -12,6 +12,7 @@
 // sizes of the product alone (no atomics), so a token's result does not depend
 // on which other tokens are in the batch beyond the choice of kernel, which
 // follows M.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -457,6 +458,104 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   }
 }
 
+// ------------------------------------------------------------ the output head
+// Float logits of few rows (a decode step's) against a matrix of very many rows: C[M, N] = A . W^T
+// with N in the hundred thousands.  The work is one long read of W, and such a read is fastest
+// with few, long-lived waves (two workgroups of four waves per compute unit reached 6.1 TB/s in a
+// plain read of this size, one wave per 16 rows of W as gemm_skinny_kernel would have it 4.6-4.8):
+// a wave here takes 16 rows of W at a time, all of K, and then the next 16 that are its turn.
+// With `cand` every workgroup also leaves, per token, the largest logit among the rows it computed
+// and the first place it stands at: cand[token][workgroup].  The sampler then needs no pass over
+// the row to find the maximum.
+template <typename T, int MB>
+__global__ __launch_bounds__(256) void lm_head_kernel(const T* __restrict__ A, const T* __restrict__ W,
+                                                      float* __restrict__ C, int M, int N, int K, int lda, int ldw,
+                                                      int ldc, ArgMax* __restrict__ cand) {
+  using MM = Mma16Wide<T>;
+  using Frag = typename MM::Frag;
+  constexpr int NF = 16 / MM::kElems;
+  constexpr int kWaves = 4;
+  __shared__ ArgMax s_best[kWaves][MB][16];
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int r = lane % 16, j = lane / 16;
+  const int row_blocks = (N + 15) / 16, chunks = K / 64;
+  const T* ap[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) ap[b] = A + static_cast<size_t>(min(b * 16 + r, M - 1)) * lda + j * MM::kElems;
+  ArgMax best[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) best[b] = ArgMax{LYP_NEG_INF, 0x7fffffff};
+
+  for (int blk = blockIdx.x * kWaves + wave; blk < row_blocks; blk += gridDim.x * kWaves) {
+    const int n0 = blk * 16;
+    const T* wp = W + static_cast<size_t>(min(n0 + r, N - 1)) * ldw + j * MM::kElems;
+    f32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto chunks_at = [&](auto count, int c) {
+      constexpr int U = decltype(count)::value;
+      Frag wf[U][NF];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) wf[u][f] = *reinterpret_cast<const Frag*>(wp + (c + u) * 64 + f * 4 * MM::kElems);
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        Frag xf[U][NF];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int f = 0; f < NF; ++f) xf[u][f] = *reinterpret_cast<const Frag*>(ap[b] + (c + u) * 64 + f * 4 * MM::kElems);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[u][f], xf[u][f], acc[b]);
+      }
+    };
+    int c = 0;
+    for (; c + 4 <= chunks; c += 4) chunks_at(std::integral_constant<int, 4>{}, c);
+    for (; c < chunks; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
+
+    // acc[b][i]: row n0 + 4 j + i of W (a logit's index), token 16 b + r
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = 16 * b + r, n = n0 + 4 * j;
+      ArgMax mine{LYP_NEG_INF, 0x7fffffff};
+      if (m < M) {
+        float* crow = C + static_cast<size_t>(m) * ldc + n;
+        if (n + 3 < N && ldc % 4 == 0) {
+          *reinterpret_cast<f32x4*>(crow) = acc[b];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) crow[i] = acc[b][i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) mine = better(mine, ArgMax{acc[b][i], n + i});
+      }
+      if (cand) {
+#pragma unroll
+        for (int off = 16; off < kWave; off *= 2) mine = better(mine, ArgMax{__shfl_xor(mine.v, off, kWave), __shfl_xor(mine.i, off, kWave)});
+        best[b] = better(best[b], mine);
+      }
+    }
+  }
+  if (cand) {
+    if (j == 0)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) s_best[wave][b][r] = best[b];
+    __syncthreads();
+    for (int t = threadIdx.x; t < MB * 16; t += blockDim.x) {
+      if (t >= M) continue;
+      ArgMax a = s_best[0][t / 16][t % 16];
+      for (int w = 1; w < kWaves; ++w) a = better(a, s_best[w][t / 16][t % 16]);
+      cand[static_cast<size_t>(t) * gridDim.x + blockIdx.x] = a;
+    }
+  }
+}
+
 static bool skinny_ok(int M, int K, int lda, int ldw, const void* A, const void* W, int dtype) {
   const int vec = dtype == kF32 ? 4 : 8;
   return M >= 1 && M <= 64 && K % 64 == 0 && lda % vec == 0 && ldw % vec == 0 &&
@@ -572,6 +671,37 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
 #undef LYP_GEMM
   LYP_LAUNCH_CHECK("gemm_nt");
   return 0;
+}
+
+// Float logits C[M, N] = A . W^T for up to 64 rows (see lm_head_kernel), with `blocks` workgroups
+// (0: two per compute unit of this machine's 256, as a plain read of such a matrix likes it).
+// cand (optional): [M][blocks] pairs of (float, int32) that receive every workgroup's largest logit
+// per row and its index.  Returns the number of workgroups used (the stride of cand), 0 when the
+// kernel does not take the operands (then use lyp_gemm_nt), negative on error.
+extern "C" int lyp_lm_head(const void* A, const void* W, float* C, int dtype, int M, int N, int K, int lda, int ldw,
+                           int ldc, void* cand, int blocks, hipStream_t stream) {
+  LYP_REQUIRE(N > 0 && K > 0 && ldc >= N && blocks >= 0 && blocks <= 4096, "lm_head: N=%d K=%d stride %d blocks %d", N, K,
+              ldc, blocks);
+  if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 0;
+  if (blocks == 0) blocks = 512;
+  blocks = std::min(blocks, (N + 63) / 64);  // no workgroup without a wave's worth of rows
+  ArgMax* cd = static_cast<ArgMax*>(cand);
+#define LYP_HEAD(T, MB) \
+  lm_head_kernel<T, MB><<<blocks, 256, 0, stream>>>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, cd)
+#define LYP_HEAD_T(T)                  \
+  do {                                 \
+    if (M <= 16) LYP_HEAD(T, 1);       \
+    else if (M <= 32) LYP_HEAD(T, 2);  \
+    else if (M <= 48) LYP_HEAD(T, 3);  \
+    else LYP_HEAD(T, 4);               \
+  } while (0)
+  if (dtype == kF32) LYP_HEAD_T(float);
+  else if (dtype == kBF16) LYP_HEAD_T(bf16_t);
+  else LYP_REQUIRE(false, "lm_head: unknown dtype %d", dtype);
+#undef LYP_HEAD_T
+#undef LYP_HEAD
+  LYP_LAUNCH_CHECK("lm_head");
+  return blocks;
 }
 
 // How many partial sums lyp_gemm_nt_parts would produce for this product; 0 if

@@ -28,15 +28,6 @@ __device__ __forceinline__ uint32_t order_key(float z) {
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
-struct ArgMax {
-  float v;
-  int i;
-};
-__device__ __forceinline__ ArgMax better(ArgMax a, ArgMax b) {
-  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
-  return a;
-}
-
 __device__ __forceinline__ ArgMax block_argmax(ArgMax a, ArgMax* scratch) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
 #pragma unroll
@@ -296,7 +287,7 @@ __device__ uint32_t select_in_list(const uint32_t* list, int n, uint32_t floor_k
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int32_t* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
-    const ArgMax* __restrict__ cand, int32_t* __restrict__ out, int32_t* __restrict__ mirror) {
+    const ArgMax* __restrict__ cand, int n_cand, int32_t* __restrict__ out, int32_t* __restrict__ mirror) {
   __shared__ ArgMax s_arg[kSampleThreads / kWave];
   __shared__ int s_cnt[kSampleThreads / kWave];
   __shared__ float s_f[kSampleThreads / kWave];
@@ -316,7 +307,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
   ArgMax am{LYP_NEG_INF, 0x7fffffff};
   if (cand) {  // the pieces' winners instead of the whole row
-    if (tid < kArgmaxChunks) am = cand[row * kArgmaxChunks + tid];
+    for (int i = tid; i < n_cand; i += kSampleThreads) am = better(am, cand[static_cast<size_t>(row) * n_cand + i]);
   } else {
     for (int i = tid; i < V; i += kSampleThreads) am = better(am, ArgMax{x[i], i});
   }
@@ -574,8 +565,30 @@ extern "C" int lyp_sample(const float* logits, int ld, int rows, int V, const fl
   }
   ArgMax* cand = static_cast<ArgMax*>(workspace);
   if (cand) argmax_chunks_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(logits, ld, V, cand);
-  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, cand, out,
-                                                      mirror);
+  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform, cand,
+                                                      kArgmaxChunks, out, mirror);
+  LYP_LAUNCH_CHECK("sample");
+  return 0;
+}
+
+// The same for logits whose maxima are known in pieces already: cand [rows][n_cand] (value, index)
+// pairs, each the largest logit of one piece of its row and the first place it stands at, the
+// pieces together covering the row (what lyp_lm_head leaves behind).  One kernel instead of two.
+extern "C" int lyp_sample_cand(const float* logits, int ld, int rows, int V, const float* temperature,
+                               const int32_t* top_k, const float* top_p, const float* uniform, const void* cand,
+                               int n_cand, int32_t* out, int32_t* mirror, hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
+  LYP_REQUIRE(cand && n_cand > 0, "sample: %d candidates per row", n_cand);
+  if (rows == 0) return 0;
+  LYP_REQUIRE(rows <= 65535, "sample: %d rows in one launch", rows);
+  if (mirror) {
+    void* mapped = nullptr;
+    LYP_REQUIRE(hipHostGetDevicePointer(&mapped, mirror, 0) == hipSuccess && mapped,
+                "sample: the mirror is no pinned host memory that the device can write");
+    mirror = static_cast<int32_t*>(mapped);
+  }
+  sample_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, ld, V, temperature, top_k, top_p, uniform,
+                                                      static_cast<const ArgMax*>(cand), n_cand, out, mirror);
   LYP_LAUNCH_CHECK("sample");
   return 0;
 }

@@ -17,6 +17,12 @@ int lyp_sample(const float* logits, int ld, int rows, int V, const float* temper
                const float* top_p, const float* uniform, void* workspace, int32_t* out, int32_t* mirror,
                hipStream_t stream);
 
+// lyp_sample for logits whose row maxima are known in pieces: cand [rows][n_cand] pairs of (float
+// value, int32 index), the largest logit of each piece and the first place it stands at.
+int lyp_sample_cand(const float* logits, int ld, int rows, int V, const float* temperature, const int32_t* top_k,
+                    const float* top_p, const float* uniform, const void* cand, int n_cand, int32_t* out,
+                    int32_t* mirror, hipStream_t stream);
+
 // lyp_sample for callers that cannot allocate device memory: code under graph
 // capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
 // counterpart in the reference (whose sampler, engine/sampling.py:15-72, runs

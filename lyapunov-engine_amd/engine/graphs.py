@@ -93,7 +93,11 @@ class _Captured:
         # one small kernel reads the pinned table (and the device's token ids) into place
         ops.table_load(host, self.dev, None if tokens_dev is None else tokens_dev[:len(ids)], self.token_words)
         self.graph.replay()
-        return self.logits[:len(ids)]
+        out = self.logits[:len(ids)]
+        cand = getattr(self.logits, "argmax_candidates", None)
+        if cand is not None:     # what the head's kernel left for the sampler travels with the rows
+            out.argmax_candidates = cand
+        return out
 
 
 class StepGraphs:

@@ -73,6 +73,10 @@ def core() -> ctypes.CDLL:
                                     c_int, c_void_p]
         lib.lyp_sample.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_void_p, c_void_p]
+        lib.lyp_sample_cand.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_void_p, c_void_p, c_void_p]
+        lib.lyp_lm_head.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void_p, c_int, c_void_p]
         lib.lyp_sample_workspace.argtypes = [c_int]
         lib.lyp_sample_workspace.restype = c_longlong
         lib.lyp_norm_threads_override.argtypes = [c_int]
@@ -649,6 +653,34 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     return cast(gemm_nt(x, w, out), out_dtype)
 
 
+LM_HEAD_MAX_ROWS = 16     # beyond that the activations are read again per 16 rows and the general products are ahead
+LM_HEAD_BLOCKS = 1024     # workgroups of the output-head kernel (measured: 256 129 us, 512 116, 1024 104, 2048 105)
+
+
+def lm_head(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """Float logits x @ w.T for the output head [vocab, hidden].  Few rows (a
+    decode step's) take a kernel of their own that reads the matrix with few
+    long-lived waves and leaves, beside the logits, every workgroup's largest
+    logit per row: the tensor returned then carries ``argmax_candidates`` (a
+    tensor [rows, workgroups, 2] of (value bits, index) pairs), which ``sample``
+    uses instead of a pass over the row.  Anything else goes through ``linear``."""
+    M, K = x.shape
+    if M <= LM_HEAD_MAX_ROWS and w.dtype == x.dtype and w.shape[1] == K and w.stride(1) == 1 and x.stride(1) == 1:
+        _dev(x)
+        lib = core()
+        V = w.shape[0]
+        out = torch.empty((M, V), dtype=torch.float32, device=x.device)
+        cand = torch.empty((M, LM_HEAD_BLOCKS, 2), dtype=torch.int32, device=x.device)
+        rc = lib.lyp_lm_head(_p(x), _p(w), _p(out), _code(x.dtype), M, V, K, x.stride(0), w.stride(0), out.stride(0),
+                             _p(cand), LM_HEAD_BLOCKS, _stream())
+        if rc < 0:
+            _check(rc, lib)
+        if rc > 0:
+            out.argmax_candidates = cand if rc == LM_HEAD_BLOCKS else cand.view(-1)[:M * rc * 2].view(M, rc, 2)
+            return out
+    return linear(x, w, out_dtype=torch.float32)
+
+
 def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """Add up the partial sums ``linear(..., may_split=True)`` may return."""
     if parts.dim() == 2:
@@ -783,7 +815,9 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     the search for each row's maximum is spread over the chip.  ``mirror``: pinned
     host memory (int32, a row each) that receives the tokens as well, readable
     once the work on the stream up to here is done."""
-    _dev(logits, temperature, top_k, top_p, uniform, out, workspace)
+    _dev(temperature, top_k, top_p, uniform, out, workspace)
+    if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be a 2-d GPU tensor whose rows are contiguous")
     if mirror is not None:
         _pinned(mirror, torch.int32, "sample: the mirror")
         if mirror.numel() != out.numel():
@@ -795,8 +829,17 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if any(t.numel() != R for t in (temperature, top_k, top_p, uniform, out)):
         raise KernelError("sample: one parameter per row")
     lib = core()
+    cand = getattr(logits, "argmax_candidates", None)
+    if cand is not None:   # the head's kernel left the row maxima in pieces: no pass over the row for them
+        if cand.dtype != torch.int32 or cand.dim() != 3 or cand.shape[0] < R or cand.shape[2] != 2 or \
+                not cand.is_contiguous() or cand.device != logits.device:
+            raise KernelError("sample: the logits' argmax candidates must be a contiguous int32 tensor [rows, pieces, 2]")
+        _check(lib.lyp_sample_cand(_p(logits), logits.stride(0), R, V, _p(temperature), _p(top_k), _p(top_p),
+                                   _p(uniform), _p(cand), cand.shape[1], _p(out),
+                                   mirror.data_ptr() if mirror is not None else None, _stream()), lib)
+        return out
     if workspace is not None and workspace.numel() < lib.lyp_sample_workspace(R):
         raise KernelError("sample: workspace too small")
-    _check(lib.lyp_sample(_p(logits), V, R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform), _p(workspace),
-                          _p(out), mirror.data_ptr() if mirror is not None else None, _stream()), lib)
+    _check(lib.lyp_sample(_p(logits), logits.stride(0), R, V, _p(temperature), _p(top_k), _p(top_p), _p(uniform),
+                          _p(workspace), _p(out), mirror.data_ptr() if mirror is not None else None, _stream()), lib)
     return out

@@ -163,7 +163,7 @@ class DecoderModel(Part):
         if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
             delta = delta.run()
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
-        return ops.linear(x, self.lm_head, out_dtype=torch.float32)
+        return ops.lm_head(x, self.lm_head)
 
 
 def build_model(spec: ModelSpec) -> DecoderModel:

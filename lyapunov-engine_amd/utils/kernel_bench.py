@@ -5,6 +5,7 @@
     python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 8 --out-features 16384 --in-features 2048
     python -m lyapunov_engine_amd.utils.kernel_bench residual --rows 8 --out-features 2048 --in-features 8192
     python -m lyapunov_engine_amd.utils.kernel_bench sample --rows 8 --vocab 128256 --top-k 50 --top-p 0.9
+    python -m lyapunov_engine_amd.utils.kernel_bench head --rows 8
     python -m lyapunov_engine_amd.utils.kernel_bench stream --megabytes 64
     python -m lyapunov_engine_amd.utils.kernel_bench rmsnorm --rows 2048 --in-features 4100 --threads 256
 
@@ -111,6 +112,20 @@ def linear(a) -> None:
           f"{flops / t / 1e12:.1f} TFLOP/s  {w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
 
 
+def head(a) -> None:
+    """The output head's kernel: float logits of ``rows`` rows, with every workgroup's row maxima."""
+    dt, dev = _dtype(a.dtype), a.device
+    x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
+    w = torch.randn(a.vocab, a.in_features, device=dev, dtype=dt) * 0.02
+    for blocks in ([a.blocks] if a.blocks else [256, 512, 1024, 2048]):
+        ops.LM_HEAD_BLOCKS = blocks
+        t = _time(lambda: ops.lm_head(x, w), a.repeat)
+        print(f"head rows={a.rows} {a.vocab}x{a.in_features} {a.dtype} in {blocks} workgroups: {t * 1e6:.1f} us  "
+              f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
+    t = _time(lambda: ops.linear(x, w, out_dtype=torch.float32), a.repeat)
+    print(f"(the weight-streaming product, one wave per 16 rows: {t * 1e6:.1f} us)")
+
+
 def residual(a) -> None:
     """The product that adds to the float residual stream and prepares the next norm."""
     dt, dev = _dtype(a.dtype), a.device
@@ -187,7 +202,7 @@ def rmsnorm(a) -> None:
 
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
-    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample", "stream", "rmsnorm"])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample", "stream", "rmsnorm", "head"])
     ap.add_argument("--megabytes", type=int, default=0, help="stream: size of the buffer (0: a range of sizes)")
     ap.add_argument("--blocks", type=int, default=0, help="stream: workgroups (0: a range)")
     ap.add_argument("--threads", type=int, default=0, help="rmsnorm: threads per row of the two-pass kernels (0: sweep)")
@@ -214,7 +229,7 @@ def main(argv=None) -> None:
     ops.require_gpu()
     torch.manual_seed(0)
     {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual,
-     "sample": sample, "stream": stream, "rmsnorm": rmsnorm}[a.kernel](a)
+     "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head}[a.kernel](a)
 
 
 if __name__ == "__main__":

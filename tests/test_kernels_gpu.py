@@ -788,6 +788,47 @@ def test_attention_finds_a_key_anywhere_in_8192(ops, dtype, kind, nh, nkv, hd):
         torch.testing.assert_close(got, want, rtol=1e-2, atol=1e-2, msg=lambda m: f"request {b}, key {f}: {m}")
 
 
+# ----------------------------------------------------------------- output head
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,V,K", [(1, 1003, 128), (8, 32000, 192), (16, 515, 64), (11, 2051, 256), (3, 128256, 64)])
+def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
+    """The head's own kernel (few long-lived waves walking the matrix): float logits against the
+    product in float64, and per row the pieces' maxima: the largest of them is the row's largest
+    logit at the first place it stands.  Vocabularies that are no multiple of 16 or of 4; 1 to 16
+    rows; few workgroups (every wave walks many row blocks) and many."""
+    x = rnd(M, K, dtype=dtype, seed=81)
+    w = rnd(V, K, dtype=dtype, scale=0.2, seed=82)
+    w[V // 3] = w[7]                                   # two equal logits in every row: the first one is to win
+    want = x.double() @ w.double().T
+    for blocks in (8, 512):
+        monkeypatch.setattr(ops, "LM_HEAD_BLOCKS", blocks)
+        out = ops.lm_head(x.to(DEV), w.to(DEV))
+        torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 1e-2))
+        cand = out.argmax_candidates.cpu()
+        assert cand.shape[0] == M and cand.shape[2] == 2 and cand.shape[1] <= blocks
+        values, places = cand[..., 0].contiguous().view(torch.float32), cand[..., 1]
+        got = out.cpu()
+        for m in range(M):
+            best = int(values[m].argmax())
+            top = float(got[m].max())
+            assert float(values[m, best]) == top
+            first = int((got[m] == top).nonzero()[0])
+            assert int(places[m][values[m] == top].min()) == first
+        # the sampler takes them: greedy and drawn tokens equal those found with a pass over the row
+        R = M
+        temperature = torch.tensor(([0.0, 0.9, 1.2] * R)[:R]).to(DEV)
+        top_k = torch.tensor(([-1, 40, -1] * R)[:R], dtype=torch.int32).to(DEV)
+        top_p = torch.tensor(([1.0, 1.0, 0.8] * R)[:R]).to(DEV)
+        u = torch.rand(R, generator=torch.Generator().manual_seed(3)).to(DEV)
+        a, b = torch.empty(R, dtype=torch.int32, device=DEV), torch.empty(R, dtype=torch.int32, device=DEV)
+        ops.sample(out, temperature, top_k, top_p, u, a)
+        plain_logits = out.clone()                      # a copy carries no candidates
+        assert getattr(plain_logits, "argmax_candidates", None) is None
+        ops.sample(plain_logits, temperature, top_k, top_p, u, b, ops.sample_workspace(R, DEV))
+        assert a.tolist() == b.tolist()
+        assert a[0] == int(got[0].argmax())
+
+
 # --------------------------------------------------------------------- sampler
 def test_sampler_greedy_and_draws(ops):
     V = 1003
