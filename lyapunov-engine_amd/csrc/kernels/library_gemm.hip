@@ -70,6 +70,7 @@ State& state() {
 int g_tuning_candidates = 0;   // > 1: a new plan is chosen by measurement among this many candidates
 bool g_tuning_no_workspace = false;  // a new plan's algorithm is one that needs no workspace
 constexpr int kMostCandidates = 32;
+constexpr float kTuningMargin = 0.95f;  // what a candidate's time has to stay under, relative to the heuristic's first choice
 bool g_tuning_all = true;      // screen all of the library's solutions, not only the heuristic's first few
 
 
@@ -131,7 +132,11 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
         if (fastest < 0.f || ms < fastest) fastest = ms;
       }
       if (c == 0) *first_ms = fastest;
-      if (fastest >= 0.f && (best_ms < 0.f || fastest < best_ms)) best_ms = fastest, best = c;
+      // Another candidate has to be ahead of the heuristic's first choice by a clear margin: a
+      // few per cent are within what two timings of the same kernel differ by, and what wins
+      // such a toss here has lost by more than that inside a model step.
+      const float bar = (c > 0 && *first_ms >= 0.f && best == 0) ? kTuningMargin * best_ms : best_ms;
+      if (fastest >= 0.f && (best_ms < 0.f || fastest < bar)) best_ms = fastest, best = c;
     }
   }
   if (e0) (void)hipEventDestroy(e0);
