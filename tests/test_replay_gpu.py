@@ -439,3 +439,42 @@ def test_bfloat16_without_the_vendor_library(model_folders, tmp_path, monkeypatc
     t.step([("a", 27), ("b", 15), ("c", 7)], end=["a", "b", "c"])
     compare(t, replay(d, dtype, t), plain_logits(d, reqs), dtype, "own products, wide layer")
     assert not called
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_prompts_do_not_depend_on_their_portions(tmp_path, dtype):
+    """The 1B shape's layer over 20,000 tokens, where no plain model reaches in the time a test has:
+    the logits at the end of the prompt and of 3 decoded tokens are the same whether the prompt came
+    in portions of 4,096 or of 777 tokens (in 32-bit to 5e-5 of the largest logit; in bfloat16 to what
+    the kernels' roundings differ by, see trace_util).  Block tables are 1,250 entries wide here and
+    a late portion's keys are cut into runs."""
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import TOL_ALONE
+
+    cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               max_position_embeddings=32768, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                 original_max_position_embeddings=8192))
+    d = str(tmp_path / "wide")
+    write_random_model(cfg, d, 14, dtype, init_std=0.03, norm_init_std=0.1)
+    n = 20000
+    reqs = {"a": random_tokens(n + 3, 1000, seed=8)}
+    got = {}
+    for portion in (4096, 777):
+        t = Trace(reqs)
+        left = n
+        while left:
+            take = min(portion, left)
+            t.step([("a", take)], want="last" if take == left else "none")
+            left -= take
+        for _ in range(3):
+            t.step([("a", 1)])
+        t.steps[-1]["end"] = ["a"]
+        t.live.clear()
+        out = replay(d, dtype, t)
+        got[portion] = np.concatenate([out[s] for s in sorted(out)])
+    assert got[4096].shape == (4, 1000)
+    scale = np.abs(got[4096]).max(axis=1, keepdims=True)
+    err = np.abs(got[777] - got[4096]) / np.maximum(scale, 1.0)
+    assert err.max() <= TOL_ALONE[dtype]["atol"], f"portions of 777 against 4,096: {err.max(axis=1)}"
