@@ -219,11 +219,20 @@ class LLMEngine:
             pending = ahead.pending
             self.steps_taken_ahead += 1
         else:
-            if decoding:
-                logits = self.graphs.step_arrays(ids, start, tokens)
-            elif self.graphs is not None and bool(wants.all()) and self.graphs.prompt_usable(count):
-                logits = self.graphs.prompt_step_arrays(ids, start, count, tokens)   # a short prompt alone in its step
-            else:
+            logits = None
+            recorded = decoding or (self.graphs is not None and bool(wants.all()) and self.graphs.prompt_usable(count))
+            if recorded:
+                # A recorded step that cannot be had (a new shape that cannot be recorded, no memory
+                # for it) is no reason to lose the step: it runs eagerly, and so do all later ones.
+                try:
+                    if decoding:
+                        logits = self.graphs.step_arrays(ids, start, tokens)
+                    else:   # a short prompt alone in its step
+                        logits = self.graphs.prompt_step_arrays(ids, start, count, tokens)
+                except Exception as err:  # noqa: BLE001
+                    self.graphs.safe, self._look_ahead, decoding = False, False, False
+                    print(f"[lyapunov-amd] recorded steps switched off: {type(err).__name__}: {err}", file=sys.stderr)
+            if logits is None:
                 rows = (np.cumsum(count, dtype=np.int32) - 1)[wants != 0]   # the last token of each request that wants
                 logits = self.core.runner.step_arrays(ids, start, count, tokens, rows)
             wanting = [r for r, w in zip(reqs, wants) if w]

@@ -458,3 +458,32 @@ def test_a_recorded_prompt_step_of_two_requests_equals_the_eager_step(model_fold
     both([StepEntry(2, toks[2][:64], 0, [63])])                              # one request, every token row live
     both([StepEntry(1, toks[1][30:31], 30, [0]), StepEntry(0, toks[0][29:70], 29, [40])])   # a single token beside a portion
     both([StepEntry(3, toks[3][:2], 0, [1]), StepEntry(2, toks[2][64:66], 64, [1])])
+
+
+def test_a_step_that_cannot_be_recorded_runs_eagerly(model_folders, capsys):
+    """Recording a step is an optimisation: when it fails, the planned step runs the eager way, later
+    steps too, and generation gives the tokens it gives without graphs."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.engine import graphs as G
+
+    folder = model_folders["B"]["float32"]
+    prompts = [random_tokens(n, 515, seed=60 + n) for n in (12, 70)]
+    sp = L.SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+    want = [o.output_tokens for o in L.LLM(folder, dtype="float32", num_blocks=24, enable_graphs=False).generate(prompts, sp)]
+
+    llm = L.LLM(folder, dtype="float32", num_blocks=24)
+    calls = []
+
+    def failing(self, fixed):
+        calls.append(fixed)
+        raise RuntimeError("out of memory while recording")
+
+    real = G.StepGraphs._captured
+    G.StepGraphs._captured = failing
+    try:
+        got = [o.output_tokens for o in llm.generate(prompts, sp)]
+    finally:
+        G.StepGraphs._captured = real
+    assert got == want and len(calls) == 1 and llm.engine.graphs.safe is False
+    assert "recorded steps switched off" in capsys.readouterr().err
+    llm.engine.core.cache.check()
