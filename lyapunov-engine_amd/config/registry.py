@@ -3,7 +3,8 @@
 ``ARCHITECTURES`` maps the string in config.json's ``architectures`` list to an
 architecture (a typed configuration class plus a function that turns such a
 configuration into a ``ModelSpec``).  ``MIXERS``, ``FEED_FORWARDS``, ``NORMS``,
-``POSITION_ENCODINGS`` and ``BLOCKS`` map a ``PartSpec.kind`` to a part class.
+``POSITION_ENCODINGS``, ``BLOCKS``, ``EMBEDDINGS`` and ``HEADS`` map a
+``PartSpec.kind`` to a part class.
 Code outside this package (a test, a plug-in) adds an entry with
 ``@REGISTRY.register("name")`` and needs no change to the package's files.
 
@@ -65,6 +66,8 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
 
 
 def register_architecture(name: str, config_class: Any, to_spec: Callable[[Any], Any], *, replace: bool = False):

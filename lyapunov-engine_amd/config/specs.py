@@ -4,10 +4,11 @@ data, of which parts make up each layer and in which order the layers run.
 Nothing in here knows Llama.  An architecture (``models/llama.py`` is the one in
 this package) turns its own typed configuration into a ``ModelSpec``; the
 builder (``models/decoder.py``) looks every part up by its kind in the
-registries and puts the model together.  Because the description is per layer,
-one model may use different mixers and feed-forwards in different layers, and
-because the running order is a list of its own, a layer may run twice or read
-the cache that another call of a layer filled.
+registries (the embedding and the output head too) and puts the model together.
+Because the description is per layer, one model may use different mixers and
+feed-forwards in different layers, and because the running order is a list of
+its own, a layer may run twice or read the cache that another call of a layer
+filled.
 """
 from __future__ import annotations
 
@@ -33,6 +34,11 @@ class LayerSpec:
     # Names of the parts inside the layer's tensor-name prefix.
     names: dict = field(default_factory=lambda: {
         "norm1": "input_layernorm", "mixer": "self_attn", "norm2": "post_attention_layernorm", "ffn": "mlp"})
+    # Further parts for an arrangement that has more than these four (a norm
+    # after each branch, a second feed-forward): name -> PartSpec; the block
+    # kind decides which registry each comes from and what its tensors are
+    # called.  "prenorm" takes none.
+    extra: dict = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -58,11 +64,16 @@ class ModelSpec:
     layers: tuple                    # of LayerSpec
     schedule: tuple                  # of LayerCall
     final_norm: PartSpec
-    tie_word_embeddings: bool
+    tie_word_embeddings: bool       # the output head uses the embedding's matrix (Head.tie)
     max_position: int
-    embed_name: str = "model.embed_tokens.weight"
+    # The parts at the two ends, built with vocab_size= and hidden_size= beside
+    # their own parameters: from token ids to the residual stream's first value,
+    # and from normed rows to float logits.
+    embedding: PartSpec = PartSpec("lookup")
+    head: PartSpec = PartSpec("linear")
+    embed_prefix: str = "model.embed_tokens."
     final_norm_prefix: str = "model.norm."
-    head_name: str = "lm_head.weight"
+    head_prefix: str = "lm_head."
     layer_prefix: str = "model.layers.{i}."
     eos_token_ids: tuple = ()
     ignorable_tensors: tuple = ()    # shell-style patterns of tensor names a file may hold unused

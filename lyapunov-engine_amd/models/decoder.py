@@ -1,5 +1,5 @@
 """A decoder put together from a ModelSpec: embedding, the layers in their
-running order, final norm, output head.
+running order, final norm, output head, each looked up by its kind.
 
 The order of work is the reference's LlamaForCausalLM.forward
 (python/lyapunov_engine/models/llama.py:196-225): embed, layers, final norm,
@@ -17,7 +17,7 @@ from typing import Iterator, Optional
 
 import torch
 
-from ..config.registry import BLOCKS, NORMS
+from ..config.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 from ..config.specs import LayerCall, ModelSpec
 from ..kernels import ops
 from ..parts.base import (KVCacheSpec, LayerCache, Part, PositionEncoding, StateSpec, StepContext, WeightSource,
@@ -45,18 +45,30 @@ class CacheLayout:
 class DecoderModel(Part):
     def __init__(self, spec: ModelSpec):
         self.spec = spec
+        self.embedding = EMBEDDINGS.build(spec.embedding, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
         self.layers = [BLOCKS.get(ls.block)(ls) for ls in spec.layers]
         self.final_norm = NORMS.build(spec.final_norm)
+        self.head = HEADS.build(spec.head, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size)
+        if spec.tie_word_embeddings:
+            self.head.tie(self.embedding)
         self.schedule: tuple = tuple(spec.schedule)
         for call in self.schedule:
             if not 0 <= call.layer < len(self.layers):
                 raise ValueError(f"the running order names layer {call.layer}; there are {len(self.layers)}")
-        self.embed: Optional[torch.Tensor] = None
-        self.lm_head: Optional[torch.Tensor] = None
         self.device: Optional[torch.device] = None
         self.dtype: Optional[torch.dtype] = None
         self.max_positions = spec.max_position      # positions a step may reach; ``materialize`` may lower it
         self._layout = self._plan_cache()
+
+    @property
+    def embed(self) -> Optional[torch.Tensor]:
+        """The embedding's matrix."""
+        return self.embedding.weight
+
+    @property
+    def lm_head(self) -> Optional[torch.Tensor]:
+        """The output head's matrix (the embedding's when they are tied)."""
+        return getattr(self.head, "weight", None)
 
     # -------------------------------------------------------------- structure
     def named_parts(self) -> Iterator[tuple]:
@@ -66,17 +78,15 @@ class DecoderModel(Part):
             for piece, child in part.children().items():
                 yield from walk(prefix + piece, child)
 
+        yield from walk(self.spec.embed_prefix, self.embedding)
         for i, layer in enumerate(self.layers):
             yield from walk(self.spec.layer_prefix.format(i=i), layer)
         yield from walk(self.spec.final_norm_prefix, self.final_norm)
+        yield from walk(self.spec.head_prefix, self.head)
 
     def weight_table(self) -> list:
         """(owner, WeightSpec with full tensor names) for the whole model."""
         out = []
-        V, H = self.spec.vocab_size, self.spec.hidden_size
-        out.append((self, WeightSpec("embed", (WeightSource(self.spec.embed_name, (V, H)),))))
-        if not self.spec.tie_word_embeddings:
-            out.append((self, WeightSpec("lm_head", (WeightSource(self.spec.head_name, (V, H)),))))
         for prefix, part in self.named_parts():
             for ws in part.weight_specs():
                 full = tuple(WeightSource(prefix + s.name, tuple(s.shape)) for s in ws.sources)
@@ -98,7 +108,7 @@ class DecoderModel(Part):
         tied model's separate head, and what the architecture declares
         (``ModelSpec.ignorable_tensors``: shell-style patterns, for buffers that
         exporters write and that are computed here, not loaded)."""
-        if self.spec.tie_word_embeddings and name == self.spec.head_name:
+        if self.spec.tie_word_embeddings and name.startswith(self.spec.head_prefix):
             return True
         return any(fnmatch.fnmatchcase(name, pat) for pat in self.spec.ignorable_tensors)
 
@@ -142,19 +152,18 @@ class DecoderModel(Part):
             for _, part in self.named_parts():
                 if isinstance(part, PositionEncoding):
                     part.limit_positions(self.max_positions)
+        self.embedding.materialize(self.device, dtype)
         for layer in self.layers:
             layer.materialize(self.device, dtype)
         self.final_norm.materialize(self.device, dtype)
-        if self.spec.tie_word_embeddings:
-            self.lm_head = self.embed
+        self.head.materialize(self.device, dtype)
 
     # ---------------------------------------------------------------- compute
     def forward(self, ctx: StepContext, caches: list) -> Optional[torch.Tensor]:
         """Run the step's tokens through every call of the running order;
         returns float logits [R, vocab] for ``ctx.logit_rows`` (None if R == 0).
         ``caches[i]`` is the LayerCache of ``schedule[i]``."""
-        h = torch.empty((ctx.T, self.spec.hidden_size), dtype=torch.float32, device=ctx.device)
-        ops.embedding(ctx.token_ids, self.embed, h)
+        h = self.embedding.forward(ctx, ctx.token_ids)
         delta = None
         for call, cache in zip(self.schedule, caches):
             h, delta = self.layers[call.layer].forward(ctx, h, delta, cache)
@@ -163,7 +172,7 @@ class DecoderModel(Part):
         if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
             delta = delta.run()
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
-        return ops.lm_head(x, self.lm_head)
+        return self.head.forward(ctx, x)
 
 
 def build_model(spec: ModelSpec) -> DecoderModel:

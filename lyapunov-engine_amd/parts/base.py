@@ -231,6 +231,30 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """From token ids to the residual stream's first value.  ``weight`` is the
+    matrix [vocab, hidden] that a tied output head uses as its own."""
+
+    weight: Optional[torch.Tensor] = None
+
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
+        """float [T, hidden] for int32 ``token_ids`` [T]."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    """From the normed rows whose logits are wanted to float logits [R, vocab]."""
+
+    def tie(self, embedding: Embedding) -> None:
+        """The model ties its head to the embedding: use ``embedding.weight``
+        (available from ``materialize`` on) and own no matrix.  A head that
+        cannot raises."""
+        raise NotImplementedError(f"{type(self).__name__} cannot share the embedding's matrix")
+
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class PositionEncoding(Part):
     """Turns positions into whatever the mixer applies.  The rotary kind exposes
     ``table`` (float [max_position, rotary_dim]: cosines then sines)."""

@@ -615,3 +615,166 @@ def test_a_stateful_mixer_with_lists_of_its_own_decodes_through_graphs(tmp_path,
     finally:
         ARCHITECTURES.unregister("ToyScanForCausalLM")
         MIXERS.unregister("toy_scan_on_device")
+
+
+# ----------------------- a fourth toy: other ends (a scaled embedding, capped logits), four norms a layer
+TOY4 = dict(architectures=["ToyEndsForCausalLM"], vocab_size=130, hidden_size=64, intermediate_size=112,
+            num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=16, max_position_embeddings=160,
+            rms_norm_eps=1e-5, rope_theta=10000.0, embed_scale=8.0, logit_cap=2.0)
+
+
+def register_toy4():
+    """An embedding that scales its rows, an output head that caps its logits and has a bias of
+    its own, and an arrangement of a layer with a norm after each branch as well as before it: all
+    defined and registered here; mixer, feed-forward and norms are the package's."""
+    from lyapunov_engine_amd.config import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, LayerSpec, ModelSpec,
+                                            PartSpec, default_schedule, register_architecture)
+    from lyapunov_engine_amd.kernels import ops
+    from lyapunov_engine_amd.parts import Block, Embedding, Head, WeightSource, WeightSpec
+
+    class Sandwich(Block):
+        """h += post1(mixer(norm1(h))); h += post2(ffn(norm2(h))).  The two further norms come
+        from LayerSpec.extra."""
+
+        def __init__(self, spec):
+            self.norm1, self.norm2 = NORMS.build(spec.norm1), NORMS.build(spec.norm2)
+            self.post1, self.post2 = NORMS.build(spec.extra["post_mixer"]), NORMS.build(spec.extra["post_ffn"])
+            self.mixer, self.ffn = MIXERS.build(spec.mixer), FEED_FORWARDS.build(spec.ffn)
+
+        def children(self):
+            return {"input_layernorm.": self.norm1, "self_attn.": self.mixer, "post_mixer_norm.": self.post1,
+                    "post_attention_layernorm.": self.norm2, "mlp.": self.ffn, "post_ffn_norm.": self.post2}
+
+        def branch(self, ctx, norm, part, post, h, delta, *cache):
+            x = norm.forward(ctx, h, ops.as_delta(delta, ctx.dtype))
+            y = ops.as_delta(part.forward(ctx, x, *cache), torch.float32)       # the branch's output, summed up
+            return post.forward(ctx, y)
+
+        def forward(self, ctx, h, delta, cache):
+            a = self.branch(ctx, self.norm1, self.mixer, self.post1, h, delta, cache)
+            return h, self.branch(ctx, self.norm2, self.ffn, self.post2, h, a)
+
+    BLOCKS.register("toy_sandwich", Sandwich, replace=True)
+
+    class ScaledLookup(Embedding):
+        def __init__(self, vocab_size, hidden_size, scale):
+            self.vocab_size, self.hidden_size, self.scale = vocab_size, hidden_size, scale
+            self.weight = None
+
+        def weight_specs(self):
+            return [WeightSpec("weight", (WeightSource("weight", (self.vocab_size, self.hidden_size)),))]
+
+        def forward(self, ctx, token_ids):
+            h = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=ctx.device)
+            return ops.embedding(token_ids, self.weight, h).mul_(self.scale)
+
+    class CappedHead(Head):
+        """cap * tanh((x W^T + b) / cap): the embedding's matrix, a bias of its own."""
+
+        def __init__(self, vocab_size, hidden_size, cap):
+            self.vocab_size, self.hidden_size, self.cap = vocab_size, hidden_size, cap
+            self.bias, self.table = None, None
+
+        def tie(self, embedding):
+            self.table = embedding
+
+        def weight_specs(self):
+            return [WeightSpec("bias", (WeightSource("bias", (self.vocab_size,)),))]
+
+        def forward(self, ctx, x):
+            logits = ops.lm_head(x, self.table.weight) + self.bias.float()
+            return torch.tanh(logits / self.cap) * self.cap
+
+    EMBEDDINGS.register("toy_scaled_lookup", ScaledLookup, replace=True)
+    HEADS.register("toy_capped_head", CappedHead, replace=True)
+
+    def to_spec(cfg: ToyConfig) -> ModelSpec:
+        c = dict(cfg.raw)
+        H = c["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": c["rms_norm_eps"]})
+        pos = PartSpec("rope", {"dim": c["head_dim"], "theta": c["rope_theta"], "max_position": c["max_position_embeddings"],
+                                "scaling": None})
+        attn = PartSpec("paged_attention", dict(hidden_size=H, num_heads=c["num_attention_heads"],
+                                                num_kv_heads=c["num_key_value_heads"], head_dim=c["head_dim"], position=pos))
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
+        n = c["num_hidden_layers"]
+        layer = LayerSpec("toy_sandwich", attn, ffn, norm, norm, extra={"post_mixer": norm, "post_ffn": norm})
+        return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=tuple(layer for _ in range(n)),
+                         schedule=default_schedule(n), final_norm=norm, tie_word_embeddings=True,
+                         max_position=c["max_position_embeddings"],
+                         embedding=PartSpec("toy_scaled_lookup", {"scale": c["embed_scale"]}),
+                         head=PartSpec("toy_capped_head", {"cap": c["logit_cap"]}))
+
+    register_architecture("ToyEndsForCausalLM", ToyConfig, to_spec, replace=True)
+
+
+def toy4_plain(folder, tokens):
+    from safetensors.torch import load_file
+
+    c = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    positions = torch.arange(len(tokens))
+    inv_freq = P.model_inv_freq(c)
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)] * c["embed_scale"]
+    eps = c["rms_norm_eps"]
+    for i in range(c["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        a = P.attention_layer(P.rms_norm(h, w[p + "input_layernorm.weight"], eps), positions, w, p + "self_attn.", c, inv_freq)
+        h = h + P.rms_norm(a, w[p + "post_mixer_norm.weight"], eps)
+        m = P.mlp(P.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps), w[p + "mlp.gate_proj.weight"],
+                  w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        h = h + P.rms_norm(m, w[p + "post_ffn_norm.weight"], eps)
+    logits = P.rms_norm(h, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T + w["lm_head.bias"]
+    return torch.tanh(logits / c["logit_cap"]) * c["logit_cap"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_another_embedding_and_another_output_head(tmp_path, dtype):
+    """The model's two ends are parts like the others: an architecture names an embedding and a
+    head of its own, with their own tensors and constants, and an arrangement of a layer with more
+    parts than the usual four, and nothing in the package changes.  Whole prompts, portions
+    beside decoded tokens, and recorded decode steps through the engine."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.config import ARCHITECTURES, BLOCKS, EMBEDDINGS, HEADS
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import compare
+
+    register_toy4()
+    try:
+        folder = str(tmp_path / "toy4")
+        write_random_model(dict(TOY4), folder, seed=9, dtype=dtype, init_std=0.08, norm_init_std=0.1)
+        from safetensors.torch import load_file
+        names = set(load_file(os.path.join(folder, "model.safetensors")))
+        assert "lm_head.bias" in names and "lm_head.weight" not in names and "model.layers.1.post_ffn_norm.weight" in names
+        reqs = {"x": random_tokens(60, 130, seed=15), "y": random_tokens(23, 130, seed=16)}
+        want = {k: toy4_plain(folder, v) for k, v in reqs.items()}
+        assert float(want["x"].abs().max()) > 0.8 * TOY4["logit_cap"]        # the cap is felt
+        whole = Trace(reqs)
+        for rid in reqs:
+            whole.step([(rid, len(reqs[rid]))], end=[rid])
+        compare(whole, replay(folder, dtype, whole), want, dtype, "ends whole")
+        cut = Trace(reqs)
+        cut.step([("x", 13), ("y", 4)])
+        cut.step([("x", 2), ("y", 19)], end=["y"])
+        for _ in range(10):
+            cut.step([("x", 1)])
+        cut.step([("x", 35)], end=["x"])
+        compare(cut, replay(folder, dtype, cut), want, dtype, "ends cut")
+        # through the engine, decode steps recorded: greedy tokens against the plain model's
+        llm = L.LLM(folder, dtype=dtype, num_blocks=32, block_size=16, enable_graphs=True, warmup=False)
+        assert llm.engine.graphs is not None and llm.engine.graphs.safe
+        prompt = reqs["y"]
+        got = llm.generate([prompt], L.SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))[0].output_tokens
+        toks = list(prompt)
+        for i in range(6):
+            logits = toy4_plain(folder, toks)[-1]
+            top = torch.topk(logits, 2).values
+            if got[i] != int(logits.argmax()):
+                assert dtype == "bfloat16" and float(top[0] - top[1]) < 0.25, (i, got)
+                break
+            toks.append(got[i])
+    finally:
+        ARCHITECTURES.unregister("ToyEndsForCausalLM")
+        EMBEDDINGS.unregister("toy_scaled_lookup")
+        HEADS.unregister("toy_capped_head")
+        BLOCKS.unregister("toy_sandwich")
