@@ -34,6 +34,7 @@ class EngineConfig:
     num_blocks: int = 1024
     num_gpu_blocks: Optional[int] = None
     block_size: int = 16
+    cache_groups: Optional[tuple] = None    # per cache group of the model (pages, page size) where they differ; see EngineCore
     max_num_seqs: int = 64
     max_num_batched_tokens: int = 2048
     dtype: object = "bfloat16"

@@ -15,12 +15,23 @@ from .runner import ModelRunner, StepEntry
 
 class EngineCore:
     def __init__(self, model: DecoderModel, model_config, *, dtype, device="cuda:0", num_blocks: int,
-                 block_size: int = 16, num_state_slots: int = 64):
+                 block_size: int = 16, num_state_slots: int = 64, cache_groups: Optional[list] = None):
+        """``cache_groups``: (pages, page size) for each of the model's cache
+        groups in turn (``model.cache_layout().groups``: layers whose keys and
+        values have one shape and one window share a group), where they are to
+        differ from ``num_blocks`` and ``block_size``; None in place of a pair
+        keeps those.  A group of windowed layers needs far fewer pages than one
+        that keeps every key."""
         self.model, self.model_config = model, model_config
         self.dtype, self.device = parse_dtype(dtype), torch.device(device)
         self.block_size = block_size
         layout = model.cache_layout()
-        groups = [GroupConfig(num_blocks, block_size, gl.spec.window) for gl in layout.groups]
+        sizes = list(cache_groups or [])
+        if len(sizes) > len(layout.groups):
+            raise ValueError(f"cache_groups names {len(sizes)} groups, the model has {len(layout.groups)}")
+        sizes += [None] * (len(layout.groups) - len(sizes))
+        sizes = [(num_blocks, block_size) if s is None else (int(s[0]), int(s[1])) for s in sizes]
+        groups = [GroupConfig(pages, size, gl.spec.window) for (pages, size), gl in zip(sizes, layout.groups)]
         # A model without keys and values (state only) still gets a group, so
         # that requests have a length and the manager one code path.
         self.cache = CacheManager(groups or [GroupConfig(num_blocks, block_size, 0)], num_state_slots)
@@ -34,6 +45,9 @@ class EngineCore:
         (``num_blocks * block_size``) it bounds the positions the model is set
         up for (the rows of its position tables)."""
         reach = kw["num_blocks"] * kw.get("block_size", 16)
+        for pair in kw.get("cache_groups") or []:   # which group bounds a request is known once the model is built
+            if pair is not None:
+                reach = max(reach, int(pair[0]) * int(pair[1]))
         if max_model_len:
             reach = min(reach, int(max_model_len))
         model, cfg = load_model(model_dir, parse_dtype(dtype), device, source=source, max_positions=reach)

@@ -88,7 +88,7 @@ class LLMEngine:
         else:
             self.core = EngineCore.from_folder(str(model), dtype=config.dtype, device=config.device,
                                                num_blocks=config.num_blocks, block_size=config.block_size,
-                                               num_state_slots=config.max_num_seqs,
+                                               cache_groups=config.cache_groups, num_state_slots=config.max_num_seqs,
                                                max_model_len=config.max_model_len)
         spec = self.core.model.spec
         # (the model's position tables may have fewer rows than spec.max_position: as many as the
@@ -129,7 +129,7 @@ class LLMEngine:
         from ..kernels import ops
 
         cache, cfg = self.core.cache, self.config
-        pages = min(cache.num_free_pages(g) for g in range(len(cache.groups)))
+        room = min(cache.num_free_pages(g) * gc.page_size for g, gc in enumerate(cache.groups))  # tokens a step may bring
         sizes = {cfg.max_num_batched_tokens}
         if cfg.max_chunk:
             sizes.add(min(cfg.max_chunk, cfg.max_num_batched_tokens))
@@ -138,7 +138,7 @@ class LLMEngine:
             while n < cfg.max_num_batched_tokens:
                 sizes.add(n)
                 n *= 2
-        for n in sorted({min(s, self.max_model_len, pages * self.core.block_size) for s in sizes}):
+        for n in sorted({min(s, self.max_model_len, room) for s in sizes}):
             if n < 1 or cache.has(self.WARMUP_ID) or cache.num_free_slots() < 1:
                 continue
             cache.add(self.WARMUP_ID)

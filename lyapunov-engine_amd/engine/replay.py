@@ -18,10 +18,12 @@ MAX_LIVE_REQUESTS = 8
 
 
 class TraceReplayer:
-    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0"):
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0",
+                 cache_groups=None):
         num_blocks = max(1, -(-max_tokens // block_size))
         self.core = EngineCore.from_folder(model_dir, dtype=dtype, device=device, num_blocks=num_blocks,
-                                           block_size=block_size, num_state_slots=MAX_LIVE_REQUESTS)
+                                           block_size=block_size, num_state_slots=MAX_LIVE_REQUESTS,
+                                           cache_groups=cache_groups)
         self._ids: dict = {}
         self._next_id = 0
 

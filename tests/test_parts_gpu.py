@@ -286,6 +286,12 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
             cut.step([("x", 1), ("z", 1)])
         cut.step([("x", 42), ("z", 2)], end=["x", "z"])
         compare(cut, replay(folder, dtype, cut), want, dtype, "toy cut")
+        # the windowed layers' group with a pool of its own size and smaller pages: a window of 6 keys needs
+        # few pages per request beside those of the portion a step brings (here up to 42 tokens)
+        got = replay(folder, dtype, cut, cache_groups=[None, (24, 4)])
+        compare(cut, got, want, dtype, "toy cut, pools of two sizes")
+        with pytest.raises(ValueError, match="cache_groups names 3 groups"):
+            replay(folder, dtype, cut, cache_groups=[None, None, (8, 8)])
 
         # through the generating engine: greedy tokens are the plain model's; with a state that a step
         # changes in place no step is started ahead (one that had to be dropped could not be run again)

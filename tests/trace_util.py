@@ -121,11 +121,11 @@ def plain_logits_at(folder: str, tokens: list, rows: list, chunk: int = 256) -> 
     return {int(r): logits[j] for j, r in enumerate(keep.tolist())}
 
 
-def replay(folder: str, dtype: str, trace: Trace, max_tokens=None) -> dict:
+def replay(folder: str, dtype: str, trace: Trace, max_tokens=None, **core_options) -> dict:
     """Run the trace through the engine in this process: step -> [rows, vocab]."""
     from lyapunov_engine_amd.engine.replay import TraceReplayer
 
-    rp = TraceReplayer(folder, dtype, max_tokens or trace.max_tokens)
+    rp = TraceReplayer(folder, dtype, max_tokens or trace.max_tokens, **core_options)
     out = {}
     for s in trace.steps:
         logits = rp.run(s)
