@@ -247,8 +247,12 @@ def main():
     esz = 2 if args.dtype == "bf16" else 4
     block_size = 16
     max_batch = 64
-    num_blocks = max_batch * (args.context // block_size + 1) + 64
+    # the pool holds the largest batch that runs: 64 for the points beside the headline
+    pool_batch = max(args.batch, 1) if args.skip_points and args.workload == "decode" else max_batch
+    num_blocks = pool_batch * (args.context // block_size + 1) + 64
     shape = SHAPES[args.shape]
+    if args.context > shape["max_position_embeddings"]:     # a longer context than the baseline's: the models allow it
+        shape = dict(shape, max_position_embeddings=args.context)
     full_layers = shape["num_hidden_layers"]
     engine, cfg = build_engine(args.layers or full_layers, args.dtype, num_blocks, max_batch, block_size, budget=8192,
                                shape=shape)
