@@ -1249,10 +1249,14 @@ int lyp_attn_decode_plan(int n_seqs, int max_ctx, int nh, int nkv) {
   const int B = pow2(n_seqs, 1), C = pow2(max_ctx, 256);
   const int g = nh / (nkv > 0 ? nkv : 1);
   const long long base = static_cast<long long>(B) * nkv * ((g + 15) / 16);
+  // Partitions grow while the launch keeps this many workgroups: one or two requests do best with one
+  // workgroup per compute unit (batch 1 at 32,768 keys: 21.2 us a layer with 256 workgroups of
+  // 1,024 keys, 23.7 with 512 of 512), more requests with two.
+  const int enough = base < 32 ? 256 : 512;
   int kpw = kPartKeys;
   while (kpw < 1024) {
     const int next_block = kDecodeWaves * kpw * 2;
-    if (base * ((C + next_block - 1) / next_block) < 512) break;
+    if (base * ((C + next_block - 1) / next_block) < enough) break;
     kpw *= 2;
   }
   // Two partitions per request are not worth the combine pass they need: one workgroup takes the
