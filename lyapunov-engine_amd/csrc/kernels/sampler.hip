@@ -312,6 +312,9 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     for (int i = tid; i < V; i += kSampleThreads) am = better(am, ArgMax{x[i], i});
   }
   am = block_argmax(am, s_arg);
+  // A row without a single logit that compares (all NaN, or all -inf) has no largest one: token 0
+  // stands for it, so that what is written is a token in any case (the next step looks it up).
+  if (am.i < 0 || am.i >= V) am = ArgMax{LYP_NEG_INF, 0};
   const float T = temperature[row];
   if (T < 1e-4f) {
     if (tid == 0) {

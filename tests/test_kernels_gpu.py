@@ -856,6 +856,41 @@ def test_sampler_greedy_and_draws(ops):
             assert lo - 1e-5 <= u_val <= float(cdf[got[r]]) + 1e-5, f"row {r}: u={u_val} not in [{lo}, {float(cdf[got[r]])}]"
 
 
+def test_sampler_writes_a_token_for_rows_without_a_largest_logit(ops):
+    """Rows of NaN or of -inf only (broken weights, an overflow) have no largest logit; what the
+    sampler writes is still a token of the vocabulary, which the next step can look up, and rows
+    beside them are not disturbed.  With and without the pass that finds the maxima first, and with
+    the output head's candidates."""
+    V, K = 2051, 64
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(6, V, generator=g)
+    logits[1] = float("nan")
+    logits[2] = float("-inf")
+    logits[4] = float("nan")
+    logits[4, 77] = 1.5                                  # one logit that compares: it is the row's choice
+    temperature = torch.tensor([0.0, 0.0, 0.9, 0.8, 0.0, 1.1])
+    top_k = torch.tensor([-1, -1, 10, -1, -1, 20], dtype=torch.int32)
+    top_p = torch.tensor([1.0, 1.0, 0.9, 1.0, 1.0, 0.7])
+    u = torch.full((6,), 0.42)
+    for work in (None, ops.sample_workspace(6, DEV)):
+        out = torch.full((6,), -1, dtype=torch.int32, device=DEV)
+        ops.sample(logits.to(DEV), temperature.to(DEV), top_k.to(DEV), top_p.to(DEV), u.to(DEV), out, work)
+        got = out.cpu().tolist()
+        assert all(0 <= t < V for t in got), got
+        assert got[0] == P.greedy(logits[0]) and got[1] == 0 and got[2] == 0 and got[4] == 77
+    # through the head's kernel: activations of NaN give rows of NaN logits and candidates without a place
+    x = rnd(3, K, dtype=torch.bfloat16, seed=7)
+    x[1] = float("nan")
+    w = rnd(V, K, dtype=torch.bfloat16, scale=0.2, seed=8)
+    head = ops.lm_head(x.to(DEV), w.to(DEV))
+    assert getattr(head, "argmax_candidates", None) is not None
+    out = torch.full((3,), -1, dtype=torch.int32, device=DEV)
+    z = torch.zeros(3, device=DEV)
+    ops.sample(head, z, torch.full((3,), -1, dtype=torch.int32, device=DEV), torch.ones(3, device=DEV), z, out)
+    got = out.cpu().tolist()
+    assert got[1] == 0 and got[0] == int(head[0].argmax()) and got[2] == int(head[2].argmax())
+
+
 def _row(kind, V, g):
     if kind == "peaked":       # as a trained model's: a few tokens stand out
         x = torch.randn(V, generator=g) * 2.5
