@@ -1251,8 +1251,10 @@ int lyp_attn_decode_plan(int n_seqs, int max_ctx, int nh, int nkv) {
   const long long base = static_cast<long long>(B) * nkv * ((g + 15) / 16);
   // Partitions grow while the launch keeps this many workgroups: one or two requests do best with one
   // workgroup per compute unit (batch 1 at 32,768 keys: 21.2 us a layer with 256 workgroups of
-  // 1,024 keys, 23.7 with 512 of 512), more requests with two.
-  const int enough = base < 32 ? 256 : 512;
+  // 1,024 keys, 23.7 with 512 of 512), more requests with two; with heads of more than 64 values
+  // (a key is twice the bytes) one per compute unit at every batch (heads of 128, batch 8 at
+  // 8,192 keys: 53.2 us with partitions of 2,048 keys, 56.7 with 1,024).
+  const int enough = (base < 32 || HD > 64) ? 256 : 512;
   int kpw = kPartKeys;
   while (kpw < 1024) {
     const int next_block = kDecodeWaves * kpw * 2;
