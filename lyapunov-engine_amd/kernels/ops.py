@@ -493,6 +493,11 @@ LIBRARY_GEMM_MIN_ROWS = 65
 # matrix is large; measured, the library is ahead from this many weights on.
 LIBRARY_GEMM_MID_ROWS = 17
 LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
+# From 49 rows on (a step of 64 in its recorded form) also for the smaller matrices, q/k/v and o of
+# the 1B shape among them: batch 64 at 2,048 tokens 30,200 -> 30,800 tokens/s (2 %); at 48 rows the
+# weight-streaming kernel is still ahead (25,400 against 25,200).
+LIBRARY_GEMM_WIDE_ROWS = 49
+LIBRARY_GEMM_WIDE_WEIGHTS = 1 << 22
 # In an engine's warm-up step and in the run before a graph is captured, a library product's algorithm is
 # chosen by measurement among this many of the library's candidates (at the shape's first call).
 # Which candidate wins a timing may differ from process to process, and with it the last bits of
@@ -581,7 +586,8 @@ def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torc
 def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     if not LIBRARY_GEMM or dtype != torch.bfloat16:
         return False
-    return M >= LIBRARY_GEMM_MIN_ROWS or (M >= LIBRARY_GEMM_MID_ROWS and N * K >= LIBRARY_GEMM_MID_WEIGHTS)
+    return (M >= LIBRARY_GEMM_MIN_ROWS or (M >= LIBRARY_GEMM_MID_ROWS and N * K >= LIBRARY_GEMM_MID_WEIGHTS)
+            or (M >= LIBRARY_GEMM_WIDE_ROWS and N * K >= LIBRARY_GEMM_WIDE_WEIGHTS))
 
 
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
