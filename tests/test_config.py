@@ -188,3 +188,68 @@ def test_layers_with_equal_position_parameters_share_one_table():
     other = build_model(llama_spec(LlamaConfig.from_dict(dict(raw, rope_theta=10000.0, max_position_embeddings=4096))))
     other.materialize("cpu", torch.float32)
     assert other.layers[0].mixer.position.table.data_ptr() != small.layers[0].mixer.position.table.data_ptr()
+
+
+def test_embedding_and_head_are_parts_an_architecture_may_replace():
+    """The model's two ends come from registries like every other part: the built-in kinds bind the
+    usual two tensors (one when tied, and then the head uses the embedding's matrix itself); kinds
+    registered from outside bring their own tensors and constants, a head that cannot share the
+    embedding's matrix says so, and an unknown kind names the known ones."""
+    import dataclasses
+
+    import torch
+
+    from lyapunov_engine_amd.config import EMBEDDINGS, HEADS, PartSpec
+    from lyapunov_engine_amd.parts import Embedding, Head, WeightSource, WeightSpec
+
+    tied = build_model(llama_spec(LlamaConfig.from_dict(TINY_A)))
+    assert type(tied.embedding).__name__ == "TokenEmbedding" and type(tied.head).__name__ == "LinearHead"
+    assert "lm_head.weight" not in tied.expected_tensors() and tied.ignorable("lm_head.weight")
+    tied.embedding.weight = torch.zeros(3, 2)
+    tied.materialize("cpu", torch.float32)
+    assert tied.lm_head is tied.embed and tied.head.weight is tied.embedding.weight     # one matrix, two uses
+    untied = build_model(llama_spec(LlamaConfig.from_dict(TINY_B)))
+    assert "lm_head.weight" in untied.expected_tensors() and not untied.ignorable("lm_head.weight")
+
+    class Scaled(Embedding):
+        def __init__(self, vocab_size, hidden_size, scale):
+            self.sizes, self.scale, self.weight = (vocab_size, hidden_size), scale, None
+
+        def weight_specs(self):
+            return [WeightSpec("weight", (WeightSource("weight", self.sizes),)),
+                    WeightSpec("offset", (WeightSource("offset", (self.sizes[1],)),))]
+
+    class Biased(Head):
+        def __init__(self, vocab_size, hidden_size):
+            self.vocab_size, self.shared = vocab_size, None
+
+        def tie(self, embedding):
+            self.shared = embedding
+
+        def weight_specs(self):
+            return [WeightSpec("bias", (WeightSource("bias", (self.vocab_size,)),))]
+
+    class Alone(Head):          # keeps the default tie(): it cannot share
+        def __init__(self, vocab_size, hidden_size):
+            pass
+
+    EMBEDDINGS.register("test_scaled", Scaled)
+    HEADS.register("test_biased", Biased)
+    HEADS.register("test_alone", Alone)
+    try:
+        spec = dataclasses.replace(llama_spec(LlamaConfig.from_dict(TINY_A)), embedding=PartSpec("test_scaled", {"scale": 3.0}),
+                                   head=PartSpec("test_biased"), embed_prefix="tok.", head_prefix="out.")
+        model = build_model(spec)
+        names = model.expected_tensors()
+        assert names["tok.weight"][0] == (TINY_A["vocab_size"], TINY_A["hidden_size"]) and names["tok.offset"][0] == (TINY_A["hidden_size"],)
+        assert names["out.bias"][0] == (TINY_A["vocab_size"],) and "lm_head.weight" not in names and "model.embed_tokens.weight" not in names
+        assert model.embedding.scale == 3.0 and model.head.shared is model.embedding
+        assert model.ignorable("out.weight") and not model.ignorable("lm_head.weight")   # tied: the head's prefix
+        with pytest.raises(NotImplementedError, match="cannot share"):
+            build_model(dataclasses.replace(spec, head=PartSpec("test_alone")))
+        with pytest.raises(KeyError, match="unknown output head 'nope'.*linear"):
+            build_model(dataclasses.replace(spec, head=PartSpec("nope")))
+    finally:
+        EMBEDDINGS.unregister("test_scaled")
+        HEADS.unregister("test_biased")
+        HEADS.unregister("test_alone")
