@@ -878,6 +878,14 @@ def test_sampler_writes_a_token_for_rows_without_a_largest_logit(ops):
         got = out.cpu().tolist()
         assert all(0 <= t < V for t in got), got
         assert got[0] == P.greedy(logits[0]) and got[1] == 0 and got[2] == 0 and got[4] == 77
+        # the same rows drawn from, with and without cut-offs: still a token, and the one logit that compares
+        for tk, tp in ((-1, 1.0), (5, 1.0), (-1, 0.5), (7, 0.3)):
+            hot = torch.full((6,), 0.8)
+            ops.sample(logits.to(DEV), hot.to(DEV), torch.full((6,), tk, dtype=torch.int32, device=DEV),
+                       torch.full((6,), tp, device=DEV), u.to(DEV), out, work)
+            got = out.cpu().tolist()
+            assert all(0 <= t < V for t in got), (tk, tp, got)
+            assert got[4] == 77, (tk, tp, got)
     # through the head's kernel: activations of NaN give rows of NaN logits and candidates without a place
     x = rnd(3, K, dtype=torch.bfloat16, seed=7)
     x[1] = float("nan")
