@@ -210,7 +210,7 @@ def check_logits(shape=MODEL, layers=2, context=8192, portion=2048):
         core.cache.extend(0, context)
         graphs = DecodeGraphs(core.runner, max_batch=1)
         out = graphs.step_arrays(np.zeros(1, np.int64), np.asarray([context - 1], np.int32),
-                                 np.asarray(prompt[-1:], np.int32))
+                                 np.asarray(prompt[-1:], np.int32)).values
         rows.append(out.float().cpu()[0])
         assert list(graphs.captured) == [(1, context)]
         core.cache.commit(0, context)

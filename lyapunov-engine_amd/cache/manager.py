@@ -4,11 +4,12 @@ numbers for.
 ``CacheManager`` wraps the C++ class of csrc/runtime/cache_manager.hpp (pages in
 groups, block tables, windows, state slots; after the reference's
 BlockSpaceManager, csrc/engine/block_manager.cpp:7-101).  ``CachePools`` holds
-the tensors: per group one key pool and one value pool for every cache buffer of
-the group, and per stateful buffer one tensor of slots.  The reference allocates
-two zero tensors [num_blocks, nkv, block_size, head_dim] per layer
-(python/lyapunov_engine/engine/llm_engine.py:143-158); the value pool here is
-[num_blocks, nkv, head_dim, block_size], the layout the attention kernels read.
+the tensors: per group, for every cache buffer of the group, the tensors its
+mixers' ``PagedSpec`` names, and per stateful buffer one tensor of slots.  The
+reference allocates two zero tensors [num_blocks, nkv, block_size, head_dim] per
+layer (python/lyapunov_engine/engine/llm_engine.py:143-158); the layout here is
+the mixer's choice (attention: keys as there, values
+[num_blocks, nkv, head_dim, block_size], which its kernels read).
 """
 from __future__ import annotations
 
@@ -151,23 +152,24 @@ class CacheManager:
 class CachePools:
     """Device memory behind the page and slot numbers.
 
-    ``kv[g]`` is (keys, values) of group g with a leading dimension over the
-    group's cache buffers; ``index[cache_id]`` says where a buffer lives;
-    ``state[cache_id]`` is the slot tensor of a stateful buffer (its last slot
-    belongs to no request: rows that are only padding use it).  Everything
-    starts at zero: a page that was never written must not hold a NaN pattern.
+    ``paged[g]`` maps the names of group g's page tensors (its ``PagedSpec``:
+    what the group's mixers keep per token, in the layout they chose) to
+    tensors [buffers, pages, *page shape]; ``index[cache_id]`` says where a
+    buffer lives; ``state[cache_id]`` is the slot tensor of a stateful buffer
+    (its last slot belongs to no request: rows that are only padding use it).
+    Everything starts at zero: a page that was never written must not hold a
+    NaN pattern.
     """
 
     def __init__(self, layout, group_configs: list, num_state_slots: int, dtype: torch.dtype, device):
         if len(group_configs) != len(layout.groups):
             raise CacheError(f"{len(layout.groups)} cache groups need as many pool configurations")
-        self.kv = []
+        self.paged = []
         self.index = {}
         for g, (gl, gc) in enumerate(zip(layout.groups, group_configs)):
-            nb, s = len(gl.buffers), gl.spec
-            k = torch.zeros((nb, gc.num_pages, s.num_kv_heads, gc.page_size, s.head_dim), dtype=dtype, device=device)
-            v = torch.zeros((nb, gc.num_pages, s.num_kv_heads, s.head_dim, gc.page_size), dtype=dtype, device=device)
-            self.kv.append((k, v))
+            nb = len(gl.buffers)
+            self.paged.append({t.name: torch.zeros((nb, gc.num_pages) + t.page_shape(gc.page_size),
+                                                   dtype=t.dtype or dtype, device=device) for t in gl.spec.tensors})
             for i, cache_id in enumerate(gl.buffers):
                 self.index[cache_id] = (g, i)
         # one slot more than requests can hold: the padded rows of a recorded step are pointed at it
@@ -175,10 +177,10 @@ class CachePools:
                       for cid, st in layout.states.items()}
 
     def buffer(self, cache_id: int):
+        """-> (group, {page tensor name: [pages, *page shape]}) of one cache buffer."""
         g, i = self.index[cache_id]
-        k, v = self.kv[g]
-        return g, k[i], v[i]
+        return g, {name: t[i] for name, t in self.paged[g].items()}
 
     def bytes(self) -> int:
-        total = sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in self.kv)
+        total = sum(t.numel() * t.element_size() for group in self.paged for t in group.values())
         return total + sum(s.numel() * s.element_size() for s in self.state.values())

@@ -3,7 +3,7 @@ declares its C interface for ctypes."""
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_void_p
 
 from ..kernels import build
 
@@ -48,7 +48,7 @@ def lib() -> ctypes.CDLL:
     L.lyp_sched_create.restype = c_void_p
     L.lyp_sched_create.argtypes = [c_void_p, c_int, c_int, c_int, c_int, i32p, c_int]
     L.lyp_sched_destroy.argtypes = [c_void_p]
-    L.lyp_sched_add.argtypes = [c_void_p, c_int64, i32p, c_int, c_float, c_float, c_int, c_int, c_int, c_uint64]
+    L.lyp_sched_add.argtypes = [c_void_p, c_int64, i32p, c_int, c_int, c_int]
     L.lyp_sched_abort.argtypes = [c_void_p, c_int64]
     for name in ("has_unfinished", "num_waiting", "num_running"):
         getattr(L, f"lyp_sched_{name}").argtypes = [c_void_p]
@@ -59,7 +59,6 @@ def lib() -> ctypes.CDLL:
     L.lyp_sched_last_preempted.argtypes = [c_void_p, i64p, c_int]
     L.lyp_sched_info.argtypes = [c_void_p, c_int64, i32p]
     L.lyp_sched_tokens.argtypes = [c_void_p, c_int64, c_int, i32p, c_int]
-    L.lyp_sched_params.argtypes = [c_void_p, c_int64, POINTER(c_float), i32p, POINTER(c_uint64)]
     L.lyp_sched_forget.argtypes = [c_void_p, c_int64]
     L.lyp_sched_counters.argtypes = [c_void_p, i64p]
     L.lyp_sched_counters.restype = None

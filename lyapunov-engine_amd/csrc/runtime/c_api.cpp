@@ -219,17 +219,12 @@ void* lyp_sched_create(void* cache, int max_num_seqs, int max_num_batched_tokens
 }
 void lyp_sched_destroy(void* h) { delete static_cast<Scheduler*>(h); }
 
-int lyp_sched_add(void* h, int64_t id, const int32_t* prompt, int n, float temperature, float top_p, int top_k,
-                  int max_tokens, int ignore_eos, uint64_t seed) {
+int lyp_sched_add(void* h, int64_t id, const int32_t* prompt, int n, int max_tokens, int ignore_eos) {
   return guarded([&] {
-    lyp::SamplingParams sp;
-    sp.temperature = temperature;
-    sp.top_p = top_p;
-    sp.top_k = top_k;
-    sp.max_tokens = max_tokens;
-    sp.ignore_eos = ignore_eos != 0;
-    sp.seed = seed;
-    static_cast<Scheduler*>(h)->add(id, std::vector<int32_t>(prompt, prompt + n), sp);
+    lyp::StopRule rule;
+    rule.max_tokens = max_tokens;
+    rule.ignore_eos = ignore_eos != 0;
+    static_cast<Scheduler*>(h)->add(id, std::vector<int32_t>(prompt, prompt + n), rule);
     return 0;
   });
 }
@@ -313,19 +308,6 @@ int lyp_sched_tokens(void* h, int64_t id, int from, int32_t* out, int cap) {
     const int n = std::max(0, std::min(cap, s.total_len() - from));
     if (n > 0) std::memcpy(out, s.tokens.data() + from, sizeof(int32_t) * static_cast<size_t>(n));
     return n;
-  });
-}
-// out = {temperature, top_p} / {top_k, max_tokens, ignore_eos}; seed separately.
-int lyp_sched_params(void* h, int64_t id, float* fout, int32_t* iout, uint64_t* seed) {
-  return guarded([&] {
-    const auto& p = static_cast<Scheduler*>(h)->get(id).params;
-    fout[0] = p.temperature;
-    fout[1] = p.top_p;
-    iout[0] = p.top_k;
-    iout[1] = p.max_tokens;
-    iout[2] = p.ignore_eos ? 1 : 0;
-    *seed = p.seed;
-    return 0;
   });
 }
 int lyp_sched_forget(void* h, int64_t id) {

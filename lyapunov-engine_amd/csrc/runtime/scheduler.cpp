@@ -11,7 +11,7 @@ Scheduler::Scheduler(SchedulerConfig config, CacheManager* cache) : config_(std:
     throw std::invalid_argument("scheduler limits must be positive");
 }
 
-void Scheduler::add(int64_t id, const std::vector<int32_t>& prompt, const SamplingParams& params) {
+void Scheduler::add(int64_t id, const std::vector<int32_t>& prompt, const StopRule& params) {
   if (seqs_.count(id)) throw std::runtime_error("request id " + std::to_string(id) + " is in use");
   if (prompt.empty()) throw std::runtime_error("empty prompt");
   const int prompt_len = static_cast<int>(prompt.size());

@@ -29,14 +29,12 @@
 
 namespace lyp {
 
-// python/lyapunov_engine/engine/sampling.py:6-12 and sequence.hpp:20-26, plus a seed.
-struct SamplingParams {
-  float temperature = 1.0f;
-  float top_p = 1.0f;
-  int top_k = -1;
+// The part of a request's sampling parameters (python/lyapunov_engine/engine/sampling.py:6-12,
+// sequence.hpp:20-26) that decides when the request ends.  How a token is chosen (temperature,
+// top-k, top-p, seed) is the sampler's business and never comes here.
+struct StopRule {
   int max_tokens = 128;
   bool ignore_eos = false;
-  uint64_t seed = 0;
 };
 
 enum class Status : int {
@@ -52,7 +50,7 @@ struct Sequence {
   std::vector<int32_t> tokens;  // prompt, then what was generated
   int prompt_len = 0;
   int num_computed = 0;  // tokens whose keys are in the cache
-  SamplingParams params;
+  StopRule params;
   Status status = Status::Waiting;
   int preemptions = 0;
 
@@ -82,7 +80,7 @@ class Scheduler {
 
   // Throws if the id is in use, the prompt is empty, it reaches the model's
   // length, or prompt + max_tokens could not fit in the page pools even alone.
-  void add(int64_t id, const std::vector<int32_t>& prompt, const SamplingParams& params);
+  void add(int64_t id, const std::vector<int32_t>& prompt, const StopRule& params);
   bool abort(int64_t id);
   bool has_unfinished() const { return !waiting_.empty() || !running_.empty(); }
   int num_waiting() const { return static_cast<int>(waiting_.size()); }

@@ -51,7 +51,7 @@ static int one_round(std::mt19937& rng) {
     if (pick(0, 3) == 0) {
       std::vector<int32_t> prompt(pick(1, cfg.max_model_len + 2));
       for (auto& t : prompt) t = pick(8, 99);
-      SamplingParams sp;
+      StopRule sp;
       sp.max_tokens = pick(1, 24);
       sp.ignore_eos = pick(0, 1) != 0;
       try {

@@ -27,7 +27,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from ..parts.base import FixedStep
+from ..parts.base import FixedStep, Logits
 from .runner import ModelRunner, StepError
 
 
@@ -80,7 +80,7 @@ class _Captured:
             with torch.cuda.graph(self.graph, pool=pool):
                 self.logits = runner.model.forward(self.ctx, caches)
 
-    def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None, counts=None) -> torch.Tensor:
+    def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None, counts=None) -> Logits:
         """``tokens_dev``: the token ids as an int32 tensor on the device, for a
         step whose tokens the host does not know yet (``tokens`` is ignored).
         ``counts``: new tokens per request, for a recorded step with prompt tokens."""
@@ -93,11 +93,7 @@ class _Captured:
         # one small kernel reads the pinned table (and the device's token ids) into place
         ops.table_load(host, self.dev, None if tokens_dev is None else tokens_dev[:len(ids)], self.token_words)
         self.graph.replay()
-        out = self.logits[:len(ids)]
-        cand = getattr(self.logits, "argmax_candidates", None)
-        if cand is not None:     # what the head's kernel left for the sampler travels with the rows
-            out.argmax_candidates = cand
-        return out
+        return self.logits.first(len(ids))
 
 
 class StepGraphs:
@@ -136,12 +132,12 @@ class StepGraphs:
         """Logits [len(entries), vocab]; valid until the next graph step."""
         return self.step_arrays(np.asarray([e.seq_id for e in entries], dtype=np.int64),
                                 np.asarray([e.start for e in entries], dtype=np.int32),
-                                np.asarray([e.tokens[0] for e in entries], dtype=np.int32))
+                                np.asarray([e.tokens[0] for e in entries], dtype=np.int32)).values
 
-    def step_arrays(self, ids, starts, tokens, tokens_dev=None) -> torch.Tensor:
+    def step_arrays(self, ids, starts, tokens, tokens_dev=None) -> Logits:
         """The same from numpy arrays: request ids (int64), position and id of
         each request's one new token (int32); or the ids of the tokens as a
-        tensor on the device (``tokens_dev``)."""
+        tensor on the device (``tokens_dev``).  Returns the rows' ``Logits``."""
         fixed = FixedStep(rows=_batch_bucket(len(ids)), max_context=self._context_bucket(int(starts.max()) + 1))
         return self._captured(fixed).run(self.runner, ids, starts, tokens, tokens_dev)
 
@@ -150,7 +146,7 @@ class StepGraphs:
         prompt step: one request, more than one token, no more than the largest bucket."""
         return self.safe and len(count) == 1 and 1 < int(count[0]) <= self.PROMPT_TOKENS[-1]
 
-    def prompt_step_arrays(self, ids, starts, counts, tokens) -> torch.Tensor:
+    def prompt_step_arrays(self, ids, starts, counts, tokens) -> Logits:
         """A short prompt (or its last portion) alone in a step: logits [1, vocab] of its last token."""
         rows = next(t for t in self.PROMPT_TOKENS if t >= int(counts.sum()))
         fixed = FixedStep(rows=len(ids), max_context=self._context_bucket(int((starts + counts).max())), tokens=rows)

@@ -91,8 +91,9 @@ class LLMEngine:
                                                cache_groups=config.cache_groups, num_state_slots=config.max_num_seqs,
                                                max_model_len=config.max_model_len)
         spec = self.core.model.spec
-        # (the model's position tables may have fewer rows than spec.max_position: as many as the
-        # pool could ever hold; a request longer than that is refused for its pages, not its length)
+        # (the model's position tables may have fewer rows than spec.max_position: as many as a request
+        # can reach, EngineCore.reach; where a pool that keeps every token is the bound, a longer request
+        # is refused for its pages, not its length)
         self.max_model_len = min(config.max_model_len or spec.max_position, spec.max_position)
         eos = config.eos_token_ids if config.eos_token_ids is not None else spec.eos_token_ids
         self.scheduler = Scheduler(self.core.cache, max_num_seqs=config.max_num_seqs,

@@ -23,7 +23,7 @@ import torch
 from ..cache.manager import CacheError, CacheManager, CachePools
 from ..kernels import ops
 from ..models.decoder import DecoderModel
-from ..parts.base import FixedStep, GroupView, LayerCache, StepBatch, StepContext, StepPlan
+from ..parts.base import FixedStep, GroupView, LayerCache, Logits, StepBatch, StepContext, StepPlan
 
 
 @dataclass
@@ -108,15 +108,13 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.max_position = model.max_positions
         self.workspace: dict = {}
-        ops.require_gpu()
+        self._gpu_checked = False      # the tables are host work; the device is asked for at the first launch
         # what each call of the running order gets, apart from the step's tables
         self._calls = []
         for call in model.schedule:
             g = self.layout.group_of(call.cache)
-            k = v = None
-            if g is not None:
-                _, k, v = pools.buffer(call.cache)
-            self._calls.append((g, k, v, pools.state.get(call.cache), call.writes))
+            pages = pools.buffer(call.cache)[1] if g is not None else {}
+            self._calls.append((g, pages, pools.state.get(call.cache), call.writes))
         # the parts' planners, one per distinct key, in the order the parts come
         self.planners: dict = {}
         for _, part in model.named_parts():
@@ -301,6 +299,9 @@ class ModelRunner:
     def build_context_arrays(self, ids, start, count, tokens, rows) -> StepContext:
         """The eager step's context: tables written into pinned memory and read
         from there by one small kernel (see ``step_tables`` for the arguments)."""
+        if not self._gpu_checked:
+            ops.require_gpu()
+            self._gpu_checked = True
         tables = self.step_tables(ids, start, count, tokens, rows, host_for=lambda n: self._ring.take(n).numpy())
         dev = torch.empty(tables.host.size, dtype=torch.int32, device=self.device)
         ops.table_load(self._ring.buffers[self._ring.turn], dev)
@@ -308,8 +309,8 @@ class ModelRunner:
         return self.context(tables, dev)
 
     def layer_caches(self, ctx: StepContext) -> list:
-        return [LayerCache(group=ctx.groups[g] if g is not None else None, k=k, v=v, state=state, writes=writes)
-                for g, k, v, state, writes in self._calls]
+        return [LayerCache(group=ctx.groups[g] if g is not None else None, pages=pages, state=state, writes=writes)
+                for g, pages, state, writes in self._calls]
 
     # --------------------------------------------------------------- the step
     def step(self, entries: list) -> Optional[torch.Tensor]:
@@ -317,9 +318,11 @@ class ModelRunner:
         ``want`` lists, or None when nothing is wanted.  The cache is written
         for every token of the step either way."""
         ctx = self.build_context(entries)
-        return self.model.forward(ctx, self.layer_caches(ctx))
+        out = self.model.forward(ctx, self.layer_caches(ctx))
+        return None if out is None else out.values
 
-    def step_arrays(self, ids, start, count, tokens, rows) -> Optional[torch.Tensor]:
-        """``step`` from numpy arrays (see ``step_tables``)."""
+    def step_arrays(self, ids, start, count, tokens, rows) -> Optional[Logits]:
+        """``step`` from numpy arrays (see ``step_tables``); the result with what the head left
+        for the sampler beside the values (``parts.base.Logits``)."""
         ctx = self.build_context_arrays(ids, start, count, tokens, rows)
         return self.model.forward(ctx, self.layer_caches(ctx))

@@ -4,7 +4,7 @@ csrc/engine/scheduler.cpp:7-138, bound there with pybind11,
 csrc/bindings.cpp:552-621)."""
 from __future__ import annotations
 
-from ctypes import POINTER, c_float, c_int32, c_int64, c_uint64
+from ctypes import POINTER, c_int32, c_int64
 from dataclasses import dataclass
 
 import numpy as np
@@ -72,10 +72,9 @@ class Scheduler:
 
     def add(self, seq_id: int, prompt: list, params: SamplingParams) -> None:
         arr = np.ascontiguousarray(prompt, dtype=np.int32)
+        # the scheduler gets what decides when a request ends; how tokens are chosen stays with the sampler
         self._rc(self._lib.lyp_sched_add(self._h, seq_id, arr.ctypes.data_as(POINTER(c_int32)), len(arr),
-                                         params.temperature, params.top_p,
-                                         params.top_k, params.max_tokens, int(params.ignore_eos),
-                                         c_uint64((params.seed or 0) & ((1 << 64) - 1))))
+                                         params.max_tokens, int(params.ignore_eos)))
 
     def abort(self, seq_id: int) -> bool:
         return bool(self._rc(self._lib.lyp_sched_abort(self._h, seq_id)))

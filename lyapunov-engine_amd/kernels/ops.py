@@ -663,13 +663,13 @@ LM_HEAD_MAX_ROWS = 16     # beyond that the activations are read again per 16 ro
 LM_HEAD_BLOCKS = 1024     # workgroups of the output-head kernel (measured: 256 129 us, 512 116, 1024 104, 2048 105)
 
 
-def lm_head(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """Float logits x @ w.T for the output head [vocab, hidden].  Few rows (a
-    decode step's) take a kernel of their own that reads the matrix with few
-    long-lived waves and leaves, beside the logits, every workgroup's largest
-    logit per row: the tensor returned then carries ``argmax_candidates`` (a
-    tensor [rows, workgroups, 2] of (value bits, index) pairs), which ``sample``
-    uses instead of a pass over the row.  Anything else goes through ``linear``."""
+def lm_head(x: torch.Tensor, w: torch.Tensor) -> tuple:
+    """-> (float logits x @ w.T for the output head [vocab, hidden], row maxima
+    or None).  Few rows (a decode step's) take a kernel of their own that reads
+    the matrix with few long-lived waves and leaves, beside the logits, every
+    workgroup's largest logit per row: an int32 tensor [rows, workgroups, 2] of
+    (value bits, index) pairs, which ``sample`` takes as ``row_maxima`` instead
+    of a pass over the row.  Anything else goes through ``linear``."""
     M, K = x.shape
     if M <= LM_HEAD_MAX_ROWS and w.dtype == x.dtype and w.shape[1] == K and w.stride(1) == 1 and x.stride(1) == 1:
         _dev(x)
@@ -682,9 +682,8 @@ def lm_head(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         if rc < 0:
             _check(rc, lib)
         if rc > 0:
-            out.argmax_candidates = cand if rc == LM_HEAD_BLOCKS else cand.view(-1)[:M * rc * 2].view(M, rc, 2)
-            return out
-    return linear(x, w, out_dtype=torch.float32)
+            return out, (cand if rc == LM_HEAD_BLOCKS else cand.view(-1)[:M * rc * 2].view(M, rc, 2))
+    return linear(x, w, out_dtype=torch.float32), None
 
 
 def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -816,11 +815,12 @@ def table_load(src: torch.Tensor, dst: torch.Tensor, patch: torch.Tensor | None 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            uniform: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor | None = None,
-           mirror: torch.Tensor | None = None) -> torch.Tensor:
+           mirror: torch.Tensor | None = None, row_maxima: torch.Tensor | None = None) -> torch.Tensor:
     """One token per row of logits.  With a ``workspace`` (``sample_workspace``)
-    the search for each row's maximum is spread over the chip.  ``mirror``: pinned
-    host memory (int32, a row each) that receives the tokens as well, readable
-    once the work on the stream up to here is done."""
+    the search for each row's maximum is spread over the chip; with
+    ``row_maxima`` (what ``lm_head`` returns beside these very logits) there is
+    no search.  ``mirror``: pinned host memory (int32, a row each) that receives
+    the tokens as well, readable once the work on the stream up to here is done."""
     _dev(temperature, top_k, top_p, uniform, out, workspace)
     if not logits.is_cuda or logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("sample: logits must be a 2-d GPU tensor whose rows are contiguous")
@@ -835,11 +835,11 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     if any(t.numel() != R for t in (temperature, top_k, top_p, uniform, out)):
         raise KernelError("sample: one parameter per row")
     lib = core()
-    cand = getattr(logits, "argmax_candidates", None)
+    cand = row_maxima
     if cand is not None:   # the head's kernel left the row maxima in pieces: no pass over the row for them
         if cand.dtype != torch.int32 or cand.dim() != 3 or cand.shape[0] < R or cand.shape[2] != 2 or \
                 not cand.is_contiguous() or cand.device != logits.device:
-            raise KernelError("sample: the logits' argmax candidates must be a contiguous int32 tensor [rows, pieces, 2]")
+            raise KernelError("sample: the row maxima must be a contiguous int32 tensor [rows, pieces, 2]")
         _check(lib.lyp_sample_cand(_p(logits), logits.stride(0), R, V, _p(temperature), _p(top_k), _p(top_p),
                                    _p(uniform), _p(cand), cand.shape[1], _p(out),
                                    mirror.data_ptr() if mirror is not None else None, _stream()), lib)

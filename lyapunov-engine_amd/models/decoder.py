@@ -20,13 +20,13 @@ import torch
 from ..config.registry import BLOCKS, EMBEDDINGS, HEADS, NORMS
 from ..config.specs import LayerCall, ModelSpec
 from ..kernels import ops
-from ..parts.base import (KVCacheSpec, LayerCache, Part, PositionEncoding, StateSpec, StepContext, WeightSource,
+from ..parts.base import (LayerCache, Logits, PagedSpec, Part, PositionEncoding, StateSpec, StepContext, WeightSource,
                           WeightSpec)
 
 
 @dataclass(frozen=True)
 class CacheGroupLayout:
-    spec: KVCacheSpec
+    spec: PagedSpec
     buffers: tuple          # cache ids (LayerCall.cache) whose keys and values live in this group
 
 
@@ -159,9 +159,10 @@ class DecoderModel(Part):
         self.head.materialize(self.device, dtype)
 
     # ---------------------------------------------------------------- compute
-    def forward(self, ctx: StepContext, caches: list) -> Optional[torch.Tensor]:
+    def forward(self, ctx: StepContext, caches: list) -> Optional[Logits]:
         """Run the step's tokens through every call of the running order;
-        returns float logits [R, vocab] for ``ctx.logit_rows`` (None if R == 0).
+        returns the float logits [R, vocab] for ``ctx.logit_rows`` as a
+        ``Logits`` (None if R == 0).
         ``caches[i]`` is the LayerCache of ``schedule[i]``."""
         h = self.embedding.forward(ctx, ctx.token_ids)
         delta = None
@@ -172,7 +173,8 @@ class DecoderModel(Part):
         if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
             delta = delta.run()
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
-        return self.head.forward(ctx, x)
+        out = self.head.forward(ctx, x)
+        return out if isinstance(out, Logits) else Logits(out)
 
 
 def build_model(spec: ModelSpec) -> DecoderModel:

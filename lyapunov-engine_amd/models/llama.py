@@ -11,7 +11,7 @@ from __future__ import annotations
 
 from ..config.model_config import LlamaConfig
 from ..config.registry import register_architecture
-from ..config.specs import LayerSpec, ModelSpec, PartSpec, default_schedule
+from ..config.specs import HF_LAYER_NAMES, HF_PREFIXES, LayerSpec, ModelSpec, PartSpec, default_schedule
 
 
 def llama_spec(cfg: LlamaConfig) -> ModelSpec:
@@ -30,7 +30,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         "position": position,
     })
     ffn = PartSpec("swiglu", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size})
-    layer = LayerSpec(block="prenorm", mixer=mixer, ffn=ffn, norm1=norm, norm2=norm)
+    layer = LayerSpec(block="prenorm", mixer=mixer, ffn=ffn, norm1=norm, norm2=norm, names=HF_LAYER_NAMES)
     return ModelSpec(
         vocab_size=cfg.vocab_size,
         hidden_size=cfg.hidden_size,
@@ -42,6 +42,7 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
         eos_token_ids=tuple(cfg.eos_token_id),
         # older exports carry every layer's rotary frequencies as a buffer; they are computed here
         ignorable_tensors=("*.rotary_emb.inv_freq",),
+        **HF_PREFIXES,   # model.embed_tokens., model.layers.{i}., model.norm., lm_head. (models/weight_loader.py:85-170)
     )
 
 

@@ -23,7 +23,7 @@ import torch
 from ..config.registry import MIXERS, POSITION_ENCODINGS
 from ..config.specs import PartSpec
 from ..kernels import ops
-from .base import KVCacheSpec, LayerCache, Mixer, StepBatch, StepContext, StepPlanner, WeightSource, WeightSpec
+from .base import LayerCache, PagedSpec, Mixer, StepBatch, StepContext, StepPlanner, WeightSource, WeightSpec
 
 PREFILL_TILE = 64   # new tokens of one request per workgroup of the prefill attention kernel
 
@@ -122,10 +122,38 @@ class PagedAttention(Mixer):
         return {"rotary.": self.position} if self.position is not None else {}
 
     def cache_spec(self):
-        return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
+        return PagedSpec.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
 
     def step_planner(self):
         return _WORK
+
+    # The launch shapes of the two attention kernels for a step, from the planner's host values
+    # alone (no device work: a test can check them against the kernels' index ranges).
+    def prefill_launch(self, meta: dict, dtype: torch.dtype, page_size: int) -> Optional[dict]:
+        """For the tiles of requests that bring several tokens: in how many runs every tile's keys
+        are cut, whether workgroups pair a light tile with a heavy one, and the floats of the
+        workspaces the runs' partial results need.  None: no tiles."""
+        n_tiles = meta["n_tiles"]
+        if not n_tiles:
+            return None
+        # Tiles come in rising order of the keys they see; when the first sees less than half
+        # of what the last does, a workgroup may take one from each end.
+        few, many = (min(k, self.window + 64) if self.window else k for k in meta["tile_keys"])
+        # few new tokens over many keys: the keys in runs, for workgroups of their own
+        parts = ops.attn_prefill_plan(n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim, dtype, page_size)
+        n = n_tiles * PREFILL_TILE * self.num_heads * parts if parts > 1 else 0
+        return dict(n_tiles=n_tiles, parts=parts, pair=2 * few <= many, part_o=n * self.head_dim, part_ml=n * 2)
+
+    def decode_launch(self, meta: dict) -> Optional[dict]:
+        """For the requests that bring one token: keys per workgroup, the most partitions a
+        request can have, and the floats of the partitions' workspaces.  None: no such request."""
+        n_dec, max_ctx = meta["n_dec"], meta["max_ctx_dec"]
+        if not n_dec:
+            return None
+        part = ops.attn_decode_plan(n_dec, max_ctx, self.num_heads, self.num_kv_heads, self.head_dim)
+        max_parts = max(1, (max_ctx + part - 1) // part)
+        n = n_dec * self.num_heads * max_parts
+        return dict(n_dec=n_dec, part_keys=part, max_parts=max_parts, part_o=n * self.head_dim, part_ml=n * 2)
 
     takes_pending_norm = True   # x may be an ops.PendingNorm: the q/k/v product norms on its way in
 
@@ -141,28 +169,20 @@ class PagedAttention(Mixer):
         common = dict(num_heads=self.num_heads, num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                       window=self.window, scale=self.scale)
         work = ctx.plans[AttentionWork.key]
-        n_tiles, n_dec, max_ctx_dec = work.meta["n_tiles"], work.meta["n_dec"], work.meta["max_ctx_dec"]
-        if n_tiles:
-            # Tiles come in rising order of the keys they see; when the first sees less than half
-            # of what the last does, a workgroup may take one from each end.
-            few, many = (min(k, self.window + 64) if self.window else k for k in work.meta["tile_keys"])
-            # few new tokens over many keys: the keys in runs, for workgroups of their own
-            parts = ops.attn_prefill_plan(n_tiles, many, self.num_heads, self.num_kv_heads, self.head_dim,
-                                          ctx.dtype, g.page_size)
+        pre = self.prefill_launch(work.meta, ctx.dtype, g.page_size)
+        if pre is not None:
             part_o = part_ml = None
-            if parts > 1:
-                n = n_tiles * PREFILL_TILE * self.num_heads * parts
-                part_o = ctx.scratch("attn_part_o", n * self.head_dim)
-                part_ml = ctx.scratch("attn_part_ml", n * 2)
+            if pre["parts"] > 1:
+                part_o = ctx.scratch("attn_part_o", pre["part_o"])
+                part_ml = ctx.scratch("attn_part_ml", pre["part_ml"])
             ops.attn_prefill(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len,
-                             work.arrays["tile_seq"], work.arrays["tile_q0"], n_tiles, pair=2 * few <= many,
-                             parts=parts, part_o=part_o, part_ml=part_ml, **common)
-        if n_dec:
-            part = ops.attn_decode_plan(n_dec, max_ctx_dec, self.num_heads, self.num_kv_heads, self.head_dim)
-            max_parts = max(1, (max_ctx_dec + part - 1) // part)
-            n = n_dec * self.num_heads * max_parts
-            part_o = ctx.scratch("attn_part_o", n * self.head_dim)
-            part_ml = ctx.scratch("attn_part_ml", n * 2)
+                             work.arrays["tile_seq"], work.arrays["tile_q0"], pre["n_tiles"], pair=pre["pair"],
+                             parts=pre["parts"], part_o=part_o, part_ml=part_ml, **common)
+        dec = self.decode_launch(work.meta)
+        if dec is not None:
+            part_o = ctx.scratch("attn_part_o", dec["part_o"])
+            part_ml = ctx.scratch("attn_part_ml", dec["part_ml"])
             ops.attn_decode(qkv, out, cache.k, cache.v, g.block_tables, ctx.q_start, ctx.ctx_len,
-                            work.arrays.get("dec"), n_dec, part_o, part_ml, max_parts, part, **common)
+                            work.arrays.get("dec"), dec["n_dec"], part_o, part_ml, dec["max_parts"], dec["part_keys"],
+                            **common)
         return ops.linear(out, self.o_proj, out_dtype=ctx.dtype, may_split=True, pending=True)

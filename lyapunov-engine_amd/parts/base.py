@@ -81,14 +81,43 @@ class Part:
 
 
 # ----------------------------------------------------------------------- cache
-@dataclass(frozen=True)
-class KVCacheSpec:
-    """Keys and values in pages.  Calls whose specs are equal share a group:
-    one pool of pages, one block table per request."""
+SLOT = -1   # in a PageTensor's shape: the dimension that runs over the token slots of a page
 
-    num_kv_heads: int
-    head_dim: int
-    window: int = 0        # 0: all keys; W: a token sees the last W keys, itself included
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One of the tensors a mixer keeps per token in pages.  ``shape`` is the
+    shape of one page with ``SLOT`` where the page's token slots run (its
+    extent is the group's page size): ``(heads, SLOT, head_dim)`` keeps a
+    token's values side by side, ``(heads, head_dim, SLOT)`` keeps the slots of
+    one dimension side by side.  ``dtype`` None: the engine's activation type."""
+
+    name: str
+    shape: tuple
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> tuple:
+        if self.shape.count(SLOT) != 1:
+            raise ValueError(f"page tensor {self.name!r}: exactly one dimension is the token slot, got {self.shape}")
+        return tuple(page_size if d == SLOT else int(d) for d in self.shape)
+
+
+@dataclass(frozen=True)
+class PagedSpec:
+    """What a mixer keeps per token, in pages: the layout is the mixer's, the
+    pages, block tables and their reuse are the cache manager's.  Calls whose
+    specs are equal share a group: one pool of pages, one block table per
+    request."""
+
+    tensors: tuple         # of PageTensor
+    window: int = 0        # 0: every token is kept; W: a token needs the last W tokens' entries, its own included
+
+    @classmethod
+    def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int = 0) -> "PagedSpec":
+        """The layout the attention kernels of this package read: keys
+        [heads][slot][head_dim], values [heads][head_dim][slot]."""
+        return cls((PageTensor("k", (num_kv_heads, SLOT, head_dim)), PageTensor("v", (num_kv_heads, head_dim, SLOT))),
+                   int(window))
 
 
 @dataclass(frozen=True)
@@ -116,10 +145,19 @@ class LayerCache:
     """What one call of a layer gets from the cache."""
 
     group: Optional[GroupView] = None
-    k: Optional[torch.Tensor] = None      # [pages, kv heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None      # [pages, kv heads, head_dim, page_size]
+    pages: dict = field(default_factory=dict)   # PageTensor.name -> [pages, *PageTensor.page_shape(page size)]
     state: Optional[torch.Tensor] = None  # [slots, *StateSpec.shape]
     writes: bool = True                   # false: read what another call stored
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        """The pool named "k" (``PagedSpec.keys_and_values``: [pages, kv heads, page_size, head_dim])."""
+        return self.pages.get("k")
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        """The pool named "v" ([pages, kv heads, head_dim, page_size])."""
+        return self.pages.get("v")
 
 
 @dataclass
@@ -242,8 +280,27 @@ class Embedding(Part):
         raise NotImplementedError
 
 
+@dataclass
+class Logits:
+    """What a step returns for the rows whose logits were wanted: the float
+    logits [R, vocab] and, when the head's kernel produced them on its way,
+    ``row_maxima``: int32 [R, pieces, 2], for every row the largest logit
+    (its bits) and the first place it stands at within each of ``pieces``
+    stretches of the vocabulary.  The sampler uses them instead of a pass over
+    the row; a head that changes the logits after its product (a bias, a cap)
+    returns none, or ones that hold for the changed values."""
+
+    values: torch.Tensor
+    row_maxima: Optional[torch.Tensor] = None
+
+    def first(self, n: int) -> "Logits":
+        """The first ``n`` rows (views)."""
+        return Logits(self.values[:n], None if self.row_maxima is None else self.row_maxima[:n])
+
+
 class Head(Part):
-    """From the normed rows whose logits are wanted to float logits [R, vocab]."""
+    """From the normed rows whose logits are wanted to float logits [R, vocab]:
+    ``forward`` returns a ``Logits``, or just the tensor of values."""
 
     def tie(self, embedding: Embedding) -> None:
         """The model ties its head to the embedding: use ``embedding.weight``
@@ -251,7 +308,7 @@ class Head(Part):
         cannot raises."""
         raise NotImplementedError(f"{type(self).__name__} cannot share the embedding's matrix")
 
-    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> "Logits | torch.Tensor":
         raise NotImplementedError
 
 
@@ -276,7 +333,7 @@ class Mixer(Part):
     # computed), which the part's first product folds in.
     takes_pending_norm = False
 
-    def cache_spec(self) -> Optional[KVCacheSpec]:
+    def cache_spec(self) -> Optional[PagedSpec]:
         return None
 
     def state_spec(self) -> Optional[StateSpec]:
@@ -306,7 +363,7 @@ class Block(Part):
 
 
 __all__ = [
-    "WeightSource", "WeightSpec", "Part", "KVCacheSpec", "StateSpec", "GroupView", "LayerCache", "StepContext",
+    "WeightSource", "WeightSpec", "Part", "PagedSpec", "PageTensor", "SLOT", "StateSpec", "GroupView", "LayerCache", "StepContext",
     "StepBatch", "StepPlan", "StepPlanner", "FixedStep",
-    "Norm", "PositionEncoding", "Mixer", "FeedForward", "Block", "Any",
+    "Norm", "PositionEncoding", "Mixer", "FeedForward", "Block", "Logits", "Any",
 ]

@@ -16,7 +16,7 @@ import torch
 
 from ..config.registry import EMBEDDINGS, HEADS
 from ..kernels import ops
-from .base import Embedding, Head, StepContext, WeightSource, WeightSpec
+from .base import Embedding, Head, Logits, StepContext, WeightSource, WeightSpec
 
 
 @EMBEDDINGS.register("lookup")
@@ -52,5 +52,5 @@ class LinearHead(Head):
         if self._tied_to is not None:
             self.weight = self._tied_to.weight      # one matrix, two uses
 
-    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
-        return ops.lm_head(x, self.weight)
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> Logits:
+        return Logits(*ops.lm_head(x, self.weight))

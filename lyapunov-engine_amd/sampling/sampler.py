@@ -15,6 +15,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from ..parts.base import Logits
 from .params import SamplingParams
 
 _MASK = (1 << 64) - 1
@@ -74,10 +75,14 @@ class Sampler:
             self._work = ops.sample_workspace(self._cap, self.device)
             self._greedy_on_device = True   # the device block is all zeros: temperature 0 everywhere
 
-    def launch(self, logits: torch.Tensor, params: list, streams: list, indices: list) -> PendingSample:
-        """logits [R, vocab] float on the device; one SamplingParams, stream id
-        and output index per row.  Starts the choice of R token ids and their
-        copy to the host; nothing waits here."""
+    def launch(self, logits, params: list, streams: list, indices: list) -> PendingSample:
+        """``logits``: a step's ``Logits`` (values [R, vocab] float on the device,
+        with the row maxima its head may have left), or just the tensor of
+        values; one SamplingParams, stream id and output index per row.  Starts
+        the choice of R token ids and their copy to the host; nothing waits here."""
+        row_maxima = None
+        if isinstance(logits, Logits):
+            logits, row_maxima = logits.values, logits.row_maxima
         R = logits.shape[0]
         if not (len(params) == len(streams) == len(indices) == R):
             raise ValueError("one set of sampling parameters per row of logits")
@@ -102,7 +107,8 @@ class Sampler:
         out = bufs["out"][:R]
         host = bufs["out_host"][:R]
         # the kernel writes the tokens to the pinned buffer itself: no copy after it
-        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work, mirror=host)
+        ops.sample(logits, d[0, :R], d[3, :R].view(torch.int32), d[1, :R], d[2, :R], out, self._work, mirror=host,
+                   row_maxima=row_maxima)
         bufs["event"].record()
         return PendingSample(out, host, bufs["event"])
 

@@ -121,8 +121,12 @@ def load_model(model_dir: str, dtype: torch.dtype, device="cuda:0", source: Opti
                max_positions: Optional[int] = None):
     """config.json -> architecture -> model, with its tensors from the folder's
     safetensors files.  Returns (model, typed configuration).  ``max_positions``:
-    see ``DecoderModel.materialize``."""
+    see ``DecoderModel.materialize``; a function is called with the model as
+    built (its parts and cache layout are known, its weights not yet loaded) and
+    returns the number."""
     arch, cfg = load_config(model_dir)
     model = build_model(arch.to_spec(cfg))
+    if callable(max_positions):
+        max_positions = max_positions(model)
     load_weights(model, source or FolderSource(model_dir), dtype, device, max_positions)
     return model, cfg

@@ -141,7 +141,11 @@ def test_model_structure_follows_the_configuration():
         assert len(names) == 9 * cfg.num_hidden_layers + 2 + (0 if cfg.tie_word_embeddings else 1)
         layout = model.cache_layout()
         assert len(layout.groups) == 1 and layout.groups[0].buffers == tuple(range(cfg.num_hidden_layers))
-        assert layout.groups[0].spec.num_kv_heads == cfg.num_key_value_heads and not layout.states
+        from lyapunov_engine_amd.parts import SLOT
+        k, v = layout.groups[0].spec.tensors      # the layout is the mixer's: keys [heads][slot][hd], values [heads][hd][slot]
+        assert (k.name, k.shape) == ("k", (cfg.num_key_value_heads, SLOT, cfg.head_dim)) and not layout.states
+        assert (v.name, v.shape) == ("v", (cfg.num_key_value_heads, cfg.head_dim, SLOT))
+        assert k.page_shape(16) == (cfg.num_key_value_heads, 16, cfg.head_dim)
         assert sum(1 for _ in model.named_parts()) > 0
         total = sum(int(__import__("math").prod(s)) for s, _ in names.values())
         assert total == cfg.num_parameters()

@@ -802,9 +802,9 @@ def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     want = x.double() @ w.double().T
     for blocks in (8, 512):
         monkeypatch.setattr(ops, "LM_HEAD_BLOCKS", blocks)
-        out = ops.lm_head(x.to(DEV), w.to(DEV))
+        out, maxima = ops.lm_head(x.to(DEV), w.to(DEV))
         torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 1e-2))
-        cand = out.argmax_candidates.cpu()
+        cand = maxima.cpu()
         assert cand.shape[0] == M and cand.shape[2] == 2 and cand.shape[1] <= blocks
         values, places = cand[..., 0].contiguous().view(torch.float32), cand[..., 1]
         got = out.cpu()
@@ -821,10 +821,8 @@ def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
         top_p = torch.tensor(([1.0, 1.0, 0.8] * R)[:R]).to(DEV)
         u = torch.rand(R, generator=torch.Generator().manual_seed(3)).to(DEV)
         a, b = torch.empty(R, dtype=torch.int32, device=DEV), torch.empty(R, dtype=torch.int32, device=DEV)
-        ops.sample(out, temperature, top_k, top_p, u, a)
-        plain_logits = out.clone()                      # a copy carries no candidates
-        assert getattr(plain_logits, "argmax_candidates", None) is None
-        ops.sample(plain_logits, temperature, top_k, top_p, u, b, ops.sample_workspace(R, DEV))
+        ops.sample(out, temperature, top_k, top_p, u, a, row_maxima=maxima)
+        ops.sample(out, temperature, top_k, top_p, u, b, ops.sample_workspace(R, DEV))   # with a pass over the row
         assert a.tolist() == b.tolist()
         assert a[0] == int(got[0].argmax())
 
@@ -890,11 +888,12 @@ def test_sampler_writes_a_token_for_rows_without_a_largest_logit(ops):
     x = rnd(3, K, dtype=torch.bfloat16, seed=7)
     x[1] = float("nan")
     w = rnd(V, K, dtype=torch.bfloat16, scale=0.2, seed=8)
-    head = ops.lm_head(x.to(DEV), w.to(DEV))
-    assert getattr(head, "argmax_candidates", None) is not None
+    head, maxima = ops.lm_head(x.to(DEV), w.to(DEV))
+    assert maxima is not None
     out = torch.full((3,), -1, dtype=torch.int32, device=DEV)
     z = torch.zeros(3, device=DEV)
-    ops.sample(head, z, torch.full((3,), -1, dtype=torch.int32, device=DEV), torch.ones(3, device=DEV), z, out)
+    ops.sample(head, z, torch.full((3,), -1, dtype=torch.int32, device=DEV), torch.ones(3, device=DEV), z, out,
+               row_maxima=maxima)
     got = out.cpu().tolist()
     assert got[1] == 0 and got[0] == int(head[0].argmax()) and got[2] == int(head[2].argmax())
 

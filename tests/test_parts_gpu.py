@@ -15,6 +15,8 @@ import torch
 from plain import llama_plain as P
 from trace_util import Trace, random_tokens, replay
 
+from lyapunov_engine_amd.config import HF_LAYER_NAMES, HF_PREFIXES   # the toys' files use these tensor names
+
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
@@ -196,11 +198,11 @@ def register_toy():
         borrower = PartSpec("paged_attention", dict(attn, position=rope, own_kv=False))
         recur = PartSpec("toy_linear_recurrence", {"hidden_size": H, "state_size": c["state_size"],
                                                    "decay": c["decay"]})
-        layers = tuple(LayerSpec("prenorm", m, ffn, norm, norm) for m in (full, recur, windowed, borrower))
+        layers = tuple(LayerSpec("prenorm", m, ffn, norm, norm, HF_LAYER_NAMES) for m in (full, recur, windowed, borrower))
         # layer 0 runs twice (caches 0 and 3); layer 3 reads what the first call of layer 0 stored
         schedule = (LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2), LayerCall(0, 3), LayerCall(3, 0, writes=False))
         return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=schedule,
-                         final_norm=norm, tie_word_embeddings=False, max_position=c["max_position"])
+                         final_norm=norm, tie_word_embeddings=False, max_position=c["max_position"], **HF_PREFIXES)
 
     register_architecture("ToyMixForCausalLM", ToyConfig, to_spec, replace=True)
 
@@ -385,9 +387,10 @@ def register_toy2():
         routed = PartSpec("toy_routed_experts", {"hidden_size": H, "expert_size": c["expert_size"],
                                                  "experts": c["experts"]})
         dense = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
-        layers = (LayerSpec("prenorm", attn, routed, norm, norm), LayerSpec("prenorm", attn, dense, norm, norm))
+        layers = (LayerSpec("prenorm", attn, routed, norm, norm, HF_LAYER_NAMES),
+                  LayerSpec("prenorm", attn, dense, norm, norm, HF_LAYER_NAMES))
         return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=default_schedule(2),
-                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"])
+                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"], **HF_PREFIXES)
 
     register_architecture("ToyRoutedForCausalLM", ToyConfig, to_spec, replace=True)
 
@@ -531,9 +534,10 @@ def register_toy3():
         attn = PartSpec("paged_attention", dict(hidden_size=H, num_heads=c["num_heads"], num_kv_heads=c["num_kv_heads"],
                                                 head_dim=c["head_dim"], position=rope))
         scan = PartSpec("toy_scan_on_device", {"hidden_size": H, "state_size": c["state_size"], "decay": c["decay"]})
-        layers = (LayerSpec("prenorm", attn, ffn, norm, norm), LayerSpec("prenorm", scan, ffn, norm, norm))
+        layers = (LayerSpec("prenorm", attn, ffn, norm, norm, HF_LAYER_NAMES),
+                  LayerSpec("prenorm", scan, ffn, norm, norm, HF_LAYER_NAMES))
         return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=default_schedule(2),
-                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"])
+                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"], **HF_PREFIXES)
 
     register_architecture("ToyScanForCausalLM", ToyConfig, to_spec, replace=True)
 
@@ -688,7 +692,8 @@ def register_toy4():
             return [WeightSpec("bias", (WeightSource("bias", (self.vocab_size,)),))]
 
         def forward(self, ctx, x):
-            logits = ops.lm_head(x, self.table.weight) + self.bias.float()
+            # the product's row maxima do not hold for capped, biased logits: only the values are returned
+            logits = ops.lm_head(x, self.table.weight)[0] + self.bias.float()
             return torch.tanh(logits / self.cap) * self.cap
 
     EMBEDDINGS.register("toy_scaled_lookup", ScaledLookup, replace=True)
@@ -704,12 +709,12 @@ def register_toy4():
                                                 num_kv_heads=c["num_key_value_heads"], head_dim=c["head_dim"], position=pos))
         ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
         n = c["num_hidden_layers"]
-        layer = LayerSpec("toy_sandwich", attn, ffn, norm, norm, extra={"post_mixer": norm, "post_ffn": norm})
+        layer = LayerSpec("toy_sandwich", attn, ffn, norm, norm, HF_LAYER_NAMES, extra={"post_mixer": norm, "post_ffn": norm})
         return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=tuple(layer for _ in range(n)),
                          schedule=default_schedule(n), final_norm=norm, tie_word_embeddings=True,
                          max_position=c["max_position_embeddings"],
                          embedding=PartSpec("toy_scaled_lookup", {"scale": c["embed_scale"]}),
-                         head=PartSpec("toy_capped_head", {"cap": c["logit_cap"]}))
+                         head=PartSpec("toy_capped_head", {"cap": c["logit_cap"]}), **HF_PREFIXES)
 
     register_architecture("ToyEndsForCausalLM", ToyConfig, to_spec, replace=True)
 
