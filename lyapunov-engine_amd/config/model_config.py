@@ -9,7 +9,9 @@ not a silent 1B default.  Keys whose absence has a meaning by the convention of
 the file format have that meaning (``num_key_value_heads`` -> as many as query
 heads, ``head_dim`` -> hidden_size // num_attention_heads as in
 weight_loader.py:30-34, ``rope_scaling`` -> none, ``tie_word_embeddings`` ->
-false).
+false, ``rope_theta`` -> 10000.0: files of the format's first generation do not
+name the base and mean that one; the reference's fallback is the 1B model's
+500000.0, weight_loader.py:37, which would rotate such a model's heads wrongly).
 """
 from __future__ import annotations
 
@@ -67,8 +69,9 @@ class RopeScaling:
 
 _REQUIRED = (
     "vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
-    "max_position_embeddings", "rms_norm_eps", "rope_theta",
+    "max_position_embeddings", "rms_norm_eps",
 )
+ROPE_THETA_CONVENTION = 10000.0   # what a config.json of this format means when it does not name rope_theta
 
 
 def _as_id_tuple(v: Any) -> tuple:
@@ -118,7 +121,7 @@ class LlamaConfig:
                 raise ConfigError(f"hidden_size {hidden} does not split over {nh} heads and no head_dim is given")
             head_dim = hidden // nh
         known = set(_REQUIRED) | {
-            "num_key_value_heads", "head_dim", "rope_scaling", "tie_word_embeddings", "architectures",
+            "rope_theta", "num_key_value_heads", "head_dim", "rope_scaling", "tie_word_embeddings", "architectures",
             "eos_token_id", "bos_token_id", "torch_dtype", "attention_bias", "mlp_bias", "hidden_act",
         }
         nkv = d.get("num_key_value_heads")
@@ -132,7 +135,7 @@ class LlamaConfig:
             head_dim=int(head_dim),
             max_position_embeddings=int(d["max_position_embeddings"]),
             rms_norm_eps=float(d["rms_norm_eps"]),
-            rope_theta=float(d["rope_theta"]),
+            rope_theta=float(d.get("rope_theta", ROPE_THETA_CONVENTION)),
             rope_scaling=RopeScaling.from_dict(d.get("rope_scaling")),
             tie_word_embeddings=bool(d.get("tie_word_embeddings", False)),
             architectures=tuple(d.get("architectures") or ("LlamaForCausalLM",)),

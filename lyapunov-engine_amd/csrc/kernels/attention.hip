@@ -1250,11 +1250,11 @@ int lyp_attn_decode_plan(int n_seqs, int max_ctx, int nh, int nkv) {
   const int g = nh / (nkv > 0 ? nkv : 1);
   const long long base = static_cast<long long>(B) * nkv * ((g + 15) / 16);
   // Partitions grow while the launch keeps this many workgroups: one or two requests do best with one
-  // workgroup per compute unit (batch 1 at 32,768 keys: 21.2 us a layer with 256 workgroups of
-  // 1,024 keys, 23.7 with 512 of 512), more requests with two; with heads of more than 64 values
-  // (a key is twice the bytes) one per compute unit at every batch (heads of 128, batch 8 at
-  // 8,192 keys: 53.2 us with partitions of 2,048 keys, 56.7 with 1,024).
-  const int enough = (base < 32 || HD > 64) ? 256 : 512;
+  // workgroup per compute unit (on 256 units, batch 1 at 32,768 keys: 21.2 us a layer with 256
+  // workgroups of 1,024 keys, 23.7 with 512 of 512), more requests with two; with heads of more than
+  // 64 values (a key is twice the bytes) one per compute unit at every batch (heads of 128, batch 8
+  // at 8,192 keys: 53.2 us with partitions of 2,048 keys, 56.7 with 1,024).
+  const int enough = compute_units() * ((base < 32 || HD > 64) ? 1 : 2);
   int kpw = kPartKeys;
   while (kpw < 1024) {
     const int next_block = kDecodeWaves * kpw * 2;
@@ -1370,8 +1370,11 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
 }
 
 // part_keys: keys per workgroup, from lyp_attn_decode_plan.  part_o needs
-// n_seqs * nh * max_parts * hd floats, part_ml n_seqs * nh * max_parts * 2, with
-// max_parts >= ceil(longest context / part_keys).
+// n_seqs * nh * max_parts * hd floats, part_ml n_seqs * nh * max_parts * 2.
+// Precondition, which only the caller can check (the contexts are on the device): every request's
+// context is at most max_parts * part_keys.  The grid has max_parts workgroups per request and
+// head group; keys of a longer request beyond those partitions would be left out without a sign
+// (with max_parts == 1 the one workgroup writes the output itself from part_keys keys at most).
 int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, const void* kpool,
                     const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                     const int32_t* q_start, const int32_t* ctx_len, const int32_t* dec_seqs, int n_seqs,

@@ -339,6 +339,17 @@ __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, siz
   if (idx < n) out[idx] = from_f32<TO>(to_f32(in[idx]));
 }
 
+// out[i] = parts[0][i] + parts[1][i] + ... in that order, in 32-bit: the float partial sums of a
+// product whose inner dimension was cut into slices, for a consumer that is not a norm.
+template <typename TO>
+__global__ void sum_parts_kernel(const float* __restrict__ parts, int n_parts, size_t n, TO* __restrict__ out) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  float acc = parts[idx];
+  for (int s = 1; s < n_parts; ++s) acc += parts[static_cast<size_t>(s) * n + idx];
+  out[idx] = from_f32<TO>(acc);
+}
+
 // Threads per row of the two-pass norm kernels (rows whose length or alignment keeps them from
 // the one-pass kernel).  Measured on gfx950 with 2,048 rows (kernel_bench rmsnorm): up to 1,024
 // values one or two waves are as good as any size; at 2,050 values 256 threads take 11.4 us where
@@ -589,6 +600,22 @@ int lyp_cast(const void* in, int in_dtype, void* out, int out_dtype, long long n
   else
     LYP_REQUIRE(false, "cast: unsupported pair %d -> %d", in_dtype, out_dtype);
   LYP_LAUNCH_CHECK("cast");
+  return 0;
+}
+
+// out [n] (float or the activation type) = the sum over parts [n_parts][n] (float), slice by slice.
+int lyp_sum_parts(const float* parts, int n_parts, long long n, void* out, int out_dtype, hipStream_t stream) {
+  LYP_REQUIRE(n >= 0 && n_parts >= 1, "sum_parts: %d parts of %lld values", n_parts, n);
+  if (n == 0) return 0;
+  const int threads = 256;
+  const unsigned blocks = static_cast<unsigned>((n + threads - 1) / threads);
+  if (out_dtype == kF32)
+    sum_parts_kernel<float><<<blocks, threads, 0, stream>>>(parts, n_parts, static_cast<size_t>(n), static_cast<float*>(out));
+  else if (out_dtype == kBF16)
+    sum_parts_kernel<bf16_t><<<blocks, threads, 0, stream>>>(parts, n_parts, static_cast<size_t>(n), static_cast<bf16_t*>(out));
+  else
+    LYP_REQUIRE(false, "sum_parts: unknown output type %d", out_dtype);
+  LYP_LAUNCH_CHECK("sum_parts");
   return 0;
 }
 

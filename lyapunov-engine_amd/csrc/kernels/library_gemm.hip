@@ -83,6 +83,59 @@ bool g_tuning_all = true;      // screen all of the library's solutions, not onl
     }                                                                              \
   } while (0)
 
+// ---- a candidate's result against the heuristic's first choice
+// A solution the library lists for a shape is not thereby right for it: before a measured
+// candidate may win, its output on the call's own operands is held against the output of the
+// heuristic's first choice.  Two sums of the same products in another order differ by rounding:
+// a few units in the last place of the output type, relative to the larger of the two values,
+// and for values that cancel, relative to the matrix's largest value.
+__global__ void max_abs_kernel(const void* x, int is_f32, int M, int N, int ld, unsigned* out) {
+  float m = 0.f;
+  const size_t total = static_cast<size_t>(M) * N;
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t at = (i / N) * ld + i % N;
+    const float v = is_f32 ? static_cast<const float*>(x)[at] : to_f32(static_cast<const bf16_t*>(x)[at]);
+    m = fmaxf(m, fabsf(v));   // a NaN is not counted here; the comparison below counts it
+  }
+  atomicMax(out, __float_as_uint(m));   // non-negative floats order as their bits do
+}
+
+__global__ void count_off_kernel(const void* got, const void* ref, int is_f32, int M, int N, int ld,
+                                 const unsigned* ref_max, unsigned* off) {
+  const float scale = __uint_as_float(*ref_max);
+  const float rel = is_f32 ? 1e-4f : 1.6e-2f;   // bf16: two units in the last place (8 bits)
+  const float floor_ = (is_f32 ? 1e-5f : 2e-3f) * scale;
+  unsigned n = 0;
+  const size_t total = static_cast<size_t>(M) * N;
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t at = (i / N) * ld + i % N;
+    const float a = is_f32 ? static_cast<const float*>(got)[at] : to_f32(static_cast<const bf16_t*>(got)[at]);
+    const float b = is_f32 ? static_cast<const float*>(ref)[at] : to_f32(static_cast<const bf16_t*>(ref)[at]);
+    const float d = fabsf(a - b);
+    if (!(d <= rel * fmaxf(fabsf(a), fabsf(b)) + floor_)) ++n;   // also when either is a NaN
+  }
+  if (n) atomicAdd(off, n);
+}
+
+// How many values of `got` are off `ref` (both [M, N], rows ld apart) by more than rounding; -1 if
+// the check itself failed.  `scratch`: two unsigned values on the device.  Waits for the stream.
+long long values_off(const void* got, const void* ref, int is_f32, int M, int N, int ld, unsigned* scratch,
+                     hipStream_t stream) {
+  unsigned host[2] = {0, 0};
+  if (hipMemcpyAsync(scratch, host, sizeof(host), hipMemcpyHostToDevice, stream) != hipSuccess) return -1;
+  const int blocks = 256;
+  max_abs_kernel<<<blocks, 256, 0, stream>>>(ref, is_f32, M, N, ld, scratch);
+  count_off_kernel<<<blocks, 256, 0, stream>>>(got, ref, is_f32, M, N, ld, scratch, scratch + 1);
+  if (hipMemcpyAsync(host, scratch, sizeof(host), hipMemcpyDeviceToHost, stream) != hipSuccess ||
+      hipStreamSynchronize(stream) != hipSuccess)
+    return -1;
+  return host[1];
+}
+
+int g_rejected = 0;   // candidates turned down because their output was off (for tests and the log)
+
 // Runs the product `times` times with candidate `c`; false if the library refuses it.
 bool run_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulHeuristicResult_t& c, const void* a,
                    const void* w, void* out, void* workspace, hipStream_t stream, int times) {
@@ -101,16 +154,21 @@ bool run_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmu
 // with other data and the activations are read once.  Candidates ranked with everything still
 // in the cache from the run before were slower in the step than the library's first choice.
 int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMatmulHeuristicResult_t* found, int n_found,
-                      const void* a, size_t a_bytes, const void* w, void* out, void* workspace, size_t workspace_bytes,
-                      hipStream_t stream, float* first_ms, float* chosen_ms) {
+                      const void* a, size_t a_bytes, const void* w, void* out, int out_is_f32, int M, int N, int ldo,
+                      void* workspace, size_t workspace_bytes, hipStream_t stream, float* first_ms, float* chosen_ms) {
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return 0;
   constexpr size_t kFlushBytes = size_t{512} << 20;   // twice the memory-side cache
+  const size_t out_bytes = (static_cast<size_t>(M - 1) * ldo + N) * (out_is_f32 ? 4 : 2);
   void* other = nullptr;
-  if (hipMalloc(&other, kFlushBytes + a_bytes) != hipSuccess) {
+  if (hipMalloc(&other, kFlushBytes + ((a_bytes + 15) / 16) * 16 + ((out_bytes + 15) / 16) * 16 + 16) != hipSuccess) {
     (void)hipGetLastError();
     return 0;
   }
+  // behind the flush area and the copy of the activations: the first choice's output, and two counters
+  void* ref_out = static_cast<char*>(other) + kFlushBytes + ((a_bytes + 15) / 16) * 16;
+  unsigned* counters = reinterpret_cast<unsigned*>(static_cast<char*>(ref_out) + ((out_bytes + 15) / 16) * 16);
+  bool have_ref = false;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int best = 0;
   float best_ms = -1.f;
@@ -118,6 +176,19 @@ int fastest_candidate(hipblasLtHandle_t handle, const Plan& p, const hipblasLtMa
     for (int c = 0; c < n_found; ++c) {
       if (found[c].workspaceSize > workspace_bytes) continue;
       if (!run_candidate(handle, p, found[c], a, w, out, workspace, stream, 1)) continue;
+      if (c == 0) {
+        have_ref = hipMemcpyAsync(ref_out, out, out_bytes, hipMemcpyDeviceToDevice, stream) == hipSuccess;
+      } else {
+        // without the first choice's output to hold it against, no other candidate is taken
+        const long long off = have_ref ? values_off(out, ref_out, out_is_f32, M, N, ldo, counters, stream) : -1;
+        if (off != 0) {
+          ++g_rejected;
+          if (getenv("LYAPUNOV_AMD_GEMM_LOG"))
+            fprintf(stderr, "[lyapunov-amd] product %d x %d: candidate %d (solution %d) turned down, %lld values off the "
+                    "first choice's\n", M, N, c, hipblaslt_ext::getIndexFromAlgo(const_cast<hipblasLtMatmulAlgo_t&>(found[c].algo)), off);
+          continue;
+        }
+      }
       float fastest = -1.f;
       for (int run = 0; run < 3; ++run) {
         float ms = 0.f;
@@ -251,7 +322,8 @@ int make_plan(hipblasLtHandle_t handle, Plan& p, int device, int M, int N, int K
   float first_ms = -1.f, chosen_ms = -1.f;
   const int chosen =
       n_found > 1 ? fastest_candidate(handle, p, found.data(), n_found, a, static_cast<size_t>(M - 1) * lda * 2 + static_cast<size_t>(K) * 2,
-                                      w, out, workspace, workspace_bytes, stream, &first_ms, &chosen_ms)
+                                      w, out, out_type == kF32 ? 1 : 0, M, N, ldo, workspace, workspace_bytes, stream,
+                                      &first_ms, &chosen_ms)
                   : 0;
   if (n_found > 1 && getenv("LYAPUNOV_AMD_GEMM_LOG"))
     fprintf(stderr, "[lyapunov-amd] product %d x %d x %d: %d candidates of the heuristic, %d of the screen; the heuristic's "
@@ -337,5 +409,18 @@ void lyp_library_gemm_tuning_all(int on) { g_tuning_all = on != 0; }
 
 // Number of plans kept (for tests).
 int lyp_library_gemm_plans() { return static_cast<int>(state().plans.size()); }
+
+// Candidates that were measured and turned down because their output differed from the heuristic's
+// first choice by more than rounding (for tests).
+int lyp_library_gemm_rejected() { return g_rejected; }
+
+// How the plan of a product was made: the library's solution index, or -1 if no plan of this shape is kept.
+int lyp_library_gemm_solution(int M, int N, int K, int lda, int ldw, int ldo, int out_dtype, int for_graph) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return -1;
+  auto it = state().plans.find(Key{device, M, N, K, lda, ldw, ldo, out_dtype, for_graph ? 1 : 0});
+  if (it == state().plans.end()) return -1;
+  return hipblaslt_ext::getIndexFromAlgo(it->second.algo);
+}
 
 }  // extern "C"

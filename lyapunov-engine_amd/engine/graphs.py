@@ -31,6 +31,13 @@ from ..parts.base import FixedStep, Logits
 from .runner import ModelRunner, StepError
 
 
+class RecordingFailed(RuntimeError):
+    """A step could not be recorded for lack of a resource (device memory, the
+    graph itself): the one failure of a recorded step that the engine answers
+    by stepping eagerly.  Errors in the tables or from a kernel's checks are
+    not of this kind and are raised as they are."""
+
+
 def _bucket(n: int, smallest: int) -> int:
     b = smallest
     while b < n:
@@ -74,11 +81,16 @@ class _Captured:
         # chosen by measurement, among those that need no workspace (no memset is to be
         # recorded).
         with ops.library_gemm_tuning(for_graph=True):
-            runner.model.forward(self.ctx, caches)
-            torch.cuda.synchronize()
-            self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph, pool=pool):
-                self.logits = runner.model.forward(self.ctx, caches)
+            try:
+                runner.model.forward(self.ctx, caches)
+                torch.cuda.synchronize()
+                self.graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.graph, pool=pool):
+                    self.logits = runner.model.forward(self.ctx, caches)
+            except ops.KernelError:
+                raise                      # a kernel's own check: a defect, not a shortage
+            except (torch.cuda.OutOfMemoryError, RuntimeError) as err:   # what torch raises when memory or the capture fails
+                raise RecordingFailed(f"{fixed}: {type(err).__name__}: {err}") from err
 
     def run(self, runner: ModelRunner, ids, starts, tokens, tokens_dev=None, counts=None) -> Logits:
         """``tokens_dev``: the token ids as an int32 tensor on the device, for a

@@ -30,7 +30,6 @@ step changes in place) does not look ahead.
 """
 from __future__ import annotations
 
-import sys
 from typing import Optional
 
 import numpy as np
@@ -39,7 +38,9 @@ import torch
 from ..config.engine_config import EngineConfig
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
+from ..utils import log
 from .core import EngineCore
+from .graphs import RecordingFailed
 from .scheduler import FINISH_REASON, STATUS, Scheduler
 
 
@@ -113,8 +114,23 @@ class LLMEngine:
         self._look_ahead = bool(config.lookahead) and not self.core.pools.state
         self._ahead: Optional[_Ahead] = None
         self.steps_taken_ahead = 0    # steps whose results came from a step started ahead
+        self.recording_failures: list = []   # why recorded steps or looking ahead were switched off, if they were
         if config.warmup:
             self._warm_up()
+
+    def counters(self) -> dict:
+        """What the scheduler and the cache manager counted so far, and what this engine did beside them."""
+        return dict(scheduler=self.scheduler.counters(), cache=self.core.cache.counters(),
+                    steps_taken_ahead=self.steps_taken_ahead,
+                    graphs_recorded=len(self.graphs.captured) if self.graphs is not None else 0,
+                    recording_failures=len(self.recording_failures))
+
+    def __del__(self):
+        try:
+            if log.level() == "debug" and hasattr(self, "scheduler"):
+                log.debug(f"engine dropped: {self.counters()}")
+        except Exception:  # noqa: BLE001  (an interpreter that is shutting down may have taken the modules away)
+            pass
 
     WARMUP_ID = -1   # the cache manager's name for the warm-up step's request; the scheduler counts from 0
 
@@ -146,8 +162,7 @@ class LLMEngine:
             try:
                 cache.extend(self.WARMUP_ID, n)
                 if len(sizes) > 2:
-                    print(f"[lyapunov-amd] warm-up: a step of {n} tokens (matrix-product algorithms chosen by measurement)",
-                          file=sys.stderr, flush=True)
+                    log.info(f"warm-up: a step of {n} tokens (matrix-product algorithms chosen by measurement)")
                 with ops.library_gemm_tuning():
                     self.core.runner.step_arrays(np.asarray([self.WARMUP_ID], dtype=np.int64), np.zeros(1, dtype=np.int32),
                                                  np.asarray([n], dtype=np.int32), np.zeros(n, dtype=np.int32),
@@ -223,16 +238,19 @@ class LLMEngine:
             logits = None
             recorded = decoding or (self.graphs is not None and bool(wants.all()) and self.graphs.prompt_usable(count))
             if recorded:
-                # A recorded step that cannot be had (a new shape that cannot be recorded, no memory
-                # for it) is no reason to lose the step: it runs eagerly, and so do all later ones.
+                # A recorded step that cannot be had for lack of memory is no reason to lose the step: it
+                # runs eagerly, and so do all later ones (``recording_failures`` says so to whoever asks).
+                # Anything else that goes wrong in a recorded step (its tables, a kernel's check) is a
+                # defect and is raised.
                 try:
                     if decoding:
                         logits = self.graphs.step_arrays(ids, start, tokens)
                     else:   # a short prompt alone in its step
                         logits = self.graphs.prompt_step_arrays(ids, start, count, tokens)
-                except Exception as err:  # noqa: BLE001
+                except RecordingFailed as err:
                     self.graphs.safe, self._look_ahead, decoding = False, False, False
-                    print(f"[lyapunov-amd] recorded steps switched off: {type(err).__name__}: {err}", file=sys.stderr)
+                    self.recording_failures.append(str(err))
+                    log.warn(f"recorded steps switched off: {err}")
             if logits is None:
                 rows = (np.cumsum(count, dtype=np.int32) - 1)[wants != 0]   # the last token of each request that wants
                 logits = self.core.runner.step_arrays(ids, start, count, tokens, rows)
@@ -242,14 +260,15 @@ class LLMEngine:
                 pending = self.sampler.launch(logits, [r.params for r in wanting], [r.stream for r in wanting],
                                               [len(r.outputs) for r in wanting])
         if decoding and self._look_ahead:
-            # Optional work must not break the planned step: whatever goes wrong in starting the next
-            # one (a new graph that cannot be recorded, no memory for it), this step's tokens still
+            # Optional work must not break the planned step: when the next one cannot be started
+            # because a new graph cannot be recorded (no memory for it), this step's tokens still
             # reach the scheduler; looking ahead is then switched off.
             try:
                 self._ahead = self._start_ahead(ids, start, reqs, pending)
-            except Exception as err:  # noqa: BLE001
+            except RecordingFailed as err:
                 self._ahead, self._look_ahead = None, False
-                print(f"[lyapunov-amd] looking ahead switched off: {type(err).__name__}: {err}", file=sys.stderr)
+                self.recording_failures.append(str(err))
+                log.warn(f"looking ahead switched off: {err}")
         sampled = pending.result() if pending is not None else []
         status = self.scheduler.post_step_status(sampled)
         outputs, k = [], 0

@@ -49,7 +49,9 @@ _lock = threading.Lock()
 
 
 def _say(msg: str) -> None:
-    print(f"[lyapunov-amd build] {msg}", file=sys.stderr, flush=True)
+    from ..utils import log
+
+    log.info(msg, prefix="[lyapunov-amd build]")
 
 
 def hipcc_path() -> str:

@@ -69,6 +69,7 @@ def core() -> ctypes.CDLL:
                                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                                 c_void_p]
         lib.lyp_cast.argtypes = [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p]
+        lib.lyp_sum_parts.argtypes = [c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p]
         lib.lyp_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]
         lib.lyp_sample.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -523,6 +524,8 @@ def blas() -> ctypes.CDLL:
         lib.lyp_library_gemm_nt.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_library_gemm_plans.restype = c_int
+        lib.lyp_library_gemm_rejected.restype = c_int
+        lib.lyp_library_gemm_solution.argtypes = [c_int] * 8
         lib.lyp_library_gemm_tuning.argtypes = [c_int, c_int]
         lib.lyp_library_gemm_tuning(*_blas_tuning)   # what a tuning context asked for before the library was there
         _blas_lib = lib
@@ -581,6 +584,18 @@ def library_gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torc
     _check(lib.lyp_library_gemm_nt(_p(a), _p(w), _p(out), _code(out.dtype), M, N, K, a.stride(0), w.stride(0),
                                    out.stride(0), _p(ws), ws.numel(), _stream()), lib)
     return out
+
+
+def library_gemm_rejected() -> int:
+    """Candidates that tuning measured and turned down because their output was off the
+    heuristic's first choice by more than rounding, so far in this process."""
+    return blas().lyp_library_gemm_rejected()
+
+
+def library_gemm_solution(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, for_graph: bool = False) -> int:
+    """The library's number for the algorithm kept for this product, -1 if the shape has no plan yet."""
+    return blas().lyp_library_gemm_solution(a.shape[0], w.shape[0], a.shape[1], a.stride(0), w.stride(0), out.stride(0),
+                                            _code(out.dtype), int(for_graph))
 
 
 def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
@@ -687,14 +702,17 @@ def lm_head(x: torch.Tensor, w: torch.Tensor) -> tuple:
 
 
 def sum_parts(parts: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    """Add up the partial sums ``linear(..., may_split=True)`` may return."""
+    """Add up the partial sums ``linear(..., may_split=True)`` may return (slice
+    by slice, in 32-bit), as a tensor [rows, features] of ``dtype``."""
     if parts.dim() == 2:
         return parts if parts.dtype == dtype else cast(parts, dtype)
-    h = torch.zeros(parts.shape[1:], dtype=torch.float32, device=parts.device)
-    ones = torch.ones(parts.shape[2], dtype=torch.float32, device=parts.device)
+    if parts.dim() != 3 or parts.dtype != torch.float32:
+        raise KernelError(f"sum_parts: float partial sums [slices, rows, features], not {tuple(parts.shape)} {parts.dtype}")
+    _dev(parts)
     out = torch.empty(parts.shape[1:], dtype=dtype, device=parts.device)
-    rmsnorm(h, ones, 0.0, out, delta=parts)     # the sum lands in h; the normed output is not what is wanted
-    return h if dtype == torch.float32 else cast(h, dtype)
+    lib = core()
+    _check(lib.lyp_sum_parts(_p(parts), parts.shape[0], out.numel(), _p(out), _code(dtype), _stream()), lib)
+    return out
 
 
 # ------------------------------------------------------------------- attention
@@ -768,7 +786,11 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
                 max_parts: int, part_keys: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
                 scale: float | None = None) -> torch.Tensor:
     """Attention of requests that bring one new token each, split over
-    partitions of the context and merged."""
+    partitions of the context and merged.  ``part_keys`` comes from
+    ``attn_decode_plan``; the caller guarantees that no request's context
+    exceeds ``max_parts * part_keys`` (the contexts live on the device and are
+    not read here: keys beyond that many partitions would silently be left
+    out).  ``PagedAttention.decode_launch`` derives both from the step's bound."""
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)

@@ -15,13 +15,13 @@ become int32.  With the engine in float32 every floating tensor becomes float32.
 """
 from __future__ import annotations
 
-import sys
 from typing import Optional
 
 import torch
 
 from ..config.registry import load_config
 from ..models.decoder import DecoderModel, build_model
+from ..utils import log
 from .safetensors_io import open_model_files
 
 
@@ -97,8 +97,8 @@ def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, 
     check_tensors(model, source.shapes())
     expected = model.expected_tensors()
     for name in sorted(n for n in source.shapes() if n not in expected):
-        print(f"[lyapunov-amd] note: {name} is in the files and not used by this model (a separate head of a tied "
-              f"model, or a buffer the architecture declares ignorable); ignored", file=sys.stderr)
+        log.info(f"note: {name} is in the files and not used by this model (a separate head of a tied "
+                 f"model, or a buffer the architecture declares ignorable); ignored")
     device = torch.device(device)
     for owner, ws in model.weight_table():
         pieces = [source.get(s.name) for s in ws.sources]

@@ -29,7 +29,7 @@ def test_every_size_comes_from_the_file():
     assert "transformers_version" in cfg.extra  # unknown keys are kept aside, not an error
     # a missing size is an error, not a silent default of some model
     for key in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers", "num_attention_heads",
-                "max_position_embeddings", "rms_norm_eps", "rope_theta"):
+                "max_position_embeddings", "rms_norm_eps"):
         d = dict(LLAMA_1B)
         del d[key]
         with pytest.raises(ConfigError, match=key):
@@ -38,8 +38,9 @@ def test_every_size_comes_from_the_file():
 
 def test_conventional_fallbacks():
     d = dict(TINY_A)
-    del d["head_dim"], d["num_key_value_heads"], d["tie_word_embeddings"], d["rope_scaling"]
+    del d["head_dim"], d["num_key_value_heads"], d["tie_word_embeddings"], d["rope_scaling"], d["rope_theta"]
     cfg = LlamaConfig.from_dict(d)
+    assert cfg.rope_theta == 10000.0        # the file format's convention, not some model's value (weight_loader.py:37 says 500000)
     assert cfg.head_dim == 64 // 4          # hidden_size // heads (reference: weight_loader.py:30-34)
     assert cfg.num_key_value_heads == 4     # as many as query heads
     assert cfg.tie_word_embeddings is False and cfg.rope_scaling is None
@@ -257,3 +258,23 @@ def test_embedding_and_head_are_parts_an_architecture_may_replace():
         EMBEDDINGS.unregister("test_scaled")
         HEADS.unregister("test_biased")
         HEADS.unregister("test_alone")
+
+
+def test_one_switch_decides_what_is_said(capsys, monkeypatch):
+    from lyapunov_engine_amd.utils import log
+
+    before = log.level()
+    try:
+        log.set_level("quiet")
+        log.info("progress"), log.debug("counters"), log.warn("switched off")
+        assert capsys.readouterr().err == "[lyapunov-amd] switched off\n"
+        log.set_level("info")
+        log.info("progress"), log.debug("counters")
+        assert capsys.readouterr().err == "[lyapunov-amd] progress\n"
+        log.set_level("debug")
+        log.debug("counters")
+        assert "counters" in capsys.readouterr().err
+        with pytest.raises(ValueError, match="one of"):
+            log.set_level("loud")
+    finally:
+        log.set_level(before)

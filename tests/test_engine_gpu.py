@@ -332,6 +332,7 @@ def test_a_step_ahead_that_cannot_start_does_not_break_the_planned_step(model_fo
     recorded, no memory for it), the planned step's tokens still reach the scheduler, looking ahead
     is switched off with a note, and generation gives the tokens it gives without looking ahead."""
     from lyapunov_engine_amd.config import EngineConfig
+    from lyapunov_engine_amd.engine.graphs import RecordingFailed
     from lyapunov_engine_amd.engine.llm_engine import LLMEngine
     from lyapunov_engine_amd.sampling.params import SamplingParams
 
@@ -347,7 +348,7 @@ def test_a_step_ahead_that_cannot_start_does_not_break_the_planned_step(model_fo
 
             def failing(ids, starts, tokens, tokens_dev=None):
                 if tokens_dev is not None:
-                    raise RuntimeError("no memory for a new graph")
+                    raise RecordingFailed("no memory for a new graph")
                 return real(ids, starts, tokens)
 
             engine.graphs.step_arrays = failing
@@ -360,6 +361,7 @@ def test_a_step_ahead_that_cannot_start_does_not_break_the_planned_step(model_fo
     got, engine = run(True, True)
     assert got == want and engine._look_ahead is False and engine.steps_taken_ahead == 0
     assert "looking ahead switched off" in capsys.readouterr().err
+    assert len(engine.recording_failures) == 1 and engine.counters()["recording_failures"] == 1
 
 
 def test_sampled_tokens_are_the_plain_rules_at_the_engines_uniform_numbers(model_folders):
@@ -445,7 +447,7 @@ def test_a_recorded_prompt_step_of_two_requests_equals_the_eager_step(model_fold
         starts = np.asarray([e.start for e in entries], dtype=np.int32)
         counts = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
         flat = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-        replayed = cap.run(runner, ids, starts, flat, counts=counts).clone()
+        replayed = cap.run(runner, ids, starts, flat, counts=counts).values.clone()
         for e in entries:
             cache.commit(e.seq_id, e.start + len(e.tokens))
         torch.testing.assert_close(replayed, eager, rtol=1e-5, atol=1e-5)
@@ -476,7 +478,7 @@ def test_a_step_that_cannot_be_recorded_runs_eagerly(model_folders, capsys):
 
     def failing(self, fixed):
         calls.append(fixed)
-        raise RuntimeError("out of memory while recording")
+        raise G.RecordingFailed("out of memory while recording")
 
     real = G.StepGraphs._captured
     G.StepGraphs._captured = failing
@@ -486,4 +488,131 @@ def test_a_step_that_cannot_be_recorded_runs_eagerly(model_folders, capsys):
         G.StepGraphs._captured = real
     assert got == want and len(calls) == 1 and llm.engine.graphs.safe is False
     assert "recorded steps switched off" in capsys.readouterr().err
+    assert llm.engine.recording_failures == ["out of memory while recording"]
     llm.engine.core.cache.check()
+
+
+def test_a_defect_in_a_recorded_step_is_raised_not_swallowed(model_folders):
+    """Only a shortage while recording is answered by stepping eagerly; an error from the step's
+    tables or from a kernel's own checks comes out as it is."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.engine import graphs as G
+    from lyapunov_engine_amd.kernels.ops import KernelError
+
+    folder = model_folders["B"]["float32"]
+    llm = L.LLM(folder, dtype="float32", num_blocks=24)
+
+    def broken(self, fixed):
+        raise KernelError("attention: partition workspace too small")
+
+    real = G.StepGraphs._captured
+    G.StepGraphs._captured = broken
+    try:
+        with pytest.raises(KernelError, match="workspace too small"):
+            llm.generate([random_tokens(12, 515, seed=3)], L.SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    finally:
+        G.StepGraphs._captured = real
+    assert llm.engine.graphs.safe is True and llm.engine.recording_failures == []
+
+
+# ------------------------------------------- recorded prompt steps at long contexts, windows
+LONG = dict(architectures=["LlamaForCausalLM"], vocab_size=300, hidden_size=128, intermediate_size=192,
+            num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+            max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True)
+
+
+def register_windowed(name, windows):
+    """A Llama whose layer i sees the last ``windows[i]`` keys (0: all of them), registered from here."""
+    from lyapunov_engine_amd.config import LlamaConfig, register_architecture
+    from lyapunov_engine_amd.config.specs import LayerSpec, ModelSpec, PartSpec
+    from lyapunov_engine_amd.models.llama import llama_spec
+
+    def to_spec(cfg):
+        spec = llama_spec(cfg)
+        layers = []
+        for layer, w in zip(spec.layers, windows):
+            mixer = PartSpec(layer.mixer.kind, dict(layer.mixer.params, window=w))
+            layers.append(LayerSpec(layer.block, mixer, layer.ffn, layer.norm1, layer.norm2, layer.names))
+        fields = {f: getattr(spec, f) for f in spec.__dataclass_fields__}
+        return ModelSpec(**dict(fields, layers=tuple(layers)))
+
+    register_architecture(name, LlamaConfig, to_spec, replace=True)
+
+
+@pytest.mark.parametrize("windows", [(0, 0), (0, 48)], ids=["all keys", "a windowed layer"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_recorded_last_portion_at_a_long_context_equals_the_eager_step(tmp_path, dtype, windows):
+    """The last portion of a long prompt, alone in its step, replays a recorded step whose bound is
+    the context's bucket: in bfloat16 its keys are cut into runs for workgroups of their own, the
+    unused tile entries pass through the merging kernel, and a windowed layer walks its window only.
+    Against the same step run eagerly on the same cache (the step writes the same keys to the same
+    slots again), logits and all."""
+    import numpy as np
+
+    from lyapunov_engine_amd.config import ARCHITECTURES
+    from lyapunov_engine_amd.engine.core import EngineCore, StepEntry
+    from lyapunov_engine_amd.engine.graphs import StepGraphs
+    from lyapunov_engine_amd.weights import write_random_model
+
+    arch = "WindowedLlamaForCausalLM"
+    register_windowed(arch, windows)
+    try:
+        folder = str(tmp_path / "long")
+        write_random_model(dict(LONG, architectures=[arch]), folder, seed=11, dtype=dtype, init_std=0.1, norm_init_std=0.1)
+        core = EngineCore.from_folder(folder, dtype=dtype, num_blocks=300, block_size=16, num_state_slots=2)
+        total, last = 4170, 90
+        toks = random_tokens(total, 300, seed=12)
+        core.cache.add(0)
+        for lo in range(0, total - last, 1020):
+            hi = min(total - last, lo + 1020)
+            core.cache.extend(0, hi)
+            core.step([StepEntry(0, toks[lo:hi], lo, [])])
+            core.cache.commit(0, hi)
+        core.cache.extend(0, total)
+        eager = core.step([StepEntry(0, toks[total - last:], total - last, [last - 1])]).clone()
+        graphs = StepGraphs(core.runner, max_batch=2)
+        ids, starts = np.zeros(1, np.int64), np.asarray([total - last], np.int32)
+        counts, flat = np.asarray([last], np.int32), np.asarray(toks[total - last:], np.int32)
+        assert graphs.prompt_usable(counts)
+        for _ in range(3):      # the capture, then replays
+            replayed = graphs.prompt_step_arrays(ids, starts, counts, flat).values.clone()
+            scale = float(eager.abs().max())
+            limit = 1e-5 if dtype == "float32" else 2e-2
+            assert float((replayed - eager).abs().max()) <= limit * scale
+        (key,) = graphs.captured
+        assert key == (1, 8192, 128)
+        if dtype == "bfloat16":  # the bound's keys in runs: the recorded launch merges partial results
+            meta = graphs.captured[key].ctx.plans[core.runner.model.layers[0].mixer.step_planner().key].meta
+            launch = core.runner.model.layers[0].mixer.prefill_launch(meta, core.dtype, 16)
+            assert launch["parts"] > 1 and launch["n_tiles"] == 3
+        core.cache.check()
+    finally:
+        ARCHITECTURES.unregister(arch)
+
+
+def test_a_model_of_windows_alone_generates_past_its_pool(tmp_path):
+    """Every layer keeps a window: pages come back as the window passes, so a request is bound by the
+    model's length, not by the pool.  Through the entry point, with a pool far smaller than the
+    request: the tokens are those of an engine whose pool holds the whole request."""
+    import lyapunov_engine_amd as L
+    from lyapunov_engine_amd.config import ARCHITECTURES
+    from lyapunov_engine_amd.weights import write_random_model
+
+    arch = "WindowsOnlyLlamaForCausalLM"
+    register_windowed(arch, (40, 24))
+    try:
+        folder = str(tmp_path / "windows")
+        write_random_model(dict(LONG, architectures=[arch], max_position_embeddings=1024), folder, seed=13,
+                           dtype="float32", init_std=0.1, norm_init_std=0.1)
+        prompt = random_tokens(50, 300, seed=14)
+        sp = L.SamplingParams(temperature=0.0, max_tokens=260, ignore_eos=True)
+        roomy = L.LLM(folder, dtype="float32", num_blocks=64, block_size=16, max_chunk=32)
+        want = roomy.generate([prompt], sp)[0].output_tokens
+        small = L.LLM(folder, dtype="float32", num_blocks=10, block_size=16, max_chunk=32)   # 160 tokens of pages
+        assert small.engine.core.runner.max_position == 1024          # not the pool's 160
+        got = small.generate([prompt], sp)[0]
+        assert got.output_tokens == want and len(want) == 260 and got.finish_reason == "length"
+        small.engine.core.cache.check()
+        assert small.engine.core.cache.counters()["window_returns"] > 0
+    finally:
+        ARCHITECTURES.unregister(arch)

@@ -279,6 +279,36 @@ def test_library_products_keep_one_plan_per_shape(ops):
         ops.library_gemm_nt(a.float(), w, torch.empty(M, N, dtype=torch.float32, device=DEV))
 
 
+def test_library_products_chosen_by_measurement_are_checked_products(ops):
+    """With tuning on (the engine's default outside the test session) a shape's first call screens
+    every solution the library lists and times the fastest few; whatever wins has had its output held
+    against the heuristic's first choice.  The products it leaves behind, both output types, against
+    float64; and an odd number of rows that comes up after tuning is over takes the choice measured
+    for its neighbour and is still the product."""
+    N, K = 776, 264          # a matrix no other test multiplies: its plans are made here
+    w = rnd(N, K, dtype=torch.bfloat16, scale=0.05, seed=72).to(DEV)
+
+    def check(M, out_dtype, rel):
+        a = rnd(M, K, dtype=torch.bfloat16, seed=70 + M).to(DEV)
+        out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops.library_gemm_nt(a, w, out)
+        ops.library_gemm_nt(a, w, out)        # the kept plan, once more
+        want = a.cpu().double() @ w.cpu().double().T
+        bound = a.cpu().double().abs() @ w.cpu().double().abs().T
+        assert ((out.cpu().double() - want).abs() <= rel * bound + 1e-30).all(), (M, out_dtype)
+        return ops.library_gemm_solution(a, w, out)
+
+    plans = ops.blas().lyp_library_gemm_plans()
+    with ops.library_gemm_tuning(candidates=16):
+        chosen = {M: check(M, torch.bfloat16, 1e-2) for M in (128, 520)}
+        check(128, torch.float32, 1e-5)
+    assert ops.blas().lyp_library_gemm_plans() == plans + 3 and all(c >= 0 for c in chosen.values())
+    assert ops.library_gemm_rejected() >= 0
+    # tuning is off again: 141 rows take what was measured at 128, 500 rows what was measured at 520
+    assert check(141, torch.bfloat16, 1e-2) == chosen[128]
+    assert check(500, torch.bfloat16, 1e-2) == chosen[520]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_tiled_product_takes_operands_that_are_column_ranges(ops, dtype, monkeypatch):
     """This package's tiled kernel with rows further apart than they are long (a column range of a

@@ -404,8 +404,8 @@ def test_the_largest_bfloat16_error_a_sweep_found(model_folders):
         got = replay(f, dtype, t)
         rel = compare(t, got, plain_for(model_folders, name, dtype, reqs), dtype, "seed 1098")
         compare_with_alone(t, got, f, dtype, "seed 1098")
-        if dtype == "bfloat16":
-            assert 0.05 < max(rel) < 0.08, f"the case is kept for its error of 7.3 %; it now shows {max(rel):.3f}"
+        if dtype == "bfloat16":   # (kernels that round better may bring it down; nothing may bring it up)
+            assert max(rel) < 0.08, f"the case is kept for its error of 7.3 %; it now shows {max(rel):.3f}"
 
 
 def test_bfloat16_without_the_vendor_library(model_folders, tmp_path, monkeypatch):
