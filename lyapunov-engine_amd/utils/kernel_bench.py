@@ -102,14 +102,72 @@ def attn_decode(a) -> None:
           f"{t * 1e6:.1f} us  {nbytes / t / 1e12:.2f} TB/s of keys and values ({max_parts} partitions of {part})")
 
 
+def _weights(a, rows: int, cols: int) -> list:
+    """The weight matrix of a product; with --cold as many copies as it takes to exceed twice the
+    memory-side cache, used in turn, so that every call finds its matrix in memory as a model step does."""
+    dt, dev = _dtype(a.dtype), a.device
+    one = rows * cols * (2 if dt == torch.bfloat16 else 4)
+    copies = max(1, -(-(512 << 20) // one)) if a.cold else 1
+    return [torch.randn(rows, cols, device=dev, dtype=dt) * 0.02 for _ in range(copies)]
+
+
+def _turns(ws: list):
+    state = {"i": 0}
+
+    def next_w():
+        state["i"] = (state["i"] + 1) % len(ws)
+        return ws[state["i"]]
+
+    return next_w
+
+
 def linear(a) -> None:
     dt, dev = _dtype(a.dtype), a.device
     x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
-    w = torch.randn(a.out_features, a.in_features, device=dev, dtype=dt) * 0.02
-    t = _time(lambda: ops.linear(x, w, may_split=a.may_split), a.repeat)
+    ws = _weights(a, a.out_features, a.in_features)
+    next_w = _turns(ws)
+    t = _time(lambda: ops.linear(x, next_w(), may_split=a.may_split), a.repeat)
     flops = 2.0 * a.rows * a.in_features * a.out_features
-    print(f"linear rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}: {t * 1e6:.1f} us  "
+    w = ws[0]
+    print(f"linear rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}{' cold' if a.cold else ''}: {t * 1e6:.1f} us  "
           f"{flops / t / 1e12:.1f} TFLOP/s  {w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
+
+
+def qkv(a) -> None:
+    """The fused q/k/v projection with rotation and page write (``ops.linear_rope_kv``)."""
+    dt, dev = _dtype(a.dtype), a.device
+    M, hd, nh, nkv = a.rows, a.head_dim, a.heads, a.kv_heads
+    x = torch.randn(M, a.in_features, device=dev, dtype=dt)
+    ws = _weights(a, (nh + 2 * nkv) * hd, a.in_features)
+    next_w = _turns(ws)
+    pages = -(-M // a.page_size) + 1
+    k, v = _pools(pages, a)
+    positions = torch.arange(M, dtype=torch.int32, device=dev)
+    slots = torch.arange(M, dtype=torch.int32, device=dev)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ang = torch.arange(max(M, 16), dtype=torch.float32)[:, None] * inv[None, :]
+    table = torch.cat([ang.cos(), ang.sin()], dim=1).contiguous().to(dev)
+
+    def run():
+        ops.linear_rope_kv(x, next_w(), positions, table, slots, k, v, num_heads=nh, num_kv_heads=nkv, head_dim=hd,
+                           page_size=a.page_size)
+
+    t = _time(run, a.repeat)
+    w = ws[0]
+    print(f"qkv rows={M} {w.shape[0]}x{w.shape[1]} {a.dtype}{' cold' if a.cold else ''}: {t * 1e6:.1f} us  "
+          f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
+
+
+def gate_up(a) -> None:
+    """The gate/up projection with the SiLU gate (``ops.linear_swiglu``, rows interleaved 8/8)."""
+    dt, dev = _dtype(a.dtype), a.device
+    x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
+    ws = _weights(a, a.out_features, a.in_features)
+    next_w = _turns(ws)
+    t = _time(lambda: ops.linear_swiglu(x, next_w(), 8), a.repeat)
+    w = ws[0]
+    print(f"gate_up rows={a.rows} {w.shape[0]}x{w.shape[1]} {a.dtype}{' cold' if a.cold else ''}: {t * 1e6:.1f} us  "
+          f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
 
 
 def head(a) -> None:
@@ -130,14 +188,15 @@ def residual(a) -> None:
     """The product that adds to the float residual stream and prepares the next norm."""
     dt, dev = _dtype(a.dtype), a.device
     x = torch.randn(a.rows, a.in_features, device=dev, dtype=dt)
-    w = torch.randn(a.out_features, a.in_features, device=dev, dtype=dt) * 0.02
+    ws = _weights(a, a.out_features, a.in_features)
+    next_w = _turns(ws)
+    w = ws[0]
     h = torch.zeros(a.rows, a.out_features, device=dev)
     nw = torch.ones(a.out_features, device=dev, dtype=dt)
-    pending = ops.PendingLinear(x, w, dt)
-    if ops.linear_residual(h, pending, nw) is False:
+    if ops.linear_residual(h, ops.PendingLinear(x, w, dt), nw) is False:
         raise SystemExit("the few-rows kernel does not take this shape")
-    t = _time(lambda: ops.linear_residual(h, pending, nw), a.repeat)
-    print(f"residual rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}: {t * 1e6:.1f} us  "
+    t = _time(lambda: ops.linear_residual(h, ops.PendingLinear(x, next_w(), dt), nw), a.repeat)
+    print(f"residual rows={a.rows} {a.out_features}x{a.in_features} {a.dtype}{' cold' if a.cold else ''}: {t * 1e6:.1f} us  "
           f"{w.numel() * w.element_size() / t / 1e12:.2f} TB/s of weights")
 
 
@@ -202,7 +261,10 @@ def rmsnorm(a) -> None:
 
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
-    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "residual", "sample", "stream", "rmsnorm", "head"])
+    ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "qkv", "gate_up", "residual", "sample", "stream",
+                                       "rmsnorm", "head"])
+    ap.add_argument("--cold", action="store_true", help="linear, qkv, gate_up, residual, head: the weights come from memory "
+                    "every time (copies of the matrix in turn), not from the memory-side cache")
     ap.add_argument("--megabytes", type=int, default=0, help="stream: size of the buffer (0: a range of sizes)")
     ap.add_argument("--blocks", type=int, default=0, help="stream: workgroups (0: a range)")
     ap.add_argument("--threads", type=int, default=0, help="rmsnorm: threads per row of the two-pass kernels (0: sweep)")
@@ -228,7 +290,7 @@ def main(argv=None) -> None:
     a = ap.parse_args(argv)
     ops.require_gpu()
     torch.manual_seed(0)
-    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "residual": residual,
+    {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "qkv": qkv, "gate_up": gate_up, "residual": residual,
      "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head}[a.kernel](a)
 
 

@@ -559,7 +559,7 @@ def test_a_recorded_last_portion_at_a_long_context_equals_the_eager_step(tmp_pat
     try:
         folder = str(tmp_path / "long")
         write_random_model(dict(LONG, architectures=[arch]), folder, seed=11, dtype=dtype, init_std=0.1, norm_init_std=0.1)
-        core = EngineCore.from_folder(folder, dtype=dtype, num_blocks=300, block_size=16, num_state_slots=2)
+        core = EngineCore.from_folder(folder, dtype=dtype, num_blocks=520, block_size=16, num_state_slots=2)
         total, last = 4170, 90
         toks = random_tokens(total, 300, seed=12)
         core.cache.add(0)
