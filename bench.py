@@ -177,12 +177,15 @@ def measure_mixed(engine, cfg, requests=64, seed=0):
     return time.perf_counter() - t0, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps
 
 
-CHECK_LIMIT = 0.02   # largest bf16-against-fp32 logit difference over the largest logit that passes
+# Largest bf16-against-fp32 logit difference over the largest logit that passes.  Measured on the 1B
+# shape at context 8,192: 0.8 % through 2 layers, 1.9 % through all 16 (rounding adds up roughly with
+# the square root of the depth); twice the measured value is allowed.
+CHECK_LIMIT = 0.04
 
 
-def check_logits(shape=MODEL, layers=2, context=8192, portion=2048):
+def check_logits(shape=MODEL, layers=None, context=8192, portion=2048):
     """The bfloat16 engine against the 32-bit engine at the benchmark's context, on the same shape
-    (fewer layers) and the same weights (random, rounded to bfloat16 for both, so that only the
+    at its full depth (``layers`` None) and the same weights (random, rounded to bfloat16 for both, so that only the
     arithmetic differs): a prompt of context - 1 tokens in portions, through the eager step, then
     one decoded token through the recorded graph of that context.  Returns, for the last prompt
     position and for the decoded position, the largest difference of the logits relative to the
@@ -194,6 +197,7 @@ def check_logits(shape=MODEL, layers=2, context=8192, portion=2048):
     from lyapunov_engine_amd.engine.runner import StepEntry
 
     prompt = random_prompt(context, shape["vocab_size"], 6)
+    layers = layers or shape["num_hidden_layers"]
     logits = {}
     for dtype in ("fp32", "bf16"):
         engine, _ = build_engine(layers, dtype, num_blocks=context // 16 + 8, max_num_seqs=1, block_size=16,
@@ -219,7 +223,10 @@ def check_logits(shape=MODEL, layers=2, context=8192, portion=2048):
         del engine, core, graphs
         torch.cuda.empty_cache()
     rel = [float((b - a).abs().max() / a.abs().max()) for a, b in zip(logits["fp32"], logits["bf16"])]
-    same = [bool(a.argmax() == b.argmax()) for a, b in zip(logits["fp32"], logits["bf16"])]
+    # the best token is the same, or the 32-bit logits of the two candidates are closer than the two
+    # engines' logits differ (random weights give nearly flat logits: such ties are the rule there)
+    same = [bool(a.argmax() == b.argmax()) or float(a.max() - a[b.argmax()]) <= 2 * float((b - a).abs().max())
+            for a, b in zip(logits["fp32"], logits["bf16"])]
     return rel, same
 
 
@@ -292,12 +299,12 @@ def main():
     if not args.skip_check:
         del engine
         torch.cuda.empty_cache()
-        rel, same = check_logits(shape, context=args.context)
-        check = {"what": f"bf16 against fp32 logits, same bf16-rounded weights, 2 layers, prompt of {args.context - 1} "
+        rel, same = check_logits(shape, layers=cfg.num_hidden_layers, context=args.context)
+        check = {"what": f"bf16 against fp32 logits, same bf16-rounded weights, {cfg.num_hidden_layers} layers, prompt of {args.context - 1} "
                          f"tokens in portions of 2048 (eager), then one decoded token at context {args.context} "
                          f"through the recorded graph; largest difference over largest logit",
                  "prompt_last": round(rel[0], 5), "decoded_through_graph": round(rel[1], 5), "limit": CHECK_LIMIT,
-                 "same_argmax": all(same), "ok": max(rel) <= CHECK_LIMIT}
+                 "best_token_same_or_tied": all(same), "ok": max(rel) <= CHECK_LIMIT and all(same)}
 
     peak = MFMA_PEAK[args.dtype]
     line = {
@@ -314,6 +321,9 @@ def main():
             "rope_scaling": f"llama3 factor {shape['rope_scaling']['factor']:g}", "global_batch": args.batch, "seq_len": int(round(mean_ctx)),
             "context_len": args.context, "kv_block_size": block_size, "prefill_tokens": 2048,
             "parallelism": "single-gpu", "graphs": True, "lookahead": lookahead,
+            "logits_check": "skipped" if check is None else
+                            f"bf16 vs fp32 engine, {cfg.num_hidden_layers} layers, context {args.context}: "
+                            f"{max(rel):.4f} of the largest logit (limit {CHECK_LIMIT}), {'ok' if check['ok'] else 'FAILED'}",
         },
         "prefill": {"value": round(2048 / prefill_s, 1), "tokens": 2048, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops(cfg, 2048) / prefill_s / peak, 4)},
@@ -325,7 +335,7 @@ def main():
     print(json.dumps(line))
     if check is not None and not check["ok"]:
         print(f"bench.py: bfloat16 logits at context {args.context} are off by {max(rel):.4f} of the largest logit "
-              f"(limit {CHECK_LIMIT})", file=sys.stderr)
+              f"(limit {CHECK_LIMIT}), or the two engines' best tokens differ beyond a tie", file=sys.stderr)
         return 1
     return 0
 

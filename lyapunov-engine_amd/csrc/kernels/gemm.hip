@@ -207,7 +207,9 @@ __device__ __forceinline__ int rope_feature(const RopeTail& t, int n0, int r) {
 // does two chunks of K (on the tile's diagonal blocks; the other two are not used) and no load
 // asks for a value twice.  With TB = 2 (9 to 16 tokens, 8 rows of W) a wave keeps two such tiles over
 // one set of weights: tokens 0-7 and 8-15.
-template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false, int TB = 1>
+// RT > 1 (steps of 17 to 64 tokens): a workgroup owns RT tiles of 16 rows of W, and a wave keeps all of them
+// over one set of activations: what a compute unit asks the cache for per row of W falls accordingly.
+template <typename T, int MB, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false, int TB = 1, int RT = 1>
 __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int lda,
                                                            int ldw, int ldc, RopeTail tail, NormHead head,
@@ -220,7 +222,8 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   static_assert(!PAIRED || (EPI == kEpiResidual && ((ROWS == 8 && MB == 1) || (ROWS == 16 && MB == 2))),
                 "two chunks per tile: 8 rows (or twice 8), 8 tokens");
   static_assert(TB == 1 || (TB == 2 && PAIRED && MB == 1), "blocks of 8 tokens: for the paired tile of 8 rows");
-  constexpr int NT = MB * TB;                // tiles (accumulators) a wave keeps
+  static_assert(RT == 1 || (!PAIRED && !NORMED && ROWS == 16 && EPI != kEpiResidual), "several row tiles: the plain tile only");
+  constexpr int NT = MB * TB * RT;           // tiles (accumulators) a wave keeps: tile rt * MB + b is row tile rt, token block b
   constexpr int NB = PAIRED ? TB : MB;       // blocks of tokens whose activations it loads
   constexpr int CHUNK = PAIRED ? 128 : 64;  // values of K per step of a wave
   extern __shared__ float red[];       // [waves][NT][64][4], then [waves][16] floats for the epilogues' row values
@@ -230,7 +233,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   // can be unrolled, which is what keeps several chunks' loads in flight
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int nwaves = blockDim.x / kWave;
-  const int n0 = blockIdx.x * ROWS;
+  const int n0 = blockIdx.x * ROWS * RT;
   const int r = lane % 16, j = lane / 16;
   int wrow = min(n0 + r % (PAIRED ? 8 : ROWS), N - 1);  // rows past the end read the last row and are not stored
   if constexpr (EPI == kEpiRope) wrow = rope_feature(tail, n0, r);  // N is a multiple of 16 here
@@ -288,6 +291,14 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
   const int second = PAIRED ? (r / 8) * 64 : 0;  // the tile's upper half: the chunk's second 64 values
   const T* wp = W + static_cast<size_t>(wrow) * ldw + j * MM::kElems + second;
+  const T* wpt[RT];        // the further row tiles' rows (a tile past the end of W reads its last row and is not stored)
+  wpt[0] = wp;
+#pragma unroll
+  for (int rt = 1; rt < RT; ++rt) {
+    int row = min(n0 + 16 * rt + r, N - 1);
+    if constexpr (EPI == kEpiRope) row = n0 + 16 * rt < N ? rope_feature(tail, n0 + 16 * rt, r) : N - 1;
+    wpt[rt] = W + static_cast<size_t>(row) * ldw + j * MM::kElems;
+  }
   const T* wp_upper = wp;  // PAIRED with 16 rows: the same lanes' rows 8-15
   if constexpr (PAIRED && MB == 2) wp_upper = W + static_cast<size_t>(min(n0 + 8 + r % 8, N - 1)) * ldw + j * MM::kElems + second;
   const T* ap[NB];  // rows past the end read the last row and are not stored
@@ -324,6 +335,16 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
         }
       return;
     }
+    Frag wx[RT > 1 ? RT - 1 : 1][U][NF];
+    if constexpr (RT > 1) {
+#pragma unroll
+      for (int rt = 1; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int f = 0; f < NF; ++f)
+            wx[rt - 1][u][f] = *reinterpret_cast<const Frag*>(wpt[rt] + (c + u) * CHUNK + f * 4 * MM::kElems);
+    }
     // the activations come from the cache: four chunks of them at a time are enough
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -339,15 +360,25 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
 #pragma unroll
         for (int u = 0; u < V; ++u)
 #pragma unroll
-          for (int f = 0; f < NF; ++f) acc[b] = MM::mma(wf[u0 + u][f], xf[u][f], acc[b]);
+          for (int f = 0; f < NF; ++f) {
+            acc[b] = MM::mma(wf[u0 + u][f], xf[u][f], acc[b]);
+            if constexpr (RT > 1) {
+#pragma unroll
+              for (int rt = 1; rt < RT; ++rt) acc[rt * MB + b] = MM::mma(wx[rt - 1][u0 + u][f], xf[u][f], acc[rt * MB + b]);
+            }
+          }
       }
     }
   };
   int c = c_begin;
-  for (; c + 4 <= c_end; c += 4) chunks_at(std::integral_constant<int, 4>{}, c);
+  if constexpr (RT == 1) {
+    for (; c + 4 <= c_end; c += 4) chunks_at(std::integral_constant<int, 4>{}, c);
+  } else {  // several row tiles' weights in flight: two chunks at a time keep the registers for more waves
+    for (; c + 2 <= c_end; c += 2) chunks_at(std::integral_constant<int, 2>{}, c);
+  }
   for (; c < c_end; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
 
-  // acc[b][i]: output feature n0 + 4 j + i, token 16 b + r
+  // acc[rt * MB + b][i]: output feature n0 + 16 rt + 4 j + i, token 16 b + r
   float* mine = red + (static_cast<size_t>(wave) * NT * 64 + lane) * 4;
 #pragma unroll
   for (int b = 0; b < NT; ++b) *reinterpret_cast<f32x4*>(mine + b * 256) = acc[b];
@@ -369,8 +400,11 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     return sum;
   };
   float* sq_el = row_val + nwaves * 16;  // kEpiResidual with by-products: [NT][256] squares of the new h, by element
+  const int n0_wg = n0;
   for (int e = threadIdx.x; e < NT * 256; e += blockDim.x) {
-    const int b = e / 256, l = (e % 256) / 4, i = e % 4;
+    const int b = RT == 1 ? e / 256 : (e / 256) % MB, l = (e % 256) / 4, i = e % 4;
+    const int n0 = RT == 1 ? n0_wg : n0_wg + 16 * (e / 256 / MB);   // this tile's first row of W
+    if (RT > 1 && n0 >= N) continue;
     const int in_tile = 4 * (l / 16) + i;
     // PAIRED: tile b holds rows 8 (b / TB) .. + 7 of W for tokens 8 (b % TB) .. + 7 (its lower left block; the
     // upper right one is added by total()); else rows 0-15 for tokens 16 b .. + 15
@@ -572,28 +606,55 @@ static int skinny_slices(int N, int K) {
 }
 
 // Waves per workgroup: enough of them over the whole launch to keep every
-// compute unit loading, within what LDS holds for the final sum.
-static int skinny_waves(int N, int K, int MB, int slices, int rows = 16, int chunk = 64) {
+// compute unit loading, within what LDS holds for the final sum (a kilobyte per
+// wave and tile a wave keeps).
+constexpr int kMostSumKilobytes = 96;
+
+static int skinny_waves(int N, int K, int tiles, int slices, int rows = 16, int chunk = 64) {
   const int row_blocks = (N + rows - 1) / rows;
   const int chunks = K / chunk / slices;
+  // up to 16 rows of tokens as it was measured for them: 32 kilobytes at most
+  const int most = tiles <= 2 ? 32 : kMostSumKilobytes;
   int waves = 1;
-  while (waves < 16 && waves * 2 * MB <= 32 && row_blocks * slices * waves < 4096 && waves * 2 <= chunks) waves *= 2;
+  while (waves < 16 && waves * 2 * tiles <= most && row_blocks * slices * waves < 4096 && waves * 2 <= chunks) waves *= 2;
   return waves;
 }
 
-template <typename T, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false>
+// Row tiles per workgroup for a step of more than 16 tokens (0: the rule below).  A workgroup
+// reads the step's activations over its whole share of K whatever rows of W it owns, so with two
+// tiles of 16 rows it asks the cache for half as much per row of W; fewer, larger workgroups in
+// exchange.  `g_row_tiles` (lyp_skinny_row_tiles_override) is there for measurements.
+static int g_row_tiles = 0;
+
+static int skinny_row_tiles(int M, int N, int slices) {
+  if (M <= 16) return 1;
+  if (g_row_tiles > 0) return g_row_tiles;
+  return (N / 32) * slices >= 128 ? 2 : 1;
+}
+
+template <typename T, int EPI, bool NORMED = false, int ROWS = 16, bool PAIRED = false, int RT = 1>
 static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                           int slices, hipStream_t stream, const RopeTail& tail = RopeTail{},
                           const NormHead& head = NormHead{}, const ResidualTail& res = ResidualTail{}) {
   // tiles a wave keeps: paired, 8 rows of W each for 8 tokens each; else 16 rows of W for 16 tokens each
   const int MB = PAIRED ? (ROWS / 8) * ((M + 7) / 8) : (M + 15) / 16;
-  const int waves = skinny_waves(N, K, MB, slices, ROWS, PAIRED ? 128 : 64);
-  const dim3 grid((N + ROWS - 1) / ROWS, slices), block(waves * kWave);
-  const size_t lds = (static_cast<size_t>(waves) * MB * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
+  const int waves = skinny_waves(N, K, MB * RT, slices, ROWS * RT, PAIRED ? 128 : 64);
+  const dim3 grid((N + ROWS * RT - 1) / (ROWS * RT), slices), block(waves * kWave);
+  const size_t lds = (static_cast<size_t>(waves) * MB * RT * 256 + waves * 16 + (EPI == kEpiResidual ? MB * 256 : 0)) *
                      sizeof(float);
-#define LYP_SKINNY_TB(MBV, TBV)                                                                                   \
-  gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED, TBV><<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, \
-                                                                                           ldc, tail, head, res)
+#define LYP_SKINNY_TB(MBV, TBV)                                                                                        \
+  do {                                                                                                                 \
+    auto kernel = gemm_skinny_kernel<T, MBV, EPI, NORMED, ROWS, PAIRED, TBV, RT>;                                      \
+    if (lds > 48 * 1024) {   /* more than a kernel gets without asking: said once per kernel */                       \
+      static bool asked = false;                                                                                       \
+      if (!asked) {                                                                                                    \
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                  (kMostSumKilobytes + 8) * 1024);                                                     \
+        asked = true;                                                                                                  \
+      }                                                                                                                \
+    }                                                                                                                  \
+    kernel<<<grid, block, lds, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, tail, head, res);                            \
+  } while (0)
 #define LYP_SKINNY(MBV) LYP_SKINNY_TB(MBV, 1)
   if constexpr (PAIRED && ROWS == 16) {
     LYP_SKINNY(2);  // at most 8 rows: the caller has checked
@@ -602,6 +663,10 @@ static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, 
     else LYP_SKINNY_TB(1, 2);  // at most 16 rows: the caller has checked
   } else if constexpr (NORMED) {
     LYP_SKINNY(1);  // at most 16 rows: the callers have checked
+  } else if constexpr (RT > 1) {
+    if (MB == 2) LYP_SKINNY(2);  // more than 16 rows: the caller has checked
+    else if (MB == 3) LYP_SKINNY(3);
+    else LYP_SKINNY(4);
   } else {
     if (MB == 1) LYP_SKINNY(1);
     else if (MB == 2) LYP_SKINNY(2);
@@ -610,6 +675,16 @@ static void launch_skinny(const T* A, const T* W, void* C, int M, int N, int K, 
   }
 #undef LYP_SKINNY
 #undef LYP_SKINNY_TB
+}
+
+// The plain tile with one or two row tiles per workgroup, as skinny_row_tiles says.
+template <typename T, int EPI>
+static void launch_skinny_rows(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                               int slices, hipStream_t stream, const RopeTail& tail = RopeTail{}) {
+  if (skinny_row_tiles(M, N, slices) >= 2)
+    launch_skinny<T, EPI, false, 16, false, 2>(A, W, C, M, N, K, lda, ldw, ldc, slices, stream, tail);
+  else
+    launch_skinny<T, EPI>(A, W, C, M, N, K, lda, ldw, ldc, slices, stream, tail);
 }
 
 template <typename T, int MODE>
@@ -648,11 +723,11 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
                        vec_ok, stream)
   if (mode != kAccumF32 && skinny_ok(M, K, lda, ldw, A, W, dtype)) {
     if (dtype == kF32)
-      launch_skinny<float, kEpiF32>(static_cast<const float*>(A), static_cast<const float*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
+      launch_skinny_rows<float, kEpiF32>(static_cast<const float*>(A), static_cast<const float*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else if (dtype == kBF16 && mode == kStoreF32)
-      launch_skinny<bf16_t, kEpiF32>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
+      launch_skinny_rows<bf16_t, kEpiF32>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else if (dtype == kBF16)
-      launch_skinny<bf16_t, kEpiAct>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
+      launch_skinny_rows<bf16_t, kEpiAct>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, 1, stream);
     else
       LYP_REQUIRE(false, "gemm: unknown dtype %d", dtype);
     LYP_LAUNCH_CHECK("gemm_skinny");
@@ -704,6 +779,24 @@ extern "C" int lyp_lm_head(const void* A, const void* W, float* C, int dtype, in
   return blocks;
 }
 
+// Row tiles per workgroup of the few-rows kernel in steps of more than 16 tokens (0: the built-in rule); for measurements.
+extern "C" int lyp_skinny_row_tiles_override(int row_tiles) {
+  LYP_REQUIRE(row_tiles >= 0 && row_tiles <= 2, "row tiles per workgroup: 0 (the rule), 1 or 2, not %d", row_tiles);
+  g_row_tiles = row_tiles;
+  return 0;
+}
+
+// Workgroups the few-rows kernel would launch for this product (with_slices: as partial sums over
+// slices of K, where lyp_gemm_parts_hint cuts it), 0 if the kernel does not take the shape.  The kernel
+// is one burst of loads per workgroup, so it is at its best while the launch is a single round of
+// workgroups on the machine: what the caller holds this number against.
+extern "C" int lyp_skinny_workgroups(int M, int N, int K, int with_slices) {
+  if (M < 1 || M > 64 || K % 64 != 0) return 0;
+  const int slices = with_slices ? skinny_slices(N, K) : 1;
+  const int rows = 16 * skinny_row_tiles(M, N, slices);
+  return ((N + rows - 1) / rows) * slices;
+}
+
 // How many partial sums lyp_gemm_nt_parts would produce for this product; 0 if
 // it does not apply (then use lyp_gemm_nt).
 extern "C" int lyp_gemm_parts_hint(const void* A, const void* W, int dtype, int M, int N, int K, int lda, int ldw) {
@@ -720,9 +813,9 @@ extern "C" int lyp_gemm_nt_parts(const void* A, const void* W, float* parts, int
   LYP_REQUIRE(skinny_ok(M, K, lda, ldw, A, W, dtype) && slices == skinny_slices(N, K) && slices > 1,
               "gemm_parts: M=%d N=%d K=%d slices=%d is not a case for partial sums", M, N, K, slices);
   if (dtype == kF32)
-    launch_skinny<float, kEpiParts>(static_cast<const float*>(A), static_cast<const float*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
+    launch_skinny_rows<float, kEpiParts>(static_cast<const float*>(A), static_cast<const float*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
   else if (dtype == kBF16)
-    launch_skinny<bf16_t, kEpiParts>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
+    launch_skinny_rows<bf16_t, kEpiParts>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), parts, M, N, K, lda, ldw, N, slices, stream);
   else
     LYP_REQUIRE(false, "gemm_parts: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gemm_parts");
@@ -738,9 +831,9 @@ extern "C" int lyp_gemm_swiglu(const void* A, const void* W, void* out, int dtyp
   LYP_REQUIRE(N % 16 == 0 && ldo >= N / 2, "gemm_swiglu: %d rows of weights, output stride %d", N, ldo);
   if (!skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
   if (dtype == kF32)
-    launch_skinny<float, kEpiSwiglu>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
+    launch_skinny_rows<float, kEpiSwiglu>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
   else if (dtype == kBF16)
-    launch_skinny<bf16_t, kEpiSwiglu>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
+    launch_skinny_rows<bf16_t, kEpiSwiglu>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream);
   else
     LYP_REQUIRE(false, "gemm_swiglu: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gemm_swiglu");
@@ -768,9 +861,9 @@ extern "C" int lyp_gemm_rope_kv(const void* A, const void* W, void* out, int dty
   if (rot % 16 != 0 || !skinny_ok(M, K, lda, ldw, A, W, dtype)) return 1;
   const RopeTail tail{positions, cos_sin, slots, kpool, vpool, nh, nkv, hd, rot, bs, has_kv};
   if (dtype == kF32)
-    launch_skinny<float, kEpiRope>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
+    launch_skinny_rows<float, kEpiRope>(static_cast<const float*>(A), static_cast<const float*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
   else if (dtype == kBF16)
-    launch_skinny<bf16_t, kEpiRope>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
+    launch_skinny_rows<bf16_t, kEpiRope>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), out, M, N, K, lda, ldw, ldo, 1, stream, tail);
   else
     LYP_REQUIRE(false, "gemm_rope_kv: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gemm_rope_kv");

@@ -81,6 +81,8 @@ def core() -> ctypes.CDLL:
         lib.lyp_sample_workspace.argtypes = [c_int]
         lib.lyp_sample_workspace.restype = c_longlong
         lib.lyp_norm_threads_override.argtypes = [c_int]
+        lib.lyp_skinny_row_tiles_override.argtypes = [c_int]
+        lib.lyp_skinny_workgroups.argtypes = [c_int, c_int, c_int, c_int]
         lib.lyp_stream_read.argtypes = [c_void_p, c_longlong, c_int, c_void_p, c_void_p]
         _core = lib
     return _core
@@ -316,6 +318,13 @@ def norm_threads_override(threads: int) -> None:
     _check(lib.lyp_norm_threads_override(threads), lib)
 
 
+def skinny_row_tiles_override(row_tiles: int) -> None:
+    """Row tiles (of 16 rows of the weights) per workgroup of the weight-streaming product in steps
+    of more than 16 rows (0: the built-in rule); for measurements."""
+    lib = core()
+    _check(lib.lyp_skinny_row_tiles_override(row_tiles), lib)
+
+
 def rmsnorm_act(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
     _dev(x, weight, out)
     n, H = x.shape
@@ -489,16 +498,15 @@ if LIBRARY_GEMM_MODE not in ("library", "own"):
 LIBRARY_GEMM = LIBRARY_GEMM_MODE != "own"
 LIBRARY_WORKSPACE_BYTES = 76 << 20    # what the library may use beside the operands (stream-K partial tiles)
 LIBRARY_GEMM_MIN_ROWS = 65
-# Between 17 and 64 rows the weight-streaming kernel re-reads the activations
-# once per 16 weight rows, which costs more than the weights themselves when the
-# matrix is large; measured, the library is ahead from this many weights on.
-LIBRARY_GEMM_MID_ROWS = 17
-LIBRARY_GEMM_MID_WEIGHTS = 1 << 24
-# From 49 rows on (a step of 64 in its recorded form) also for the smaller matrices, q/k/v and o of
-# the 1B shape among them: batch 64 at 2,048 tokens 30,200 -> 30,800 tokens/s (2 %); at 48 rows the
-# weight-streaming kernel is still ahead (25,400 against 25,200).
-LIBRARY_GEMM_WIDE_ROWS = 49
-LIBRARY_GEMM_WIDE_WEIGHTS = 1 << 22
+# Between 17 and 64 rows the weight-streaming kernel is one burst of loads per workgroup: every
+# workgroup reads the step's activations over its share of K, asks for all of its weights at once,
+# sums its waves' parts and is done.  That beats the library's tiled kernels while the whole matrix
+# is taken in one round of workgroups on the machine (as many workgroups as compute units, at most),
+# and loses to them when the launch needs several rounds (``_library_product``).  Measured cold on
+# 256 compute units at 64 rows, this kernel against the library (with the passes the library cannot
+# fold in): q/k/v 3072x2048 14.7 against 18.3 us (192 workgroups), o 2048x2048 7.8 against 13.4 (256),
+# down 2048x8192 16.8 against 22.8 (256), gate/up 16384x2048 28.4 against 21.9 (512: the library's).
+LIBRARY_ROUNDS = 1
 # In an engine's warm-up step and in the run before a graph is captured, a library product's algorithm is
 # chosen by measurement among this many of the library's candidates (at the shape's first call).
 # Which candidate wins a timing may differ from process to process, and with it the last bits of
@@ -598,11 +606,30 @@ def library_gemm_solution(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, f
                                             _code(out.dtype), int(for_graph))
 
 
-def _library_product(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+_compute_units: dict = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device (asked once)."""
+    index = torch.cuda.current_device() if device is None or torch.device(device).index is None else torch.device(device).index
+    n = _compute_units.get(index)
+    if n is None:
+        n = _compute_units[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return n
+
+
+def _library_product(M: int, N: int, K: int, dtype: torch.dtype, sliced: bool = False) -> bool:
+    """Whether a bfloat16 product of M rows with a matrix [N, K] goes to the vendor's library.
+    ``sliced``: the caller takes partial sums over slices of K (which gives this package's kernel
+    more workgroups to spread a matrix of few rows over)."""
     if not LIBRARY_GEMM or dtype != torch.bfloat16:
         return False
-    return (M >= LIBRARY_GEMM_MIN_ROWS or (M >= LIBRARY_GEMM_MID_ROWS and N * K >= LIBRARY_GEMM_MID_WEIGHTS)
-            or (M >= LIBRARY_GEMM_WIDE_ROWS and N * K >= LIBRARY_GEMM_WIDE_WEIGHTS))
+    if M >= LIBRARY_GEMM_MIN_ROWS:
+        return True
+    if M <= PENDING_MAX_ROWS:
+        return False
+    workgroups = core().lyp_skinny_workgroups(M, N, K, int(sliced))
+    return workgroups == 0 or workgroups > LIBRARY_ROUNDS * compute_units()
 
 
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
@@ -654,7 +681,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
         if w.dtype != torch.float32:
             raise KernelError(f"linear: weight {w.dtype} against activations {x.dtype}")
         x = cast(x, torch.float32)
-    if may_split and x.shape[0] <= 64 and not _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype):
+    if may_split and x.shape[0] <= 64 and not _library_product(x.shape[0], w.shape[0], w.shape[1], x.dtype, sliced=True):
         _dev(x, w)
         lib = core()
         M, K, N = x.shape[0], x.shape[1], w.shape[0]

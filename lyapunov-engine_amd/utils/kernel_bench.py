@@ -287,8 +287,15 @@ def main(argv=None) -> None:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--out-features", type=int, default=16384)
     ap.add_argument("--may-split", action="store_true", help="linear: allow partial sums over slices of K")
+    ap.add_argument("--own", action="store_true", help="products of 17 to 64 rows in this package's kernel whatever "
+                    "the size of the matrix (the vendor's library otherwise takes the larger ones)")
+    ap.add_argument("--row-tiles", type=int, default=0, help="row tiles per workgroup of that kernel (0: its rule)")
     a = ap.parse_args(argv)
     ops.require_gpu()
+    if a.own:
+        ops.LIBRARY_ROUNDS = 1 << 20
+    if a.row_tiles:
+        ops.skinny_row_tiles_override(a.row_tiles)
     torch.manual_seed(0)
     {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "qkv": qkv, "gate_up": gate_up, "residual": residual,
      "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head}[a.kernel](a)
