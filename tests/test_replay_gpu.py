@@ -478,3 +478,78 @@ def test_long_prompts_do_not_depend_on_their_portions(tmp_path, dtype):
     scale = np.abs(got[4096]).max(axis=1, keepdims=True)
     err = np.abs(got[777] - got[4096]) / np.maximum(scale, 1.0)
     assert err.max() <= TOL_ALONE[dtype]["atol"], f"portions of 777 against 4,096: {err.max(axis=1)}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_recorded_prompt_steps_meet_the_plain_model(model_folders, name, dtype):
+    """A prompt of 100 tokens and one of 17, each alone in its step, through the step that the
+    generating engine records for short prompts (128 and 32 token rows, the rest padding, the unused
+    tile entries beyond any request): the last token's logits against the plain model, on the
+    capture's first run and on replays."""
+    from lyapunov_engine_amd.engine.core import EngineCore
+    from lyapunov_engine_amd.engine.graphs import StepGraphs
+    from trace_util import TOL
+
+    f = folder(model_folders, name, dtype)
+    vocab = TINY[name][0]["vocab_size"]
+    reqs = {"long": random_tokens(100, vocab, seed=301), "short": random_tokens(17, vocab, seed=302)}
+    want = plain_for(model_folders, name, dtype, reqs)
+    core = EngineCore.from_folder(f, dtype=dtype, num_blocks=32, block_size=TINY[name][1]["block_size"], num_state_slots=4)
+    graphs = StepGraphs(core.runner, max_batch=4)
+    tol = TOL[dtype]
+    for turn in range(3):
+        for i, (rid, toks) in enumerate(reqs.items()):
+            sid = 10 * turn + i
+            core.cache.add(sid)
+            core.cache.extend(sid, len(toks))
+            counts = np.asarray([len(toks)], np.int32)
+            assert graphs.prompt_usable(counts)
+            got = graphs.prompt_step_arrays(np.asarray([sid], np.int64), np.zeros(1, np.int32), counts,
+                                            np.asarray(toks, np.int32)).values[0].float().cpu().numpy()
+            ref = np.asarray(want[rid][len(toks) - 1], dtype=np.float64)
+            scale = max(1.0, float(np.abs(ref).max()))
+            err = np.abs(got.astype(np.float64) - ref)
+            assert (err <= tol["atol"] * scale + tol["rtol"] * np.abs(ref)).all(), \
+                f"{rid}, turn {turn}: max error {err.max():.3e} at scale {scale:.3f}"
+            core.cache.commit(sid, len(toks))
+            core.cache.free(sid)              # the next turn's requests get these pages, stale contents and all
+    assert sorted(k[2] for k in graphs.captured) == [32, 128]
+    core.cache.check()
+
+
+def test_bfloat16_error_against_depth(tmp_path):
+    """One layer and four layers as wide as the 1B shape's, to 2,400 tokens in bfloat16 against the
+    plain model: how the rounding error grows with depth.  Measured: the median over the rows goes
+    from 1.0e-2 of the largest logit (one layer) to 1.9e-2 (four; largest row 2.6e-2), about the square root of the
+    depth; the per-row bound of the tiny models' traces holds at four layers, their median bound
+    (set on models of two and three layers) does not, so the deeper model gets twice that."""
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import TOL
+
+    medians = {}
+    for layers in (1, 4):
+        cfg = dict(architectures=["LlamaForCausalLM"], vocab_size=1000, hidden_size=2048, intermediate_size=8192,
+                   num_hidden_layers=layers, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+                   max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+                   rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                     original_max_position_embeddings=1024))
+        d = str(tmp_path / f"deep{layers}")
+        os.makedirs(d)
+        write_random_model(cfg, d, 12, "bfloat16", init_std=0.03, norm_init_std=0.1)
+        reqs = {"a": random_tokens(2400, 1000, seed=4)}
+        t = Trace(reqs)
+        t.step([("a", 1900)], want="last")
+        t.step([("a", 460)], want="last")
+        t.step([("a", 30)])
+        for _ in range(10):
+            t.step([("a", 1)])
+        t.steps[-1]["end"] = ["a"]
+        t.live.clear()
+        rows = sorted(pos for rs in t.rows.values() for _, pos in rs)
+        tol = dict(TOL["bfloat16"], median=TOL["bfloat16"]["median"] * (2 if layers > 3 else 1))
+        rel = compare(t, replay(d, "bfloat16", t), {"a": plain_logits_at(d, reqs["a"], rows)}, "bfloat16",
+                      f"{layers} wide layers", tol=tol)
+        medians[layers] = float(np.median(rel))
+        print(f"{layers} wide layer(s), bfloat16: median {np.median(rel):.4f}, largest {max(rel):.4f} of the largest logit")
+    assert medians[4] <= 3.0 * medians[1], f"the error grew faster than depth accounts for: {medians}"
