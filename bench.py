@@ -147,7 +147,10 @@ def measure_prefill(engine, cfg, tokens, repeats=5):
 def measure_mixed(engine, cfg, requests=64, seed=0):
     """BASELINE.json configs[3]'s workload: a continuous batch of `requests` requests with prompts
     of 128 to 4096 random tokens and 128 to 512 output tokens each, prompts taken in portions of at
-    most 512 tokens.  Returns (seconds, prompt tokens, generated tokens, steps)."""
+    most 512 tokens.  Returns (seconds, prompt tokens, generated tokens, steps, latencies): per
+    request the time from the start of the run (all requests are added at once) to its first token,
+    and the mean time between its tokens after that, as the reference's serving bench reports them
+    for its batches (benchmarks/bench_serving.py:54-77: TTFT and average inter-token latency)."""
     import random
 
     import torch
@@ -170,11 +173,27 @@ def measure_mixed(engine, cfg, requests=64, seed=0):
             mixed.add_request(p_, sp)
         torch.cuda.synchronize()
         t0, steps = time.perf_counter(), 0
+        first, last, count = {}, {}, {}
         while mixed.has_unfinished_requests():
-            mixed.step()
+            outs = mixed.step()
+            now = time.perf_counter() - t0     # the step's tokens have reached the host
             steps += 1
+            for o in outs:
+                if o.output_tokens and o.request_id not in first:
+                    first[o.request_id] = now
+                if o.finished:
+                    last[o.request_id], count[o.request_id] = now, len(o.output_tokens)
         torch.cuda.synchronize()
-    return time.perf_counter() - t0, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps
+    secs = time.perf_counter() - t0
+    ttft = sorted(first.values())
+    itl = sorted((last[r] - first[r]) / max(count[r] - 1, 1) for r in last)
+
+    def spread(xs):
+        return {"mean": round(sum(xs) / len(xs) * 1e3, 3), "p50": round(xs[len(xs) // 2] * 1e3, 3),
+                "p99": round(xs[min(len(xs) - 1, int(0.99 * len(xs)))] * 1e3, 3), "max": round(xs[-1] * 1e3, 3)}
+
+    latencies = {"time_to_first_token_ms": spread(ttft), "inter_token_ms": spread(itl)}
+    return secs, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps, latencies
 
 
 # Largest bf16-against-fp32 logit difference over the largest logit that passes.  Measured on the 1B
@@ -265,7 +284,7 @@ def main():
                                shape=shape)
 
     if args.workload == "mixed":
-        secs, n_prompt, n_gen, steps = measure_mixed(engine, cfg)
+        secs, n_prompt, n_gen, steps, latencies = measure_mixed(engine, cfg)
         print(json.dumps({
             "metric": "generated tok/s of a mixed continuous batch", "value": round(n_gen / secs, 1), "unit": "tok/s",
             "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": round(secs / steps * 1e3, 4),
@@ -275,7 +294,7 @@ def main():
                        "full_layers": full_layers, "requests": 64, "prompt_tokens": n_prompt,
                        "generated_tokens": n_gen, "prompt_portion": 512, "step_token_budget": 2048,
                        "kv_block_size": block_size, "parallelism": "single-gpu", "graphs": True},
-            "total_tokens_per_s": round((n_prompt + n_gen) / secs, 1)}))
+            "total_tokens_per_s": round((n_prompt + n_gen) / secs, 1), **latencies}))
         return 0
 
     lookahead = bool(engine.config.lookahead)

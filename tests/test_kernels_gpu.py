@@ -520,6 +520,50 @@ def test_attention_prefill(ops, dtype, case, split, parts):
     torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 2e-2))
 
 
+@pytest.mark.parametrize("variant", ["two sets of waves", "keys in 4 runs", "paired tiles"])
+def test_bfloat16_prefill_kernel_rounds_like_one_rounding(ops, variant):
+    """The kernel that exists in bfloat16 only (16x16x32 products, probabilities rounded to
+    bfloat16 before they meet the values) in each of its forms, on inputs that are bfloat16
+    values already, against the formula in float64: what is measured is the kernel's own rounding,
+    and it stays inside 1e-2 (the probabilities' 8 bits, averaged over the keys)."""
+    nh, nkv, hd, bs = 32, 8, 64, 16
+    seqs = [(2065, 2065)] if variant == "paired tiles" else [(700, 200), (300, 64)]
+    s = paged_setup(seqs, nh, nkv, hd, bs, torch.bfloat16, seed=17)
+    tile_seq, tile_q0 = [], []
+    for b, (_, ql) in enumerate(seqs):
+        for q0 in range(0, ql, 64):
+            tile_seq.append(b), tile_q0.append(q0)
+    out = torch.full((s["q"].shape[0], nh * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    work = dict(split=variant == "two sets of waves")
+    if variant == "keys in 4 runs":
+        n = len(tile_seq) * 64 * nh * 4
+        work.update(parts=4, part_o=torch.full((n * hd,), float("nan"), device=DEV),
+                    part_ml=torch.full((n * 2,), float("nan"), device=DEV))
+    ops.attn_prefill(s["q"].to(DEV), out, s["kpool"].to(DEV), s["vpool"].to(DEV), s["bt"].to(DEV),
+                     s["q_start"].to(DEV), s["ctx_len"].to(DEV), torch.tensor(tile_seq, dtype=torch.int32, device=DEV),
+                     torch.tensor(tile_q0, dtype=torch.int32, device=DEV), len(tile_seq), num_heads=nh,
+                     num_kv_heads=nkv, head_dim=hd, pair=variant == "paired tiles", **work)
+    torch.testing.assert_close(out.cpu().double(), plain_attention(s, seqs, 0), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 3072, 2048), (33, 2048, 2048), (64, 2048, 8192), (48, 3072, 2048)])
+def test_bfloat16_few_rows_product_rounds_once(ops, M, N, K):
+    """The weight-streaming product's 16x16x32 path (one and two row tiles per workgroup, partial
+    sums over slices of K) on bfloat16 inputs against float64: float sums, one rounding at the end."""
+    a, w = rnd(M, K, dtype=torch.bfloat16, seed=31), rnd(N, K, dtype=torch.bfloat16, scale=0.05, seed=32)
+    want = a.double() @ w.double().T
+    scale = float(want.abs().max())
+    y = ops.linear(a.to(DEV), w.to(DEV))
+    assert float((y.cpu().double() - want).abs().max()) <= 2.0 ** -8 * scale        # the one rounding to bfloat16
+    parts = ops.linear(a.to(DEV), w.to(DEV), may_split=True)
+    total = ops.sum_parts(parts, torch.float32)
+    # float partial sums where this package's kernel took the product in slices; one rounding to
+    # bfloat16 where the launch would have needed several rounds of workgroups and the library took it
+    limit = 1e-5 if parts.dim() == 3 else 2.0 ** -8
+    assert float((total.cpu().double() - want).abs().max()) <= limit * scale
+    assert parts.dim() == 3 or M == 48
+
+
 def test_attention_prefill_plan(ops):
     plan = lambda tiles, keys, dt=torch.bfloat16, bs=16: ops.attn_prefill_plan(tiles, keys, 32, 8, 64, dt, bs)
     assert plan(32, 2048) == 1                 # a whole prompt: enough workgroups as it is

@@ -789,3 +789,137 @@ def test_another_embedding_and_another_output_head(tmp_path, dtype):
         EMBEDDINGS.unregister("toy_scaled_lookup")
         HEADS.unregister("toy_capped_head")
         BLOCKS.unregister("toy_sandwich")
+
+
+# --------------------------------- a fifth toy: a mixer with a page layout of its own
+TOY5 = dict(architectures=["ToyLatentForCausalLM"], vocab_size=110, hidden_size=64, intermediate_size=96, latent=24,
+            num_heads=2, num_kv_heads=2, head_dim=16, max_position=128, eps=1e-5, theta=10000.0)
+
+
+def register_toy5():
+    """A mixer that keeps one vector per token in pages (no separate values, kept in 32-bit whatever
+    the engine's precision), in a layout that is its own: what a page holds is said by the mixer's
+    ``PagedSpec`` and nowhere else."""
+    from lyapunov_engine_amd.config import MIXERS, LayerSpec, ModelSpec, PartSpec, default_schedule, register_architecture
+    from lyapunov_engine_amd.parts import SLOT, Mixer, PagedSpec, PageTensor, WeightSource, WeightSpec
+
+    class LatentAttention(Mixer):
+        """c_t = W_c x_t is all a token leaves behind; token t reads softmax_s<=t(q_t . c_s / sqrt(L)) c_s."""
+
+        graph_safe = False   # walks the host copy of the batch layout
+
+        def __init__(self, hidden_size, latent):
+            self.hidden_size, self.latent = hidden_size, latent
+            self.q_proj = self.c_proj = self.o_proj = None
+
+        def weight_specs(self):
+            return [WeightSpec("q_proj", (WeightSource("q_proj.weight", (self.latent, self.hidden_size)),)),
+                    WeightSpec("c_proj", (WeightSource("c_proj.weight", (self.latent, self.hidden_size)),)),
+                    WeightSpec("o_proj", (WeightSource("o_proj.weight", (self.hidden_size, self.latent)),))]
+
+        def cache_spec(self):
+            return PagedSpec((PageTensor("latent", (SLOT, self.latent), torch.float32),))
+
+        def forward(self, ctx, x, cache):
+            assert set(cache.pages) == {"latent"} and cache.k is None and cache.v is None
+            pool = cache.pages["latent"]                      # [pages, page size, latent], float32
+            assert pool.dtype == torch.float32 and pool.shape[1:] == (cache.group.page_size, self.latent)
+            flat = pool.view(-1, self.latent)
+            xf = x.float()
+            q, c = xf @ self.q_proj.float().T, xf @ self.c_proj.float().T
+            flat[cache.group.slot_mapping.long()] = c
+            out = torch.empty_like(q)
+            ps = cache.group.page_size
+            for b in range(ctx.B):
+                lo, hi, n = ctx.q_start_host[b], ctx.q_start_host[b + 1], ctx.ctx_len_host[b]
+                pages = cache.group.block_tables[b, :-(-n // ps)].long()
+                slots = (pages[:, None] * ps + torch.arange(ps, device=x.device)[None, :]).reshape(-1)[:n]
+                keys = flat[slots]                                            # [n, latent]
+                scores = q[lo:hi] @ keys.T / self.latent ** 0.5
+                pos = torch.arange(n - (hi - lo), n, device=x.device)
+                scores = scores.masked_fill(torch.arange(n, device=x.device)[None, :] > pos[:, None], float("-inf"))
+                out[lo:hi] = torch.softmax(scores, dim=-1) @ keys
+            return (out @ self.o_proj.float().T).to(ctx.dtype)
+
+    MIXERS.register("toy_latent_attention", LatentAttention, replace=True)
+
+    def to_spec(cfg: ToyConfig) -> ModelSpec:
+        c = dict(cfg.raw)
+        H = c["hidden_size"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": c["eps"]})
+        ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": c["intermediate_size"]})
+        rope = PartSpec("rope", {"dim": c["head_dim"], "theta": c["theta"], "max_position": c["max_position"]})
+        attn = PartSpec("paged_attention", dict(hidden_size=H, num_heads=c["num_heads"], num_kv_heads=c["num_kv_heads"],
+                                                head_dim=c["head_dim"], position=rope))
+        latent = PartSpec("toy_latent_attention", {"hidden_size": H, "latent": c["latent"]})
+        layers = (LayerSpec("prenorm", latent, ffn, norm, norm, HF_LAYER_NAMES),
+                  LayerSpec("prenorm", attn, ffn, norm, norm, HF_LAYER_NAMES))
+        return ModelSpec(vocab_size=c["vocab_size"], hidden_size=H, layers=layers, schedule=default_schedule(2),
+                         final_norm=norm, tie_word_embeddings=True, max_position=c["max_position"], **HF_PREFIXES)
+
+    register_architecture("ToyLatentForCausalLM", ToyConfig, to_spec, replace=True)
+
+
+def toy5_plain(folder, tokens):
+    from safetensors.torch import load_file
+
+    c = json.load(open(os.path.join(folder, "config.json")))
+    w = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    S = len(tokens)
+    pos = torch.arange(S)
+    h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    # layer 0: the latent mixer
+    p = "model.layers.0."
+    x = P.rms_norm(h, w[p + "input_layernorm.weight"], c["eps"])
+    q, lat = x @ w[p + "self_attn.q_proj.weight"].T, x @ w[p + "self_attn.c_proj.weight"].T
+    scores = (q @ lat.T / c["latent"] ** 0.5).masked_fill(pos[None, :] > pos[:, None], float("-inf"))
+    h = h + (torch.softmax(scores, dim=-1) @ lat) @ w[p + "self_attn.o_proj.weight"].T
+    x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["eps"])
+    h = h + P.mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    # layer 1: the package's attention
+    raw = dict(num_attention_heads=c["num_heads"], num_key_value_heads=c["num_kv_heads"], head_dim=c["head_dim"],
+               rms_norm_eps=c["eps"])
+    inv = P.rope_inv_freq(c["head_dim"], c["theta"])
+    h = P.decoder_layer(h, pos, w, 1, raw, inv)
+    return P.rms_norm(h, w["model.norm.weight"], c["eps"]) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_with_a_page_layout_of_its_own(tmp_path, dtype):
+    """The pages' layout belongs to the mixer: a mixer registered from here keeps one 32-bit vector
+    per token (no values), gets a pool of exactly that shape and type beside the attention layer's
+    key and value pools, and the cache manager, the step function and the replay run it, pages
+    given back and used again, without a change to the package."""
+    from lyapunov_engine_amd.config import ARCHITECTURES, MIXERS
+    from lyapunov_engine_amd.engine.core import EngineCore
+    from lyapunov_engine_amd.weights import write_random_model
+    from trace_util import compare
+
+    register_toy5()
+    try:
+        folder = str(tmp_path / "toy5")
+        write_random_model(dict(TOY5), folder, seed=21, dtype=dtype, init_std=0.15, norm_init_std=0.1)
+        core = EngineCore.from_folder(folder, dtype=dtype, num_blocks=8, block_size=4, num_state_slots=2)
+        layout = core.model.cache_layout()
+        assert len(layout.groups) == 2 and [t.name for t in layout.groups[0].spec.tensors] == ["latent"]
+        assert [t.name for t in layout.groups[1].spec.tensors] == ["k", "v"]
+        assert {n: (tuple(t.shape), t.dtype) for n, t in core.pools.paged[0].items()} == \
+            {"latent": ((1, 8, 4, TOY5["latent"]), torch.float32)}
+        assert core.pools.paged[1]["v"].shape == (1, 8, TOY5["num_kv_heads"], TOY5["head_dim"], 4)
+        del core
+        reqs = {"x": random_tokens(50, 110, seed=22), "y": random_tokens(19, 110, seed=23), "z": random_tokens(30, 110, seed=24)}
+        want = {k: toy5_plain(folder, v) for k, v in reqs.items()}
+        whole = Trace(reqs)
+        for rid in reqs:
+            whole.step([(rid, len(reqs[rid]))], end=[rid])
+        compare(whole, replay(folder, dtype, whole), want, dtype, "latent whole")
+        cut = Trace(reqs)
+        cut.step([("x", 9), ("y", 19)], end=["y"])
+        cut.step([("x", 3), ("z", 17)])
+        for _ in range(8):
+            cut.step([("x", 1), ("z", 1)])
+        cut.step([("x", 30), ("z", 5)], end=["x", "z"])
+        compare(cut, replay(folder, dtype, cut), want, dtype, "latent cut")
+    finally:
+        ARCHITECTURES.unregister("ToyLatentForCausalLM")
+        MIXERS.unregister("toy_latent_attention")
