@@ -1178,29 +1178,72 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
     int most_block_keys) {
   const int head = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
   const int seq = dec_seqs ? dec_seqs[slot] : slot;
+  const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
+  // The kernel is a chain of trips to memory and little else, so everything that can be asked for
+  // at once is: the request's length and place, and the first kFirst partitions' maxima, sums and
+  // outputs whether or not the request has that many (a partition it lacks holds whatever the
+  // workspace held; it is dropped once the length is known).  More partitions than that are
+  // walked afterwards.
+  constexpr int kFirst = 8;
   const int ctx = ctx_len[seq];
+  const int tok = q_start[seq];
+  constexpr int kPerLane = HD / kWave > 0 ? HD / kWave : 1;   // head dimensions a lane owns (d = lane + 64 k)
+  float2 ml_first[kFirst];
+  float o_first[kPerLane][kFirst];
+#pragma unroll
+  for (int p = 0; p < kFirst; ++p) {
+    const int pc = min(p, max_parts - 1);
+    ml_first[p] = ml[pc];
+#pragma unroll
+    for (int k = 0; k < kPerLane; ++k) {
+      const int d = lane + kWave * k;
+      o_first[k][p] = d < HD ? part_o[(base + pc) * HD + d] : 0.f;
+    }
+  }
   const int block_keys = kDecodeWaves * decode_keys_per_wave(ctx, most_block_keys / kDecodeWaves);
   const int lo = window > 0 ? max(0, ctx - window) : 0;
   const int p_lo = lo / block_keys;
   const int p_hi = (ctx + block_keys - 1) / block_keys;
-  const size_t base = (static_cast<size_t>(slot) * nh + head) * max_parts;
-  const float2* ml = reinterpret_cast<const float2*>(part_ml) + base;
 
   float m = LYP_NEG_INF;
-  for (int p = p_lo + lane; p < p_hi; p += kWave) m = fmaxf(m, ml[p].x);
+#pragma unroll
+  for (int p = 0; p < kFirst; ++p)
+    if (p >= p_lo && p < p_hi) m = fmaxf(m, ml_first[p].x);
+  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave) m = fmaxf(m, ml[p].x);
   m = wave_max(m);
   const float m_safe = m == LYP_NEG_INF ? 0.f : m;
+  // every lane adds up the same terms in the same order: partitions 0 .. kFirst - 1, then the rest by lanes
   float l = 0.f;
-  for (int p = p_lo + lane; p < p_hi; p += kWave) l += fast_exp2(ml[p].x - m_safe) * ml[p].y;
-  l = wave_sum(l);
+  float w_first[kFirst];
+#pragma unroll
+  for (int p = 0; p < kFirst; ++p) {
+    w_first[p] = (p >= p_lo && p < p_hi) ? fast_exp2(ml_first[p].x - m_safe) : 0.f;
+    l += (p >= p_lo && p < p_hi) ? w_first[p] * ml_first[p].y : 0.f;
+  }
+  float l_rest = 0.f;
+  for (int p = max(p_lo, kFirst) + lane; p < p_hi; p += kWave) l_rest += fast_exp2(ml[p].x - m_safe) * ml[p].y;
+  l += wave_sum(l_rest);
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 
-  T* orow = out + static_cast<size_t>(q_start[seq]) * out_stride + static_cast<size_t>(head) * HD;
-  for (int d = lane; d < HD; d += kWave) {
+  T* orow = out + static_cast<size_t>(tok) * out_stride + static_cast<size_t>(head) * HD;
+#pragma unroll
+  for (int k = 0; k < kPerLane; ++k) {
+    const int d = lane + kWave * k;
+    if (d >= HD) continue;
     float acc = 0.f;
+#pragma unroll
+    for (int p = 0; p < kFirst; ++p) acc += (p >= p_lo && p < p_hi) ? w_first[p] * o_first[k][p] : 0.f;
 #pragma unroll 4
-    for (int p = p_lo; p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+    for (int p = max(p_lo, kFirst); p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
     orow[d] = from_f32<T>(acc * inv);
+  }
+  if constexpr (HD < kWave || HD % kWave != 0) {   // head sizes that are no multiple of 64: the dimensions past the lanes' share
+    for (int d = lane + kWave * kPerLane; d < HD; d += kWave) {
+      float acc = 0.f;
+      for (int p = p_lo; p < p_hi; ++p) acc += fast_exp2(ml[p].x - m_safe) * part_o[(base + p) * HD + d];
+      orow[d] = from_f32<T>(acc * inv);
+    }
   }
 }
 

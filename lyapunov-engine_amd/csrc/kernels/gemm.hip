@@ -287,6 +287,29 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     }
   }
 
+  // kEpiRope: the position and the cache slot of the token that the thread's first element belongs
+  // to are asked for now, and the cosine and sine after the products, while the waves' sums meet in LDS;
+  // the epilogue would otherwise walk from one to the next, a trip to memory each.
+  int pos_first = 0, slot_first = -1;
+  float cos_first = 1.f, sin_first = 0.f;
+  [[maybe_unused]] auto rope_first = [&](int e, int& m, int& fi, bool& rotated) {
+    const int l = (e % 256) / 4, row = 4 * (l / 16) + e % 4;
+    const int tile_n0 = n0 + 16 * (RT == 1 ? 0 : e / 256 / MB);
+    const int head_ix = tile_n0 / tail.hd, blk = (tile_n0 % tail.hd) / 16;
+    m = (RT == 1 ? e / 256 : (e / 256) % MB) * 16 + l % 16;
+    rotated = head_ix < tail.nh + (tail.has_kv ? tail.nkv : 0) && blk < tail.rot / 16 && row < 8;
+    fi = 8 * blk + row;
+    return e < NT * 256 && m < M && tile_n0 < N;
+  };
+  if constexpr (EPI == kEpiRope) {
+    int m, fi;
+    bool rotated;
+    if (rope_first(threadIdx.x, m, fi, rotated)) {
+      pos_first = tail.positions[m];
+      if (tail.has_kv) slot_first = tail.slots[m];
+    }
+  }
+
   // of 64 values of K, fragment f of lane group j holds values 4 E f + E j .. + E - 1 (E = MM::kElems): the
   // four lane groups of one load instruction read 4 E neighbouring values of a row, whole 64-byte pieces
   const int second = PAIRED ? (r / 8) * 64 : 0;  // the tile's upper half: the chunk's second 64 values
@@ -378,6 +401,15 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   }
   for (; c < c_end; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
 
+  if constexpr (EPI == kEpiRope) {
+    int m, fi;
+    bool rotated;
+    if (rope_first(threadIdx.x, m, fi, rotated) && rotated) {
+      const float* cs = tail.cos_sin + static_cast<size_t>(pos_first) * tail.rot;
+      cos_first = cs[fi];
+      sin_first = cs[tail.rot / 2 + fi];
+    }
+  }
   // acc[rt * MB + b][i]: output feature n0 + 16 rt + 4 j + i, token 16 b + r
   float* mine = red + (static_cast<size_t>(wave) * NT * 64 + lane) * 4;
 #pragma unroll
@@ -419,10 +451,14 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
       // as two kernels would do it: the product rounded to the activations' type, then rotated
       T y0 = from_f32<T>(total(e)), y1 = y0;
       int f0 = 16 * blk + row, f1 = f0;
+      const bool first = e == static_cast<int>(threadIdx.x);
       if (rotated) {
         const int half = tail.rot / 2, fi = 8 * blk + row;
-        const float* cs = tail.cos_sin + static_cast<size_t>(tail.positions[m]) * tail.rot;
-        const float c = cs[fi], sn = cs[half + fi];
+        float c = cos_first, sn = sin_first;
+        if (!first) {
+          const float* cs = tail.cos_sin + static_cast<size_t>(tail.positions[m]) * tail.rot;
+          c = cs[fi], sn = cs[half + fi];
+        }
         const float x0 = to_f32(y0), x1 = to_f32(from_f32<T>(total(e + 128)));  // the same token, row + 8
         float r0, r1;
         rotate_pair(x0, x1, c, sn, r0, r1);
@@ -437,7 +473,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
         if (rotated) orow[f1] = y1;
         continue;
       }
-      const int slot = tail.slots[m];
+      const int slot = first ? slot_first : tail.slots[m];
       if (slot < 0) continue;
       const size_t page = slot / tail.bs, off = slot % tail.bs;
       if (is_k) {
