@@ -196,10 +196,16 @@ def measure_mixed(engine, cfg, requests=64, seed=0):
     return secs, sum(len(p_) for p_ in prompts), sum(sp.max_tokens for sp in params), steps, latencies
 
 
-# Largest bf16-against-fp32 logit difference over the largest logit that passes.  Measured on the 1B
-# shape at context 8,192: 0.8 % through 2 layers, 1.9 % through all 16 (rounding adds up roughly with
-# the square root of the depth); twice the measured value is allowed.
-CHECK_LIMIT = 0.04
+# Largest bf16-against-fp32 logit difference over the largest logit that passes, per layer of the
+# model.  Measured at context 8,192 with random weights (whose logits are nearly flat, so that the
+# largest logit is a small yardstick): 1B shape 0.8 % through 2 layers and 1.9 % through all 16, 3B
+# shape 3.8 % through 28, 8B shape 5.1 % through 32; at context 32,768 the 1B shape shows 1.8 %.
+# Allowed: a quarter of a per cent per layer, about one and a half times the largest of these.
+CHECK_LIMIT_PER_LAYER = 0.0025
+
+
+def check_limit(layers):
+    return max(0.02, CHECK_LIMIT_PER_LAYER * layers)
 
 
 def check_logits(shape=MODEL, layers=None, context=8192, portion=2048):
@@ -322,8 +328,9 @@ def main():
         check = {"what": f"bf16 against fp32 logits, same bf16-rounded weights, {cfg.num_hidden_layers} layers, prompt of {args.context - 1} "
                          f"tokens in portions of 2048 (eager), then one decoded token at context {args.context} "
                          f"through the recorded graph; largest difference over largest logit",
-                 "prompt_last": round(rel[0], 5), "decoded_through_graph": round(rel[1], 5), "limit": CHECK_LIMIT,
-                 "best_token_same_or_tied": all(same), "ok": max(rel) <= CHECK_LIMIT and all(same)}
+                 "prompt_last": round(rel[0], 5), "decoded_through_graph": round(rel[1], 5),
+                 "limit": check_limit(cfg.num_hidden_layers),
+                 "best_token_same_or_tied": all(same), "ok": max(rel) <= check_limit(cfg.num_hidden_layers) and all(same)}
 
     peak = MFMA_PEAK[args.dtype]
     line = {
@@ -342,7 +349,7 @@ def main():
             "parallelism": "single-gpu", "graphs": True, "lookahead": lookahead,
             "logits_check": "skipped" if check is None else
                             f"bf16 vs fp32 engine, {cfg.num_hidden_layers} layers, context {args.context}: "
-                            f"{max(rel):.4f} of the largest logit (limit {CHECK_LIMIT}), {'ok' if check['ok'] else 'FAILED'}",
+                            f"{max(rel):.4f} of the largest logit (limit {check['limit']}), {'ok' if check['ok'] else 'FAILED'}",
         },
         "prefill": {"value": round(2048 / prefill_s, 1), "tokens": 2048, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops(cfg, 2048) / prefill_s / peak, 4)},
@@ -354,7 +361,7 @@ def main():
     print(json.dumps(line))
     if check is not None and not check["ok"]:
         print(f"bench.py: bfloat16 logits at context {args.context} are off by {max(rel):.4f} of the largest logit "
-              f"(limit {CHECK_LIMIT}), or the two engines' best tokens differ beyond a tie", file=sys.stderr)
+              f"(limit {check['limit']}), or the two engines' best tokens differ beyond a tie", file=sys.stderr)
         return 1
     return 0
 

@@ -833,6 +833,9 @@ extern "C" int lyp_skinny_workgroups(int M, int N, int K, int with_slices) {
   return ((N + rows - 1) / rows) * slices;
 }
 
+// Slices of K that lyp_gemm_nt_parts would cut this matrix into (1: none).
+extern "C" int lyp_skinny_slices(int N, int K) { return K % 64 == 0 ? skinny_slices(N, K) : 1; }
+
 // How many partial sums lyp_gemm_nt_parts would produce for this product; 0 if
 // it does not apply (then use lyp_gemm_nt).
 extern "C" int lyp_gemm_parts_hint(const void* A, const void* W, int dtype, int M, int N, int K, int lda, int ldw) {

@@ -83,6 +83,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_norm_threads_override.argtypes = [c_int]
         lib.lyp_skinny_row_tiles_override.argtypes = [c_int]
         lib.lyp_skinny_workgroups.argtypes = [c_int, c_int, c_int, c_int]
+        lib.lyp_skinny_slices.argtypes = [c_int, c_int]
         lib.lyp_stream_read.argtypes = [c_void_p, c_longlong, c_int, c_void_p, c_void_p]
         _core = lib
     return _core
@@ -506,7 +507,19 @@ LIBRARY_GEMM_MIN_ROWS = 65
 # 256 compute units at 64 rows, this kernel against the library (with the passes the library cannot
 # fold in): q/k/v 3072x2048 14.7 against 18.3 us (192 workgroups), o 2048x2048 7.8 against 13.4 (256),
 # down 2048x8192 16.8 against 22.8 (256), gate/up 16384x2048 28.4 against 21.9 (512: the library's).
-LIBRARY_ROUNDS = 1
+# The burst also has to stay small: a workgroup reads its rows of the matrix and the step's
+# activations over all of its share of K; past about 64 KiB of weights or 192 KiB of activations per
+# workgroup the library's tiles are ahead again.  Whole decode steps at context 2,304, this package's
+# kernel for every product that fits one round against the library for every product of 17 to 64 rows:
+# 1B shape, batch 24 / 32 / 48 / 64: 15,510 / 19,430 / 24,630 / 29,280 against 14,820 / 18,870 / 24,250 /
+# 29,680 tokens a second (64 rows of 2,048 values are 256 KiB of activations; the gains are the q/k/v and
+# o products'); 8B shape, whose products of one round have 128 KiB and more of weights per workgroup:
+# 4,030 / 4,930 / 6,040 / 7,410 against 4,130 / 5,090 / 6,180 / 7,760.
+# (LYAPUNOV_AMD_LIBRARY_ROUNDS sets the number of rounds this package's kernel may take: 0 sends every
+# product of 17 to 64 rows to the library, a large number none.)
+LIBRARY_ROUNDS = float(os.environ.get("LYAPUNOV_AMD_LIBRARY_ROUNDS", "1"))
+LIBRARY_ACTIVATION_BYTES = 192 << 10
+LIBRARY_WEIGHT_BYTES = 64 << 10
 # In an engine's warm-up step and in the run before a graph is captured, a library product's algorithm is
 # chosen by measurement among this many of the library's candidates (at the shape's first call).
 # Which candidate wins a timing may differ from process to process, and with it the last bits of
@@ -628,8 +641,15 @@ def _library_product(M: int, N: int, K: int, dtype: torch.dtype, sliced: bool = 
         return True
     if M <= PENDING_MAX_ROWS:
         return False
-    workgroups = core().lyp_skinny_workgroups(M, N, K, int(sliced))
-    return workgroups == 0 or workgroups > LIBRARY_ROUNDS * compute_units()
+    lib = core()
+    workgroups = lib.lyp_skinny_workgroups(M, N, K, int(sliced))
+    if workgroups == 0 or workgroups > LIBRARY_ROUNDS * compute_units():
+        return True
+    slices = lib.lyp_skinny_slices(N, K) if sliced else 1
+    k_per_workgroup = K // slices
+    rows_per_workgroup = -(-N // (workgroups // slices))
+    return (-(-M // 16) * 16 * k_per_workgroup * 2 > LIBRARY_ACTIVATION_BYTES
+            or rows_per_workgroup * k_per_workgroup * 2 > LIBRARY_WEIGHT_BYTES)
 
 
 def gemm_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:

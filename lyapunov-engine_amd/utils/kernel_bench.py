@@ -8,6 +8,7 @@
     python -m lyapunov_engine_amd.utils.kernel_bench head --rows 8
     python -m lyapunov_engine_amd.utils.kernel_bench stream --megabytes 64
     python -m lyapunov_engine_amd.utils.kernel_bench rmsnorm --rows 2048 --in-features 4100 --threads 256
+    python -m lyapunov_engine_amd.utils.kernel_bench floor
 
 Prints the time per call and what it means in TFLOP/s or TB/s.  Small enough to
 run under ``rocprofv3 --pmc ...`` when a kernel's counters are wanted; the
@@ -242,6 +243,24 @@ def stream(a) -> None:
                   f"again and again {warm * 1e6:.1f} us {src.numel() / warm / 1e12:.2f} TB/s")
 
 
+def floor(a) -> None:
+    """What a kernel costs that does next to nothing: 64 launches of the reading kernel over 64 KiB,
+    recorded in one graph and replayed, with 1 to 1,024 workgroups; time per launch, i.e. the cost of
+    a dependent step in a recorded decode step whatever it computes."""
+    dev = a.device
+    src = torch.empty(64 << 10, dtype=torch.uint8, device=dev).random_()
+    for blocks in ([a.blocks] if a.blocks else [1, 8, 256, 1024]):
+        sink = torch.empty(blocks * 4, dtype=torch.int32, device=dev)
+        ops.stream_read(src, sink, blocks)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(64):
+                ops.stream_read(src, sink, blocks)
+        t = _time(graph.replay, a.repeat) / 64
+        print(f"floor: a kernel of {blocks} workgroups that reads 64 KiB, one of 64 in a recorded graph: {t * 1e6:.2f} us")
+
+
 def rmsnorm(a) -> None:
     """The norm kernels on ``rows`` rows of ``in-features`` values; ``--threads`` sets the
     workgroup size of the two-pass kernels (rows of odd lengths) instead of the built-in rule."""
@@ -262,7 +281,7 @@ def rmsnorm(a) -> None:
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(prog="kernel_bench", description=__doc__.splitlines()[0])
     ap.add_argument("kernel", choices=["attn_prefill", "attn_decode", "linear", "qkv", "gate_up", "residual", "sample", "stream",
-                                       "rmsnorm", "head"])
+                                       "rmsnorm", "head", "floor"])
     ap.add_argument("--cold", action="store_true", help="linear, qkv, gate_up, residual, head: the weights come from memory "
                     "every time (copies of the matrix in turn), not from the memory-side cache")
     ap.add_argument("--megabytes", type=int, default=0, help="stream: size of the buffer (0: a range of sizes)")
@@ -298,7 +317,7 @@ def main(argv=None) -> None:
         ops.skinny_row_tiles_override(a.row_tiles)
     torch.manual_seed(0)
     {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "qkv": qkv, "gate_up": gate_up, "residual": residual,
-     "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head}[a.kernel](a)
+     "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head, "floor": floor}[a.kernel](a)
 
 
 if __name__ == "__main__":

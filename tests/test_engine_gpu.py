@@ -235,9 +235,9 @@ def test_graph_of_many_rows_with_library_products_equals_eager(tmp_path):
     write_random_model(cfg, folder, 3, "bfloat16", init_std=0.02)
     n = 40
     # the gate/up product is the library's at this many rows (several rounds of this package's workgroups);
-    # the down product, one round when its inner dimension is cut into slices, is this package's
+    # the o product, one small round when its inner dimension is cut into slices, is this package's
     assert ops._library_product(n, 2 * 8192, 2048, torch.bfloat16)
-    assert not ops._library_product(n, 2048, 8192, torch.bfloat16, sliced=True)
+    assert not ops._library_product(n, 2048, 2048, torch.bfloat16, sliced=True)   # the o product: one small round
     core = EngineCore.from_folder(folder, dtype="bfloat16", num_blocks=n * 4 + 8, block_size=16, num_state_slots=64)
     graphs = DecodeGraphs(core.runner, max_batch=64)
     lens = [3 + (5 * i) % 17 for i in range(n)]

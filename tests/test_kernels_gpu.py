@@ -546,7 +546,7 @@ def test_bfloat16_prefill_kernel_rounds_like_one_rounding(ops, variant):
     torch.testing.assert_close(out.cpu().double(), plain_attention(s, seqs, 0), rtol=1e-2, atol=1e-2)
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 3072, 2048), (33, 2048, 2048), (64, 2048, 8192), (48, 3072, 2048)])
+@pytest.mark.parametrize("M,N,K", [(8, 3072, 2048), (33, 2048, 2048), (64, 2048, 8192), (48, 3072, 2048), (40, 2048, 1024)])
 def test_bfloat16_few_rows_product_rounds_once(ops, M, N, K):
     """The weight-streaming product's 16x16x32 path (one and two row tiles per workgroup, partial
     sums over slices of K) on bfloat16 inputs against float64: float sums, one rounding at the end."""
@@ -561,7 +561,7 @@ def test_bfloat16_few_rows_product_rounds_once(ops, M, N, K):
     # bfloat16 where the launch would have needed several rounds of workgroups and the library took it
     limit = 1e-5 if parts.dim() == 3 else 2.0 ** -8
     assert float((total.cpu().double() - want).abs().max()) <= limit * scale
-    assert parts.dim() == 3 or M == 48
+    assert parts.dim() == 3 or M > 40      # (the larger ones are more than one small round of workgroups)
 
 
 def test_attention_prefill_plan(ops):
