@@ -394,11 +394,12 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
     }
   };
   int c = c_begin;
+  // (a wave whose share is two or three chunks asks for two of them at once rather than one after the
+  // other: the second chunk's loads would otherwise wait for the first chunk's products, a trip to memory more)
   if constexpr (RT == 1) {
     for (; c + 4 <= c_end; c += 4) chunks_at(std::integral_constant<int, 4>{}, c);
-  } else {  // several row tiles' weights in flight: two chunks at a time keep the registers for more waves
-    for (; c + 2 <= c_end; c += 2) chunks_at(std::integral_constant<int, 2>{}, c);
   }
+  for (; c + 2 <= c_end; c += 2) chunks_at(std::integral_constant<int, 2>{}, c);  // (several row tiles: two at a time at most)
   for (; c < c_end; ++c) chunks_at(std::integral_constant<int, 1>{}, c);
 
   if constexpr (EPI == kEpiRope) {
