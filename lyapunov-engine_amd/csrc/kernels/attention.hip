@@ -1249,20 +1249,6 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(
 
 constexpr int kPrefillPartsMost = 16;
 
-// Compute units of the current device (asked once per process).
-static int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n = v;
-    else
-      n = 256;
-  }
-  return n;
-}
-
 static int check_common(const char* name, int nh, int nkv, int bs, int max_blocks, int q_stride,
                         int out_stride, int window) {
   LYP_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: %d query heads over %d key/value heads", name, nh, nkv);

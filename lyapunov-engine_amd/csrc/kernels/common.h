@@ -207,4 +207,19 @@ void set_error(const char* fmt, ...);
 
 enum DType : int { kF32 = 0, kBF16 = 1 };
 
+// Compute units of the current device (asked once per process).
+inline int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
+
 }  // namespace lyp

@@ -529,6 +529,7 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const T* __restrict__
   }
 }
 
+
 // ------------------------------------------------------------ the output head
 // Float logits of few rows (a decode step's) against a matrix of very many rows: C[M, N] = A . W^T
 // with N in the hundred thousands.  The work is one long read of W, and such a read is fastest
@@ -623,6 +624,101 @@ __global__ __launch_bounds__(256) void lm_head_kernel(const T* __restrict__ A, c
       ArgMax a = s_best[0][t / 16][t % 16];
       for (int w = 1; w < kWaves; ++w) a = better(a, s_best[w][t / 16][t % 16]);
       cand[static_cast<size_t>(t) * gridDim.x + blockIdx.x] = a;
+    }
+  }
+}
+
+// The same for at most 16 tokens of bfloat16, as one steady stream.  The tokens' activations are put
+// into LDS once (16 rows of K values, a row's start shifted by 16 bytes against the one before so
+// that the 16 rows a fragment read touches lie in different banks); after that a wave asks global
+// memory for nothing but weights, RING chunks of 64 values ahead, across the end of its 16 rows of W
+// into the next 16 that are its turn.  Loads come back in the order they were asked for, so an
+// activation fetched from global memory between the weights would wait for every weight asked
+// before it; from LDS it does not.  One workgroup per compute unit is enough to keep the memory busy
+// (8 tokens on 128256 x 2048: 256 workgroups 106.5 us, 512 107.0, 1024 111.5, against 115.7 of
+// lm_head_kernel; 16 tokens 114 against 131, one token 100 against 105).
+template <int RING>
+__global__ __launch_bounds__(256) void lm_head_stream_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                             float* __restrict__ C, int M, int N, int K, int lda, int ldw,
+                                                             int ldc, ArgMax* __restrict__ cand) {
+  using MM = Mma16Wide<bf16_t>;
+  constexpr int kWaves = 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char x_lds[];   // [16][2 K + 16] bytes
+  __shared__ ArgMax s_best[kWaves][16];
+  const int row_bytes = 2 * K + 16;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int r = lane % 16, j = lane / 16;
+  const int chunks = K / 64;
+  const int tiles = (N + 15) / 16;
+  const int stride = gridDim.x * kWaves;
+  int tile = static_cast<int>(blockIdx.x) * kWaves + wave;
+  // the first weights are asked for before the activations are staged; a wave without a tile reads the last one's
+  const bf16_t* wp = W + static_cast<size_t>(min(min(tile, tiles - 1) * 16 + r, N - 1)) * ldw + j * 8;
+  bf16x8 wf[RING][2];
+#pragma unroll
+  for (int u = 0; u < RING; ++u)
+#pragma unroll
+    for (int f = 0; f < 2; ++f) wf[u][f] = *reinterpret_cast<const bf16x8*>(wp + min(u, chunks - 1) * 64 + f * 32);
+  for (int p = tid; p < 16 * (K / 8); p += 256) {
+    const int row = p / (K / 8), c16 = p % (K / 8);
+    *reinterpret_cast<bf16x8*>(x_lds + row * row_bytes + c16 * 16) =
+        *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(min(row, M - 1)) * lda + c16 * 8);
+  }
+  __syncthreads();
+  const unsigned char* xl = x_lds + r * row_bytes + j * 16;
+  ArgMax best{LYP_NEG_INF, 0x7fffffff};
+  for (; tile < tiles; tile += stride) {
+    const bf16_t* wn = W + static_cast<size_t>(min(min(tile + stride, tiles - 1) * 16 + r, N - 1)) * ldw + j * 8;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < chunks; c += RING) {
+#pragma unroll
+      for (int u = 0; u < RING; ++u) {
+        if (c + u < chunks) {
+#pragma unroll
+          for (int f = 0; f < 2; ++f) {
+            const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xl + (c + u) * 128 + f * 64);
+            acc = MM::mma(wf[u][f], xf, acc);
+          }
+        }
+        // slot u next holds chunk c + u + RING of this tile, or the next tile's chunk past this one's end
+        const int nc = c + u + RING;
+        const int past = nc - ((chunks + RING - 1) / RING) * RING;   // >= 0: the next tile's chunk `past`
+        const bf16_t* src = past < 0 ? wp + min(nc, chunks - 1) * 64 : wn + min(past, chunks - 1) * 64;
+#pragma unroll
+        for (int f = 0; f < 2; ++f) wf[u][f] = *reinterpret_cast<const bf16x8*>(src + f * 32);
+      }
+    }
+    // acc[i]: row 16 tile + 4 j + i of W (a logit's index), token r
+    const int n = tile * 16 + 4 * j;
+    ArgMax mine{LYP_NEG_INF, 0x7fffffff};
+    if (r < M) {
+      float* crow = C + static_cast<size_t>(r) * ldc + n;
+      if (n + 3 < N && ldc % 4 == 0) {
+        *reinterpret_cast<f32x4*>(crow) = acc;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) crow[i] = acc[i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < N) mine = better(mine, ArgMax{acc[i], n + i});
+    }
+    if (cand) {
+#pragma unroll
+      for (int off = 16; off < kWave; off *= 2) mine = better(mine, ArgMax{__shfl_xor(mine.v, off, kWave), __shfl_xor(mine.i, off, kWave)});
+      best = better(best, mine);
+    }
+    wp = wn;
+  }
+  if (cand) {
+    if (j == 0) s_best[wave][r] = best;
+    __syncthreads();
+    if (tid < M) {
+      ArgMax a = s_best[0][tid];
+      for (int w = 1; w < kWaves; ++w) a = better(a, s_best[w][tid]);
+      cand[static_cast<size_t>(tid) * gridDim.x + blockIdx.x] = a;
     }
   }
 }
@@ -785,6 +881,9 @@ extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int
   return 0;
 }
 
+constexpr size_t kHeadStageBytes = 144 * 1024;   // of the 160 KB of LDS; the rest is the kernel's own
+constexpr int kHeadRing = 8;   // chunks a wave of lm_head_stream_kernel asks for ahead (16: 2-3 us slower)
+
 // Float logits C[M, N] = A . W^T for up to 64 rows (see lm_head_kernel), with `blocks` workgroups
 // (0: two per compute unit of this machine's 256, as a plain read of such a matrix likes it).
 // cand (optional): [M][blocks] pairs of (float, int32) that receive every workgroup's largest logit
@@ -798,6 +897,21 @@ extern "C" int lyp_lm_head(const void* A, const void* W, float* C, int dtype, in
   if (blocks == 0) blocks = 512;
   blocks = std::min(blocks, (N + 63) / 64);  // no workgroup without a wave's worth of rows
   ArgMax* cd = static_cast<ArgMax*>(cand);
+  // at most 16 bfloat16 tokens whose activations fit LDS: the steady stream, one workgroup per compute unit
+  const size_t staged = static_cast<size_t>(16) * (2 * K + 16);
+  if (dtype == kBF16 && M <= 16 && staged <= kHeadStageBytes) {
+    blocks = std::min(blocks, compute_units());
+    static bool asked = false;
+    if (!asked) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(lm_head_stream_kernel<kHeadRing>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kHeadStageBytes));
+      asked = true;
+    }
+    lm_head_stream_kernel<kHeadRing><<<blocks, 256, staged, stream>>>(
+        static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, cd);
+    LYP_LAUNCH_CHECK("lm_head_stream");
+    return blocks;
+  }
 #define LYP_HEAD(T, MB) \
   lm_head_kernel<T, MB><<<blocks, 256, 0, stream>>>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, cd)
 #define LYP_HEAD_T(T)                  \
@@ -833,6 +947,7 @@ extern "C" int lyp_skinny_workgroups(int M, int N, int K, int with_slices) {
   const int rows = 16 * skinny_row_tiles(M, N, slices);
   return ((N + rows - 1) / rows) * slices;
 }
+
 
 // Slices of K that lyp_gemm_nt_parts would cut this matrix into (1: none).
 extern "C" int lyp_skinny_slices(int N, int K) { return K % 64 == 0 ? skinny_slices(N, K) : 1; }

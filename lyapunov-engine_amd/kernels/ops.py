@@ -722,7 +722,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
 
 
 LM_HEAD_MAX_ROWS = 16     # beyond that the activations are read again per 16 rows and the general products are ahead
-LM_HEAD_BLOCKS = 1024     # workgroups of the output-head kernel (measured: 256 129 us, 512 116, 1024 104, 2048 105)
+LM_HEAD_BLOCKS = 1024     # most workgroups of the output-head kernels (the library says how many it used)
 
 
 def lm_head(x: torch.Tensor, w: torch.Tensor) -> tuple:

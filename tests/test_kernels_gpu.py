@@ -864,12 +864,15 @@ def test_attention_finds_a_key_anywhere_in_8192(ops, dtype, kind, nh, nkv, hd):
 
 # ----------------------------------------------------------------- output head
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,V,K", [(1, 1003, 128), (8, 32000, 192), (16, 515, 64), (11, 2051, 256), (3, 128256, 64)])
+@pytest.mark.parametrize("M,V,K", [(1, 1003, 128), (8, 32000, 192), (16, 515, 64), (11, 2051, 256), (3, 128256, 64),
+                                   (5, 5003, 576), (2, 1003, 1344), (7, 2051, 1024), (4, 50, 512)])
 def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
-    """The head's own kernel (few long-lived waves walking the matrix): float logits against the
+    """The head's own kernels (few long-lived waves walking the matrix): float logits against the
     product in float64, and per row the pieces' maxima: the largest of them is the row's largest
     logit at the first place it stands.  Vocabularies that are no multiple of 16 or of 4; 1 to 16
-    rows; few workgroups (every wave walks many row blocks) and many."""
+    rows; few workgroups (every wave walks many row blocks) and many, also more waves than blocks
+    of rows; widths of fewer chunks of 64 than a wave of the bfloat16 kernel asks for ahead, of
+    exactly as many, of twice as many, and of a number that is no multiple of it."""
     x = rnd(M, K, dtype=dtype, seed=81)
     w = rnd(V, K, dtype=dtype, scale=0.2, seed=82)
     w[V // 3] = w[7]                                   # two equal logits in every row: the first one is to win
