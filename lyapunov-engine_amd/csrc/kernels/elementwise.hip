@@ -533,7 +533,10 @@ int lyp_rope_kv_write(void* qkv, int dtype, const int32_t* positions, const floa
   const bool aligned = T >= 16 && hd % vec == 0 && (rot / 2) % vec == 0 && width % vec == 0 && bs % vec == 0 &&
                        reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_sin) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(kpool) % 16 == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;
-  const dim3 tiles((T + 15) / 16, 8);
+  // the heads of a tile of tokens go to 8 workgroups, to more while the launch would leave compute units without one
+  int per_tile = 8;
+  while (((T + 15) / 16) * per_tile < compute_units() && per_tile < nh) per_tile *= 2;
+  const dim3 tiles((T + 15) / 16, per_tile);
   if (aligned && dtype == kF32) {
     rope_kv_tile_kernel<float><<<tiles, threads, 0, stream>>>(static_cast<float*>(qkv), positions, cos_sin, slots,
                                                               static_cast<float*>(kpool), static_cast<float*>(vpool),
