@@ -135,6 +135,170 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(const T* __restrict__ A,
     }
 }
 
+// ------------------------------------------------------- many rows, bfloat16
+// The same product for prompt steps in bfloat16 with K a multiple of 64 and 16-byte aligned rows:
+// tiles of TM tokens x TN features x 64 values of K, eight waves as 2 x 4, each with (TM / 2) x (TN / 4)
+// of the output in registers as 16x16 tiles of the 16x16x32 instruction (W's rows are the row operand, so
+// a lane ends with four neighbouring features of one token).  Two LDS buffers: while a step's tiles
+// are multiplied, the next step's are on their way from memory into the other buffer; one barrier a step.
+// Workgroups go to the chip's eight dies in turn by their number; a die keeps to its own tiles of
+// features (number % 8) and walks all tiles of tokens for each, so a tile of W is read from memory by
+// one die only and the activations, which are small, by all.
+template <int TM, int TN>
+struct WideGemm {
+  static constexpr int kTK = 64;                       // values of K a step; a row of a tile is 128 bytes, eight pieces of 16
+  static constexpr int kStage = (TM + TN) * kTK;       // elements of one buffer: the tokens' tile, then the features'
+  static constexpr int kIM = TM / 2 / 16, kJN = TN / 4 / 16;   // 16x16 tiles of a wave
+  static constexpr int kLoadsA = TM / 8 / 8, kLoadsW = TN / 8 / 8;  // load instructions per wave and step: 8 rows each
+};
+
+// One step's tiles go from memory to LDS without passing registers: a wave's load instruction brings
+// 1 KB, eight rows of 128 bytes, lane l the piece at row l / 8, place l % 8.  Rows are not padded;
+// instead place p of row r holds piece p ^ ((r / 2) % 8) of the row's eight, so that the 16 rows a
+// fragment read touches lie in 16 different groups of four banks.
+template <int TM, int TN>
+__device__ __forceinline__ void wide_ask(const bf16_t* const* ga, const bf16_t* const* gw, int k0, bf16_t* stage, int wave) {
+  using G = WideGemm<TM, TN>;
+  using LdsPtr = __attribute__((address_space(3))) void*;
+#pragma unroll
+  for (int i = 0; i < G::kLoadsA; ++i)
+    __builtin_amdgcn_global_load_lds(ga[i] + k0, (LdsPtr)(stage + (wave * G::kLoadsA + i) * 8 * G::kTK), 16, 0, 0);
+#pragma unroll
+  for (int i = 0; i < G::kLoadsW; ++i)
+    __builtin_amdgcn_global_load_lds(gw[i] + k0, (LdsPtr)(stage + TM * G::kTK + (wave * G::kLoadsW + i) * 8 * G::kTK), 16, 0, 0);
+}
+
+// this wave's loads have arrived (the count of outstanding vector memory loads is zero; the other counters are left alone)
+__device__ __forceinline__ void wide_arrived() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+template <int TM, int TN, int MODE>
+__global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                             void* __restrict__ Cv, int M, int N, int K, int lda, int ldw,
+                                                             int ldc, int m_tiles, int n_tiles) {
+  using G = WideGemm<TM, TN>;
+  constexpr int IM = G::kIM, JN = G::kJN, TK = G::kTK;
+  // two buffers as two arrays: what is in flight into one is then known not to be what is read from the other
+  __shared__ __attribute__((aligned(1024))) bf16_t stage0[G::kStage];
+  __shared__ __attribute__((aligned(1024))) bf16_t stage1[G::kStage];
+
+  // which tile: die = number % 8 owns the feature tiles die, die + 8, ...
+  const int id = blockIdx.x;
+  const int die = id % 8, local = id / 8;
+  if (local >= ((n_tiles - die + 7) / 8) * m_tiles) return;   // the launch is rounded up to whole rounds of eight
+  const int nt = die + 8 * (local / m_tiles), mt = local % m_tiles;
+  const int m0 = mt * TM, n0 = nt * TN;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / 4, wn = wave % 4;
+  const int r = lane % 16, j = lane / 16;
+
+  // this lane's piece of each of the wave's load instructions
+  const bf16_t* ga[G::kLoadsA];
+  const bf16_t* gw[G::kLoadsW];
+  {
+    const int row8 = lane / 8, place = lane % 8;
+#pragma unroll
+    for (int i = 0; i < G::kLoadsA; ++i) {
+      const int row = (wave * G::kLoadsA + i) * 8 + row8;
+      ga[i] = A + static_cast<size_t>(min(m0 + row, M - 1)) * lda + (place ^ ((row / 2) % 8)) * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < G::kLoadsW; ++i) {
+      const int row = (wave * G::kLoadsW + i) * 8 + row8;
+      gw[i] = W + static_cast<size_t>(min(n0 + row, N - 1)) * ldw + (place ^ ((row / 2) % 8)) * 8;
+    }
+  }
+
+  f32x4 acc[IM][JN];
+#pragma unroll
+  for (int i = 0; i < IM; ++i)
+#pragma unroll
+    for (int jn = 0; jn < JN; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // fragment of values 32 kk + 8 j .. of row r of a 16-row tile: piece 4 kk + j, at place (4 kk + j) ^ (r / 2)
+  const int a_frag = (wm * (TM / 2) + r) * TK + (j ^ (r / 2)) * 8;              // + i * 16 * TK, ^ 32 for kk = 1
+  const int w_frag = TM * TK + (wn * (TN / 4) + r) * TK + (j ^ (r / 2)) * 8;    // + jn * 16 * TK
+
+  auto ask = [&](int k0, bf16_t* stage) { wide_ask<TM, TN>(ga, gw, k0, stage, wave); };
+  auto step = [&](const bf16_t* stage) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      // (the second half of the step's 64 values: four pieces on, which in a swizzled row is the place with bit 2 flipped)
+      const bf16_t* wrow = stage + (kk == 0 ? w_frag : w_frag ^ 32);
+      const bf16_t* arow = stage + (kk == 0 ? a_frag : a_frag ^ 32);
+      bf16x8 wf[JN];
+#pragma unroll
+      for (int jn = 0; jn < JN; ++jn) wf[jn] = *reinterpret_cast<const bf16x8*>(wrow + jn * 16 * TK);
+#pragma unroll
+      for (int i = 0; i < IM; ++i) {
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(arow + i * 16 * TK);
+#pragma unroll
+        for (int jn = 0; jn < JN; ++jn) acc[i][jn] = Mma16Wide<bf16_t>::mma(wf[jn], xf, acc[i][jn]);
+      }
+    }
+  };
+  // (Letting the workgroups that share a tile of W start at different places of K, so that one of them asks
+  // memory for a slice and the others find it in the die's cache, was measured: 5 % slower.  They walk K in
+  // step, and the cache merges their requests.)
+  const int steps = K / TK;
+  ask(0, stage0);
+  wide_arrived();
+  __syncthreads();
+  int s = 0;
+#pragma unroll 1
+  for (; s + 2 <= steps; s += 2) {
+    ask((s + 1) * TK, stage1);
+    __builtin_amdgcn_sched_barrier(0);   // the loads go out before the products, not where the scheduler finds room for them
+    step(stage0);
+    wide_arrived();
+    __syncthreads();
+    if (s + 2 < steps) ask((s + 2) * TK, stage0);
+    __builtin_amdgcn_sched_barrier(0);
+    step(stage1);
+    wide_arrived();
+    __syncthreads();
+  }
+  if (s < steps) step(stage0);   // an odd number of steps: the last one was asked for in the round before (or at the start)
+
+  // acc[i][jn][v]: token m0 + wm TM/2 + 16 i + r, feature n0 + wn TN/4 + 16 jn + 4 j + v
+#pragma unroll
+  for (int i = 0; i < IM; ++i) {
+    const int m = m0 + wm * (TM / 2) + 16 * i + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int jn = 0; jn < JN; ++jn) {
+      const int n = n0 + wn * (TN / 4) + 16 * jn + 4 * j;
+      if (n >= N) continue;
+      const size_t idx = static_cast<size_t>(m) * ldc + n;
+      const bool whole = n + 3 < N && ldc % 4 == 0;
+      if constexpr (MODE == kStoreAct) {
+        bf16_t* dst = static_cast<bf16_t*>(Cv) + idx;
+        if (whole) {
+          bf16x4 o;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o[v] = from_f32<bf16_t>(acc[i][jn][v]);
+          *reinterpret_cast<bf16x4*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (n + v < N) dst[v] = from_f32<bf16_t>(acc[i][jn][v]);
+        }
+      } else {
+        float* dst = static_cast<float*>(Cv) + idx;
+        if (whole) {
+          f32x4 o = acc[i][jn];
+          if constexpr (MODE == kAccumF32) o += *reinterpret_cast<const f32x4*>(dst);
+          *reinterpret_cast<f32x4*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (n + v < N) dst[v] = MODE == kAccumF32 ? dst[v] + acc[i][jn][v] : acc[i][jn][v];
+        }
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------- few rows
 // M <= 64 (decode steps): the weight matrix is read once from memory and the
 // time is what that read takes, so the shape is chosen for memory parallelism.
@@ -820,9 +984,29 @@ static void launch_skinny_rows(const T* A, const T* W, void* C, int M, int N, in
     launch_skinny<T, EPI>(A, W, C, M, N, K, lda, ldw, ldc, slices, stream, tail);
 }
 
+static int g_wide_gemm = 1;   // many bfloat16 rows: 1 the wide kernel, tile by rule; for tests and measurements 0 the general kernel, 2 / 3 tiles of 128 / 256 features
+template <int TM, int TN, int MODE>
+static void launch_wide(const bf16_t* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                        hipStream_t stream) {
+  const int m_tiles = (M + TM - 1) / TM, n_tiles = (N + TN - 1) / TN;
+  const int grid = 8 * ((n_tiles + 7) / 8) * m_tiles;   // every die's share rounded up to that of the first
+  gemm_bf16_wide_kernel<TM, TN, MODE><<<grid, 512, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, m_tiles, n_tiles);
+}
+
 template <typename T, int MODE>
 static void launch_gemm(const T* A, const T* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                         int vec_ok, hipStream_t stream) {
+  if constexpr (std::is_same_v<T, bf16_t>) {
+    if (M > 128 && vec_ok && K % 64 == 0 && g_wide_gemm) {
+      // tiles of 256 features while there is one for every compute unit, of 128 otherwise
+      const long long tiles = static_cast<long long>((M + 255) / 256) * ((N + 255) / 256);
+      if (g_wide_gemm == 2 || (g_wide_gemm == 1 && tiles < compute_units()))
+        launch_wide<256, 128, MODE>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+      else
+        launch_wide<256, 256, MODE>(A, W, C, M, N, K, lda, ldw, ldc, stream);
+      return;
+    }
+  }
   if (M <= 32) {
     dim3 grid((N + 127) / 128, (M + 31) / 32);
     gemm_nt_kernel<T, 32, 128, 1, 4, MODE><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc, vec_ok);
@@ -838,6 +1022,12 @@ static void launch_gemm(const T* A, const T* W, void* C, int M, int N, int K, in
 }  // namespace lyp
 
 using namespace lyp;
+
+extern "C" int lyp_gemm_wide(int which) {
+  LYP_REQUIRE(which >= 0 && which <= 3, "wide product: 0 to 3, not %d", which);
+  g_wide_gemm = which;
+  return 0;
+}
 
 extern "C" int lyp_gemm_nt(const void* A, const void* W, void* C, int dtype, int mode, int M, int N, int K,
                            int lda, int ldw, int ldc, hipStream_t stream) {

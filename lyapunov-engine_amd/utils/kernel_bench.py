@@ -309,12 +309,19 @@ def main(argv=None) -> None:
     ap.add_argument("--own", action="store_true", help="products of 17 to 64 rows in this package's kernel whatever "
                     "the size of the matrix (the vendor's library otherwise takes the larger ones)")
     ap.add_argument("--row-tiles", type=int, default=0, help="row tiles per workgroup of that kernel (0: its rule)")
+    ap.add_argument("--wide", type=int, default=-1,
+                    help="many bfloat16 rows with LYAPUNOV_AMD_GEMM=own: 0 the general tiled kernel, 1 the wide kernel (tile by rule), "
+                    "2 / 3 its tiles of 128 / 256 features")
     a = ap.parse_args(argv)
     ops.require_gpu()
     if a.own:
         ops.LIBRARY_ROUNDS = 1 << 20
     if a.row_tiles:
         ops.skinny_row_tiles_override(a.row_tiles)
+    if a.wide >= 0:
+        lib = ops.core()
+        if lib.lyp_gemm_wide(a.wide) != 0:
+            raise SystemExit(lib.lyp_last_error().decode())
     torch.manual_seed(0)
     {"attn_prefill": attn_prefill, "attn_decode": attn_decode, "linear": linear, "qkv": qkv, "gate_up": gate_up, "residual": residual,
      "sample": sample, "stream": stream, "rmsnorm": rmsnorm, "head": head, "floor": floor}[a.kernel](a)

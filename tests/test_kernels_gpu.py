@@ -255,6 +255,34 @@ def test_float_logits_of_many_rows_are_not_rounded_to_bfloat16(ops):
     assert ((y.cpu().double() - want).abs() <= 1e-5 * bound + 1e-30).all()
 
 
+@pytest.mark.parametrize("M,N,K", [(129, 96, 64), (300, 520, 192), (257, 255, 128), (1024, 384, 320), (513, 2051, 64),
+                                   (2048, 512, 1024)])
+def test_bfloat16_product_of_many_rows_in_this_package(ops, M, N, K, monkeypatch):
+    """The tiled kernel for prompt steps without the vendor's library (tiles of 256 tokens, loads that go
+    straight to LDS into swizzled rows): all three outputs, both tile widths, against float64; rows and
+    features that are no multiple of the tile, of 16 or of 4, one step of K and an odd number of them."""
+    monkeypatch.setattr(ops, "LIBRARY_GEMM", False)
+    a, w = rnd(M, K, dtype=torch.bfloat16, seed=71), rnd(N, K, dtype=torch.bfloat16, scale=0.05, seed=72)
+    want = a.double() @ w.double().T
+    bound = a.double().abs() @ w.double().abs().T
+    lib = ops.core()
+    try:
+        for which in (1, 2, 3, 0):
+            assert lib.lyp_gemm_wide(which) == 0
+            for out_dtype, rel in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
+                out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+                ops.gemm_nt(a.to(DEV), w.to(DEV), out)
+                err = (out.cpu().double() - want).abs()
+                assert (err <= rel * bound + 1e-30).all(), (which, out_dtype, float(err.max()))
+            acc = rnd(M, N, seed=73)
+            out = acc.to(DEV)
+            ops.gemm_nt(a.to(DEV), w.to(DEV), out, accumulate=True)
+            err = (out.cpu().double() - acc.double() - want).abs()
+            assert (err <= 1e-5 * bound + 2e-6 * acc.abs().double() + 1e-30).all(), (which, float(err.max()))
+    finally:
+        lib.lyp_gemm_wide(1)
+
+
 def test_library_products_keep_one_plan_per_shape(ops):
     """The vendor's library called directly: operands that are column ranges of
     wider tensors (rows further apart than they are long), both output types,
@@ -865,14 +893,15 @@ def test_attention_finds_a_key_anywhere_in_8192(ops, dtype, kind, nh, nkv, hd):
 # ----------------------------------------------------------------- output head
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,V,K", [(1, 1003, 128), (8, 32000, 192), (16, 515, 64), (11, 2051, 256), (3, 128256, 64),
-                                   (5, 5003, 576), (2, 1003, 1344), (7, 2051, 1024), (4, 50, 512)])
+                                   (5, 5003, 576), (2, 1003, 1344), (7, 2051, 1024), (4, 50, 512), (3, 1003, 4672)])
 def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     """The head's own kernels (few long-lived waves walking the matrix): float logits against the
     product in float64, and per row the pieces' maxima: the largest of them is the row's largest
     logit at the first place it stands.  Vocabularies that are no multiple of 16 or of 4; 1 to 16
     rows; few workgroups (every wave walks many row blocks) and many, also more waves than blocks
     of rows; widths of fewer chunks of 64 than a wave of the bfloat16 kernel asks for ahead, of
-    exactly as many, of twice as many, and of a number that is no multiple of it."""
+    exactly as many, of twice as many, and of a number that is no multiple of it; a width whose
+    activations do not fit LDS (bfloat16 then takes the kernel that reads them from the cache)."""
     x = rnd(M, K, dtype=dtype, seed=81)
     w = rnd(V, K, dtype=dtype, scale=0.2, seed=82)
     w[V // 3] = w[7]                                   # two equal logits in every row: the first one is to win
