@@ -909,7 +909,11 @@ def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     for blocks in (8, 512):
         monkeypatch.setattr(ops, "LM_HEAD_BLOCKS", blocks)
         out, maxima = ops.lm_head(x.to(DEV), w.to(DEV))
-        torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 1e-2))
+        if K <= 2048:
+            torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 1e-2))
+        else:   # a long sum: held to the size of what is added up, as the products' own test does
+            bound = x.double().abs() @ w.double().abs().T
+            assert ((out.cpu().double() - want).abs() <= (2e-6 if dtype == torch.float32 else 1e-5) * bound).all()
         cand = maxima.cpu()
         assert cand.shape[0] == M and cand.shape[2] == 2 and cand.shape[1] <= blocks
         values, places = cand[..., 0].contiguous().view(torch.float32), cand[..., 1]
