@@ -177,7 +177,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(const bf16_t* __res
                                                              int ldc, int m_tiles, int n_tiles) {
   using G = WideGemm<TM, TN>;
   constexpr int IM = G::kIM, JN = G::kJN, TK = G::kTK;
-  // two buffers as two arrays: what is in flight into one is then known not to be what is read from the other
+  // two buffers
   __shared__ __attribute__((aligned(1024))) bf16_t stage0[G::kStage];
   __shared__ __attribute__((aligned(1024))) bf16_t stage1[G::kStage];
 
@@ -220,21 +220,25 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(const bf16_t* __res
   const int w_frag = TM * TK + (wn * (TN / 4) + r) * TK + (j ^ (r / 2)) * 8;    // + jn * 16 * TK
 
   auto ask = [&](int k0, bf16_t* stage) { wide_ask<TM, TN>(ga, gw, k0, stage, wave); };
+  // A half step: every fragment first, then the products (the scheduler is told so: left alone it
+  // asks for two fragments at a time and waits for them before every eight products).
   auto step = [&](const bf16_t* stage) {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       // (the second half of the step's 64 values: four pieces on, which in a swizzled row is the place with bit 2 flipped)
       const bf16_t* wrow = stage + (kk == 0 ? w_frag : w_frag ^ 32);
       const bf16_t* arow = stage + (kk == 0 ? a_frag : a_frag ^ 32);
-      bf16x8 wf[JN];
+      bf16x8 wf[JN], xf[IM];
 #pragma unroll
       for (int jn = 0; jn < JN; ++jn) wf[jn] = *reinterpret_cast<const bf16x8*>(wrow + jn * 16 * TK);
 #pragma unroll
-      for (int i = 0; i < IM; ++i) {
-        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(arow + i * 16 * TK);
+      for (int i = 0; i < IM; ++i) xf[i] = *reinterpret_cast<const bf16x8*>(arow + i * 16 * TK);
 #pragma unroll
-        for (int jn = 0; jn < JN; ++jn) acc[i][jn] = Mma16Wide<bf16_t>::mma(wf[jn], xf, acc[i][jn]);
-      }
+      for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int jn = 0; jn < JN; ++jn) acc[i][jn] = Mma16Wide<bf16_t>::mma(wf[jn], xf[i], acc[i][jn]);
+      __builtin_amdgcn_sched_group_barrier(0x100, IM + JN, 0);   // LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x008, IM * JN, 0);   // matrix instructions
     }
   };
   // (Letting the workgroups that share a tile of W start at different places of K, so that one of them asks
@@ -244,21 +248,19 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(const bf16_t* __res
   ask(0, stage0);
   wide_arrived();
   __syncthreads();
-  int s = 0;
+  bf16_t* cur = stage0;
+  bf16_t* nxt = stage1;
 #pragma unroll 1
-  for (; s + 2 <= steps; s += 2) {
-    ask((s + 1) * TK, stage1);
+  for (int s = 0; s < steps; ++s) {
+    if (s + 1 < steps) ask((s + 1) * TK, nxt);
     __builtin_amdgcn_sched_barrier(0);   // the loads go out before the products, not where the scheduler finds room for them
-    step(stage0);
+    step(cur);
     wide_arrived();
     __syncthreads();
-    if (s + 2 < steps) ask((s + 2) * TK, stage0);
-    __builtin_amdgcn_sched_barrier(0);
-    step(stage1);
-    wide_arrived();
-    __syncthreads();
+    bf16_t* t = cur;
+    cur = nxt;
+    nxt = t;
   }
-  if (s < steps) step(stage0);   // an odd number of steps: the last one was asked for in the round before (or at the start)
 
   // acc[i][jn][v]: token m0 + wm TM/2 + 16 i + r, feature n0 + wn TN/4 + 16 jn + 4 j + v
 #pragma unroll
