@@ -384,6 +384,34 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const uint4* __restric
   if (threadIdx.x % kWave == 0) sink[blockIdx.x * (256 / kWave) + threadIdx.x / kWave] = acc;
 }
 
+// The same bytes read the way the weight-streaming products read a matrix [rows][row_bytes]: a wave
+// takes 16 rows at a time, an instruction 64 bytes of each of them, 8 steps of 128 bytes per row in
+// flight; then the next 16 rows that are its turn.  row_bytes a multiple of 2048.
+// FULL: 8 rows a wave and 128 bytes (a whole cache line) of each per load instead.
+template <bool FULL>
+__global__ __launch_bounds__(256) void stream_rows_kernel(const uint4* __restrict__ src, int rows, int row_bytes,
+                                                         uint32_t* __restrict__ sink) {
+  constexpr int R = FULL ? 8 : 16;       // rows a wave walks at a time
+  constexpr int G = kWave / R;           // 16-byte pieces of a row per load instruction
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int r = lane % R, j = lane / R;
+  const int tiles = rows / R, row_words = row_bytes / 16;
+  uint32_t acc = 0;
+  for (int tile = blockIdx.x * 4 + wave; tile < tiles; tile += gridDim.x * 4) {
+    const uint4* p = src + static_cast<size_t>(tile * R + r) * row_words + j;
+    for (int c = 0; c < row_words; c += 16 * G) {   // 16 loads in flight: 16 G pieces of every row
+      uint4 v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = p[c + u * G];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) acc ^= __shfl_xor(acc, off, kWave);
+  if (lane == 0) sink[blockIdx.x * 4 + wave] = acc;
+}
+
 // A step's table of small integers from pinned host memory (which the device reads through the
 // same address) to its place on the device, in one launch; `n_patch` words from `patch_at` on come
 // from `patch` on the device instead (token ids that only the device knows yet).
@@ -417,6 +445,20 @@ int lyp_stream_read(const void* src, long long bytes, int blocks, uint32_t* sink
               reinterpret_cast<uintptr_t>(src) % 16 == 0, "stream_read: %lld bytes in %d workgroups", bytes, blocks);
   stream_read_kernel<<<blocks, 256, 0, stream>>>(static_cast<const uint4*>(src), static_cast<size_t>(bytes / 16), sink);
   LYP_LAUNCH_CHECK("stream_read");
+  return 0;
+}
+
+// The same through stream_rows_kernel, as a matrix of rows of row_bytes (a multiple of 2048; bytes a multiple of 16 rows).
+int lyp_stream_rows(const void* src, long long bytes, int row_bytes, int whole_lines, int blocks, uint32_t* sink,
+                    hipStream_t stream) {
+  LYP_REQUIRE(src && sink && bytes > 0 && row_bytes > 0 && row_bytes % 2048 == 0 && bytes % (16LL * row_bytes) == 0 &&
+              blocks > 0 && blocks <= 65535 && bytes / row_bytes < (1LL << 31),
+              "stream_rows: %lld bytes in rows of %d, %d workgroups", bytes, row_bytes, blocks);
+  if (whole_lines)
+    stream_rows_kernel<true><<<blocks, 256, 0, stream>>>(static_cast<const uint4*>(src), static_cast<int>(bytes / row_bytes), row_bytes, sink);
+  else
+    stream_rows_kernel<false><<<blocks, 256, 0, stream>>>(static_cast<const uint4*>(src), static_cast<int>(bytes / row_bytes), row_bytes, sink);
+  LYP_LAUNCH_CHECK("stream_rows");
   return 0;
 }
 

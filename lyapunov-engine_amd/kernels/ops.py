@@ -85,6 +85,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_skinny_workgroups.argtypes = [c_int, c_int, c_int, c_int]
         lib.lyp_skinny_slices.argtypes = [c_int, c_int]
         lib.lyp_stream_read.argtypes = [c_void_p, c_longlong, c_int, c_void_p, c_void_p]
+        lib.lyp_stream_rows.argtypes = [c_void_p, c_longlong, c_int, c_int, c_int, c_void_p, c_void_p]
         _core = lib
     return _core
 
@@ -311,6 +312,18 @@ def stream_read(src: torch.Tensor, sink: torch.Tensor, blocks: int) -> None:
         raise KernelError("stream_read: the sink must hold four int32 values per workgroup")
     lib = core()
     _check(lib.lyp_stream_read(_p(src), nbytes, blocks, _p(sink), _stream()), lib)
+
+
+def stream_rows(src: torch.Tensor, sink: torch.Tensor, blocks: int, row_bytes: int, whole_lines: bool = False) -> None:
+    """Read all of ``src`` once as a matrix of rows of ``row_bytes``, the way the
+    weight-streaming products do (16 rows a wave, 64 bytes of each per load; with
+    ``whole_lines`` 8 rows a wave and 128 bytes of each)."""
+    _dev(src, sink)
+    nbytes = src.numel() * src.element_size()
+    if sink.dtype != torch.int32 or sink.numel() < blocks * 4:
+        raise KernelError("stream_rows: the sink must hold four int32 values per workgroup")
+    lib = core()
+    _check(lib.lyp_stream_rows(_p(src), nbytes, row_bytes, int(whole_lines), blocks, _p(sink), _stream()), lib)
 
 
 def norm_threads_override(threads: int) -> None:

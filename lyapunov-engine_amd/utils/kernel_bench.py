@@ -241,6 +241,21 @@ def stream(a) -> None:
             c = sorted(cold)[len(cold) // 2]
             print(f"stream {mb} MiB in {blocks} workgroups: cold {c * 1e6:.1f} us {src.numel() / c / 1e12:.2f} TB/s, "
                   f"again and again {warm * 1e6:.1f} us {src.numel() / warm / 1e12:.2f} TB/s")
+            if a.row_bytes and (mb << 20) % (16 * a.row_bytes) == 0:
+                for whole in (False, True):
+                    rows = []
+                    for _ in range(5):
+                        ops.stream_read(flush, torch.empty(4096 * 4, dtype=torch.int32, device=dev), 4096)
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        ops.stream_rows(src, sink, blocks, a.row_bytes, whole)
+                        e1.record()
+                        torch.cuda.synchronize()
+                        rows.append(e0.elapsed_time(e1) * 1e-3)
+                    c = sorted(rows)[len(rows) // 2]
+                    how = "8 rows a wave and 128 bytes" if whole else "16 rows a wave and 64 bytes"
+                    print(f"   as rows of {a.row_bytes} bytes, {how} of each per load: cold {c * 1e6:.1f} us "
+                          f"{src.numel() / c / 1e12:.2f} TB/s")
 
 
 def floor(a) -> None:
@@ -308,6 +323,7 @@ def main(argv=None) -> None:
     ap.add_argument("--may-split", action="store_true", help="linear: allow partial sums over slices of K")
     ap.add_argument("--own", action="store_true", help="products of 17 to 64 rows in this package's kernel whatever "
                     "the size of the matrix (the vendor's library otherwise takes the larger ones)")
+    ap.add_argument("--row-bytes", type=int, default=0, help="stream: also read the buffer as a matrix of rows of this many bytes")
     ap.add_argument("--row-tiles", type=int, default=0, help="row tiles per workgroup of that kernel (0: its rule)")
     ap.add_argument("--wide", type=int, default=-1,
                     help="many bfloat16 rows with LYAPUNOV_AMD_GEMM=own: 0 the general tiled kernel, 1 the wide kernel (tile by rule), "
