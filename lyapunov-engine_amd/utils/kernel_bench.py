@@ -7,6 +7,8 @@
     python -m lyapunov_engine_amd.utils.kernel_bench sample --rows 8 --vocab 128256 --top-k 50 --top-p 0.9
     python -m lyapunov_engine_amd.utils.kernel_bench head --rows 8
     python -m lyapunov_engine_amd.utils.kernel_bench stream --megabytes 64
+    python -m lyapunov_engine_amd.utils.kernel_bench stream --megabytes 512 --blocks 256 --row-bytes 4096
+    LYAPUNOV_AMD_GEMM=own python -m lyapunov_engine_amd.utils.kernel_bench linear --rows 2048 --wide 1
     python -m lyapunov_engine_amd.utils.kernel_bench rmsnorm --rows 2048 --in-features 4100 --threads 256
     python -m lyapunov_engine_amd.utils.kernel_bench floor
 
