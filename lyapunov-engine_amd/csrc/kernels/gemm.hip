@@ -803,14 +803,15 @@ __global__ __launch_bounds__(256) void lm_head_kernel(const T* __restrict__ A, c
 // before it; from LDS it does not.  One workgroup per compute unit is enough to keep the memory busy
 // (8 tokens on 128256 x 2048: 256 workgroups 106.5 us, 512 107.0, 1024 111.5, against 115.7 of
 // lm_head_kernel; 16 tokens 114 against 131, one token 100 against 105).
-template <int RING>
+// MB blocks of 16 tokens (what LDS holds of them: 32 tokens of 2,048 values): a fragment of weights is then used MB times.
+template <int RING, int MB>
 __global__ __launch_bounds__(256) void lm_head_stream_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
                                                              float* __restrict__ C, int M, int N, int K, int lda, int ldw,
                                                              int ldc, ArgMax* __restrict__ cand) {
   using MM = Mma16Wide<bf16_t>;
   constexpr int kWaves = 4;
-  extern __shared__ __attribute__((aligned(16))) unsigned char x_lds[];   // [16][2 K + 16] bytes
-  __shared__ ArgMax s_best[kWaves][16];
+  extern __shared__ __attribute__((aligned(16))) unsigned char x_lds[];   // [16 MB][2 K + 16] bytes
+  __shared__ ArgMax s_best[kWaves][MB][16];
   const int row_bytes = 2 * K + 16;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -826,26 +827,32 @@ __global__ __launch_bounds__(256) void lm_head_stream_kernel(const bf16_t* __res
   for (int u = 0; u < RING; ++u)
 #pragma unroll
     for (int f = 0; f < 2; ++f) wf[u][f] = *reinterpret_cast<const bf16x8*>(wp + min(u, chunks - 1) * 64 + f * 32);
-  for (int p = tid; p < 16 * (K / 8); p += 256) {
+  for (int p = tid; p < 16 * MB * (K / 8); p += 256) {
     const int row = p / (K / 8), c16 = p % (K / 8);
     *reinterpret_cast<bf16x8*>(x_lds + row * row_bytes + c16 * 16) =
         *reinterpret_cast<const bf16x8*>(A + static_cast<size_t>(min(row, M - 1)) * lda + c16 * 8);
   }
   __syncthreads();
   const unsigned char* xl = x_lds + r * row_bytes + j * 16;
-  ArgMax best{LYP_NEG_INF, 0x7fffffff};
+  ArgMax best[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) best[b] = ArgMax{LYP_NEG_INF, 0x7fffffff};
   for (; tile < tiles; tile += stride) {
     const bf16_t* wn = W + static_cast<size_t>(min(min(tile + stride, tiles - 1) * 16 + r, N - 1)) * ldw + j * 8;
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < chunks; c += RING) {
 #pragma unroll
       for (int u = 0; u < RING; ++u) {
         if (c + u < chunks) {
 #pragma unroll
-          for (int f = 0; f < 2; ++f) {
-            const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xl + (c + u) * 128 + f * 64);
-            acc = MM::mma(wf[u][f], xf, acc);
-          }
+          for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+              const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xl + b * 16 * row_bytes + (c + u) * 128 + f * 64);
+              acc[b] = MM::mma(wf[u][f], xf, acc[b]);
+            }
         }
         // slot u next holds chunk c + u + RING of this tile, or the next tile's chunk past this one's end
         const int nc = c + u + RING;
@@ -855,35 +862,41 @@ __global__ __launch_bounds__(256) void lm_head_stream_kernel(const bf16_t* __res
         for (int f = 0; f < 2; ++f) wf[u][f] = *reinterpret_cast<const bf16x8*>(src + f * 32);
       }
     }
-    // acc[i]: row 16 tile + 4 j + i of W (a logit's index), token r
+    // acc[b][i]: row 16 tile + 4 j + i of W (a logit's index), token 16 b + r
     const int n = tile * 16 + 4 * j;
-    ArgMax mine{LYP_NEG_INF, 0x7fffffff};
-    if (r < M) {
-      float* crow = C + static_cast<size_t>(r) * ldc + n;
-      if (n + 3 < N && ldc % 4 == 0) {
-        *reinterpret_cast<f32x4*>(crow) = acc;
-      } else {
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const int m = 16 * b + r;
+      ArgMax mine{LYP_NEG_INF, 0x7fffffff};
+      if (m < M) {
+        float* crow = C + static_cast<size_t>(m) * ldc + n;
+        if (n + 3 < N && ldc % 4 == 0) {
+          *reinterpret_cast<f32x4*>(crow) = acc[b];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) crow[i] = acc[b][i];
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n + i < N) crow[i] = acc[i];
+          if (n + i < N) mine = better(mine, ArgMax{acc[b][i], n + i});
       }
+      if (cand) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < N) mine = better(mine, ArgMax{acc[i], n + i});
-    }
-    if (cand) {
-#pragma unroll
-      for (int off = 16; off < kWave; off *= 2) mine = better(mine, ArgMax{__shfl_xor(mine.v, off, kWave), __shfl_xor(mine.i, off, kWave)});
-      best = better(best, mine);
+        for (int off = 16; off < kWave; off *= 2) mine = better(mine, ArgMax{__shfl_xor(mine.v, off, kWave), __shfl_xor(mine.i, off, kWave)});
+        best[b] = better(best[b], mine);
+      }
     }
     wp = wn;
   }
   if (cand) {
-    if (j == 0) s_best[wave][r] = best;
+    if (j == 0)
+#pragma unroll
+      for (int b = 0; b < MB; ++b) s_best[wave][b][r] = best[b];
     __syncthreads();
     if (tid < M) {
-      ArgMax a = s_best[0][tid];
-      for (int w = 1; w < kWaves; ++w) a = better(a, s_best[w][tid]);
+      ArgMax a = s_best[0][tid / 16][tid % 16];
+      for (int w = 1; w < kWaves; ++w) a = better(a, s_best[w][tid / 16][tid % 16]);
       cand[static_cast<size_t>(tid) * gridDim.x + blockIdx.x] = a;
     }
   }
@@ -1089,21 +1102,25 @@ extern "C" int lyp_lm_head(const void* A, const void* W, float* C, int dtype, in
   if (blocks == 0) blocks = 512;
   blocks = std::min(blocks, (N + 63) / 64);  // no workgroup without a wave's worth of rows
   ArgMax* cd = static_cast<ArgMax*>(cand);
-  // at most 16 bfloat16 tokens whose activations fit LDS: the steady stream, one workgroup per compute unit
-  const size_t staged = static_cast<size_t>(16) * (2 * K + 16);
-  if (dtype == kBF16 && M <= 16 && staged <= kHeadStageBytes) {
+  // bfloat16 tokens whose activations fit LDS (16 of up to 4,600 values, 32 of up to 2,296): the steady stream, one
+  // workgroup per compute unit
+  const int token_blocks = (M + 15) / 16;
+  const size_t staged = static_cast<size_t>(16) * token_blocks * (2 * K + 16);
+  if (dtype == kBF16 && token_blocks <= 2 && staged <= kHeadStageBytes) {
     blocks = std::min(blocks, compute_units());
-    static bool asked = false;
-    if (!asked) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(lm_head_stream_kernel<kHeadRing>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kHeadStageBytes));
-      asked = true;
+    auto kernel = token_blocks == 1 ? lm_head_stream_kernel<kHeadRing, 1> : lm_head_stream_kernel<kHeadRing, 2>;
+    static bool asked[2] = {false, false};
+    if (!asked[token_blocks - 1]) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(kHeadStageBytes));
+      asked[token_blocks - 1] = true;
     }
-    lm_head_stream_kernel<kHeadRing><<<blocks, 256, staged, stream>>>(
-        static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda, ldw, ldc, cd);
+    kernel<<<blocks, 256, staged, stream>>>(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(W), C, M, N, K, lda,
+                                            ldw, ldc, cd);
     LYP_LAUNCH_CHECK("lm_head_stream");
     return blocks;
   }
+  if (M > 16) return 0;   // beyond that the general products are ahead of lm_head_kernel
 #define LYP_HEAD(T, MB) \
   lm_head_kernel<T, MB><<<blocks, 256, 0, stream>>>(static_cast<const T*>(A), static_cast<const T*>(W), C, M, N, K, lda, ldw, ldc, cd)
 #define LYP_HEAD_T(T)                  \

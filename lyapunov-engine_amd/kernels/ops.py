@@ -734,7 +734,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype | None = Non
     return cast(gemm_nt(x, w, out), out_dtype)
 
 
-LM_HEAD_MAX_ROWS = 16     # beyond that the activations are read again per 16 rows and the general products are ahead
+LM_HEAD_MAX_ROWS = 32     # what the output-head kernels may take (the library call says no where the general products are ahead)
 LM_HEAD_BLOCKS = 1024     # most workgroups of the output-head kernels (the library says how many it used)
 
 

@@ -893,7 +893,8 @@ def test_attention_finds_a_key_anywhere_in_8192(ops, dtype, kind, nh, nkv, hd):
 # ----------------------------------------------------------------- output head
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,V,K", [(1, 1003, 128), (8, 32000, 192), (16, 515, 64), (11, 2051, 256), (3, 128256, 64),
-                                   (5, 5003, 576), (2, 1003, 1344), (7, 2051, 1024), (4, 50, 512), (3, 1003, 4672)])
+                                   (5, 5003, 576), (2, 1003, 1344), (7, 2051, 1024), (4, 50, 512), (3, 1003, 4672),
+                                   (17, 1003, 128), (24, 515, 1344), (32, 2051, 2048), (29, 5003, 64), (20, 300, 2304)])
 def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     """The head's own kernels (few long-lived waves walking the matrix): float logits against the
     product in float64, and per row the pieces' maxima: the largest of them is the row's largest
@@ -901,7 +902,9 @@ def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     rows; few workgroups (every wave walks many row blocks) and many, also more waves than blocks
     of rows; widths of fewer chunks of 64 than a wave of the bfloat16 kernel asks for ahead, of
     exactly as many, of twice as many, and of a number that is no multiple of it; a width whose
-    activations do not fit LDS (bfloat16 then takes the kernel that reads them from the cache)."""
+    activations do not fit LDS (bfloat16 then takes the kernel that reads them from the cache).
+    17 to 32 rows: bfloat16 takes the same kernel with two blocks of 16 tokens while their activations
+    fit LDS; 32-bit, and a width beyond that, go to the general products and bring no row maxima."""
     x = rnd(M, K, dtype=dtype, seed=81)
     w = rnd(V, K, dtype=dtype, scale=0.2, seed=82)
     w[V // 3] = w[7]                                   # two equal logits in every row: the first one is to win
@@ -909,11 +912,15 @@ def test_output_head_logits_and_row_maxima(ops, dtype, M, V, K, monkeypatch):
     for blocks in (8, 512):
         monkeypatch.setattr(ops, "LM_HEAD_BLOCKS", blocks)
         out, maxima = ops.lm_head(x.to(DEV), w.to(DEV))
+        if M > 16:
+            assert (maxima is not None) == (dtype == torch.bfloat16 and K <= 2296), (M, K, dtype)
         if K <= 2048:
             torch.testing.assert_close(out.cpu().double(), want, **tol(dtype, 2e-5, 1e-2))
         else:   # a long sum: held to the size of what is added up, as the products' own test does
             bound = x.double().abs() @ w.double().abs().T
             assert ((out.cpu().double() - want).abs() <= (2e-6 if dtype == torch.float32 else 1e-5) * bound).all()
+        if maxima is None:
+            continue
         cand = maxima.cpu()
         assert cand.shape[0] == M and cand.shape[2] == 2 and cand.shape[1] <= blocks
         values, places = cand[..., 0].contiguous().view(torch.float32), cand[..., 1]
